@@ -1,0 +1,120 @@
+/*
+ * C ABI of the MI355X (gfx950) implementation of mllm-advanced's W4A32 quantized
+ * Linear: f32 activations, quantized per row to asymmetric int8 at run time, times
+ * 4-bit symmetric block-32 weights with bf16 block scales, f32 output
+ * (the reference's KaiLinear_f32_qai8dxp_qsi4c32p_mxk_nxk).
+ *
+ * Every pointer named d_* is DEVICE memory on the current HIP device; `stream` is a
+ * hipStream_t passed as void* (NULL = the null stream). Calls only enqueue work on
+ * `stream` and return; none of them synchronises, allocates or frees. Return value:
+ * W4A32_OK or a negative W4A32_E* code - never exit().
+ *
+ * Each entry point names the reference interface it stands in for (paths relative to
+ * the reference tree).
+ */
+#ifndef W4A32_HIP_H
+#define W4A32_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  W4A32_OK = 0,
+  W4A32_EINVAL = -1,   /* null pointer, non-positive dimension, misaligned pointer */
+  W4A32_ESHAPE = -2,   /* K not a multiple of 32, or M outside the kernel's range */
+  W4A32_ELAUNCH = -3,  /* the HIP runtime refused the launch (see hipGetLastError) */
+  W4A32_ENOTSUP = -4   /* request needs a path this build does not provide */
+};
+
+#define W4A32_BLOCK_LEN 32          /* k per weight scale (kai_linear.cpp:328 passes 32) */
+#define W4A32_GEMV_MAX_M 8          /* largest M served by the decode (GEMV) kernels */
+
+/* bf16 rounding of the block scale: 0 = truncate (the reference's shipped build: no +bf16
+ * arch flag, tests/Arm/KaiLinearTest.hpp:138-139), 1 = round to nearest even (bfcvt). */
+#define W4A32_BF16_TRUNC 0
+#define W4A32_BF16_RNE 1
+
+const char* w4a32_error_string(int code);
+
+/* Library/version probe; also the symbol a loader checks first. */
+int w4a32_abi_version(void);
+
+/* ---- sizes ------------------------------------------------------------------------ */
+
+/* Bytes of the device weight blob for an [N][K] Linear.
+ * Replaces KaiLinear_f32_qai8dxp_qsi4c32p_mxk_nxk::quant_pack_rhs_size
+ * (mllm/Backends/Arm/Kernels/kai_linear.cpp:302-309). 0 on invalid shape. */
+size_t w4a32_packed_bytes(int N, int K);
+
+/* Bytes of the per-call activation workspace for M rows.
+ * Replaces ...::workspace_size (kai_linear.cpp:293-300), called at
+ * mllm/Backends/Arm/Ops/LinearOp.cpp:74-78. 0 on invalid shape. */
+size_t w4a32_workspace_bytes(int M, int K);
+
+/* Bytes of the row-major 4-bit plane ([N][K/2]) and of the bf16 scale plane ([N][K/32])
+ * (get_rhs_native_stride / get_rhs_scale_stride, kai_linear.cpp:317-318). */
+size_t w4a32_native_u4_bytes(int N, int K);
+size_t w4a32_native_scale_bytes(int N, int K);
+
+/* ---- offline: weights -------------------------------------------------------------- */
+
+/* f32 weights [N][K] row-major -> row-major offset-8 nibbles (even k in the low nibble)
+ * + bf16 block scales. Bit-exact restatement of
+ * ...::quant_nxk_qs4c32_f32 (kai_linear.cpp:220-291). */
+int w4a32_quant_rhs_native(const float* d_w, int N, int K, uint8_t* d_u4, uint16_t* d_scales,
+                           int bf16_mode, void* stream);
+
+/* Row-major nibbles + scales (+ optional f32 bias [N], may be NULL) -> the device blob:
+ * 16-row x 128-k tiles laid out for 128-bit per-lane loads, block scales beside each
+ * tile, then per-row sums and bias. Takes the place of the
+ * kai_run_rhs_pack_nxk_qsi4c32p_qsu4c32s1s0 call (kai_linear.cpp:331-344). */
+int w4a32_repack_native(const uint8_t* d_u4, const uint16_t* d_scales, const float* d_bias, int N,
+                        int K, void* d_packed, void* stream);
+
+/* Both steps at once = ...::quant_pack_rhs_offline (kai_linear.cpp:311-348).
+ * d_tmp: scratch of w4a32_native_u4_bytes + w4a32_native_scale_bytes (u4 first). */
+int w4a32_quant_pack_rhs(const float* d_w, const float* d_bias, int N, int K, void* d_packed,
+                         void* d_tmp, int bf16_mode, void* stream);
+
+/* Inverse of w4a32_repack_native (d_bias may be NULL): recovers the row-major planes
+ * bit for bit. No counterpart in the reference (KleidiAI has no unpack); it exists so the
+ * layout can be checked and so blobs can be exported. */
+int w4a32_unpack_native(const void* d_packed, int N, int K, uint8_t* d_u4, uint16_t* d_scales,
+                        float* d_bias, void* stream);
+
+/* Blob -> f32 [N][K]: (u4 - 8) * f32(scale), the format's definition of a weight
+ * (tests/Arm/KaiLinearTest.hpp:355-361 unpack, :340 scale). */
+int w4a32_dequant(const void* d_packed, int N, int K, float* d_out, void* stream);
+
+/* ---- online: one forward ------------------------------------------------------------ */
+
+/* Per-row asymmetric int8 quantisation of the activations into the workspace
+ * (scale, offset, int8 values), bit-exact with the scalar model
+ * tests/Arm/KaiLinearTest.hpp:163-230. Replaces the kai_run_lhs_quant_pack_qai8dxp_f32
+ * call (kai_linear.cpp:358-362). ldx = row stride of d_x in elements. */
+int w4a32_quant_lhs(const float* d_x, int M, int K, int ldx, void* d_ws, void* stream);
+
+/* Copies the quantised rows out of a workspace for inspection: int8 [M][K], f32 [M]
+ * reciprocal scale, i32 [M] negated zero point (the row header of KaiLinearTest.hpp:208-214). */
+int w4a32_export_lhs(const void* d_ws, int M, int K, int8_t* d_aq, float* d_recip_scale,
+                     int32_t* d_neg_zero_point, void* stream);
+
+/* y[M][N] = clamp(lhs_scale * sum_b scale_b * sum_k (a_q + off) * q  + bias) on rows already
+ * quantised into d_ws. M <= W4A32_GEMV_MAX_M: decode kernels; larger M: prefill kernels.
+ * Replaces the tile loop + ukernel.run_matmul of ...::matmul (kai_linear.cpp:364-397). */
+int w4a32_matmul_quantized(float* d_y, const void* d_ws, const void* d_packed, int M, int K, int N,
+                           void* stream);
+
+/* The whole op = ...::matmul (kai_linear.cpp:350-398): quantise rows of d_x into d_ws,
+ * then multiply. d_ws must hold w4a32_workspace_bytes(M, K). */
+int w4a32_matmul(float* d_y, const float* d_x, const void* d_packed, void* d_ws, int M, int K,
+                 int N, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,192 @@
+"""MI355X-native W4A32 quantized Linear: Python binding of the C ABI (include/w4a32_hip.h).
+
+The product is libw4a32_hip.so (hand-written gfx950 kernels behind a C ABI) and the C++
+operator layer in host/. This module is plumbing: it loads the library with ctypes and
+passes torch tensors' device pointers through. There is no CPU fallback: if the library
+is missing or a call fails, an exception is raised.
+"""
+import ctypes
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libw4a32_hip.so")
+CSRC_DIR = os.path.join(_HERE, "csrc")
+HOST_DIR = os.path.join(_HERE, "host")
+
+BLOCK_LEN = 32
+GEMV_MAX_M = 8
+BF16_TRUNC = 0
+BF16_RNE = 1
+
+#: every symbol include/w4a32_hip.h declares, with (restype, argtypes)
+_vp, _ci, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+ABI = {
+    "w4a32_error_string": (ctypes.c_char_p, [_ci]),
+    "w4a32_abi_version": (_ci, []),
+    "w4a32_packed_bytes": (_sz, [_ci, _ci]),
+    "w4a32_workspace_bytes": (_sz, [_ci, _ci]),
+    "w4a32_native_u4_bytes": (_sz, [_ci, _ci]),
+    "w4a32_native_scale_bytes": (_sz, [_ci, _ci]),
+    "w4a32_quant_rhs_native": (_ci, [_vp, _ci, _ci, _vp, _vp, _ci, _vp]),
+    "w4a32_repack_native": (_ci, [_vp, _vp, _vp, _ci, _ci, _vp, _vp]),
+    "w4a32_quant_pack_rhs": (_ci, [_vp, _vp, _ci, _ci, _vp, _vp, _ci, _vp]),
+    "w4a32_unpack_native": (_ci, [_vp, _ci, _ci, _vp, _vp, _vp, _vp]),
+    "w4a32_dequant": (_ci, [_vp, _ci, _ci, _vp, _vp]),
+    "w4a32_quant_lhs": (_ci, [_vp, _ci, _ci, _ci, _vp, _vp]),
+    "w4a32_export_lhs": (_ci, [_vp, _ci, _ci, _vp, _vp, _vp, _vp]),
+    "w4a32_matmul_quantized": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp]),
+    "w4a32_matmul": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
+}
+
+
+class W4A32Error(RuntimeError):
+    pass
+
+
+def build(force=True):
+    """Compile the HIP library for gfx950 with hipcc (cross-compiles without a GPU)."""
+    cmd = ["make", "-C", CSRC_DIR, "-j8"] + (["-B"] if force else [])
+    subprocess.check_call(cmd)
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    """The loaded C-ABI library. Raises if it has not been built: there is no fallback."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise W4A32Error(
+                f"{LIB_PATH} is missing: build it first (python -c 'import __graft_entry__ as g; "
+                "g.build()'). This package has no CPU or PyTorch fallback.")
+        L = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in ABI.items():
+            fn = getattr(L, name)  # AttributeError if the symbol is not exported
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def _check(code, what):
+    if code != 0:
+        msg = lib().w4a32_error_string(code).decode()
+        raise W4A32Error(f"{what} failed: {msg} (code {code})")
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    import torch
+
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def packed_bytes(N, K):
+    return int(lib().w4a32_packed_bytes(N, K))
+
+
+def workspace_bytes(M, K):
+    return int(lib().w4a32_workspace_bytes(M, K))
+
+
+def _dev_empty(nbytes, dtype=None):
+    import torch
+
+    return torch.empty(nbytes, dtype=dtype or torch.uint8, device="cuda")
+
+
+def quant_rhs_native(w, bf16_mode=BF16_TRUNC):
+    """f32 cuda tensor [N,K] -> (u4 uint8 [N,K/2], scales int16-view-of-bf16 [N,K/32])."""
+    import torch
+
+    N, K = w.shape
+    assert w.is_cuda and w.dtype == torch.float32 and w.is_contiguous()
+    u4 = torch.empty((N, K // 2), dtype=torch.uint8, device="cuda")
+    sc = torch.empty((N, K // BLOCK_LEN), dtype=torch.int16, device="cuda")
+    _check(lib().w4a32_quant_rhs_native(_ptr(w), N, K, _ptr(u4), _ptr(sc), bf16_mode, _stream()),
+           "w4a32_quant_rhs_native")
+    return u4, sc
+
+
+def repack_native(u4, sc, bias, N, K):
+    packed = _dev_empty(packed_bytes(N, K))
+    _check(lib().w4a32_repack_native(_ptr(u4), _ptr(sc), _ptr(bias), N, K, _ptr(packed), _stream()),
+           "w4a32_repack_native")
+    return packed
+
+
+def quant_pack_rhs(w, bias=None, bf16_mode=BF16_TRUNC):
+    N, K = w.shape
+    L = lib()
+    packed = _dev_empty(packed_bytes(N, K))
+    tmp = _dev_empty(int(L.w4a32_native_u4_bytes(N, K)) + int(L.w4a32_native_scale_bytes(N, K)))
+    _check(L.w4a32_quant_pack_rhs(_ptr(w), _ptr(bias), N, K, _ptr(packed), _ptr(tmp), bf16_mode,
+                                  _stream()), "w4a32_quant_pack_rhs")
+    return packed
+
+
+def unpack_native(packed, N, K, want_bias=True):
+    import torch
+
+    u4 = torch.empty((N, K // 2), dtype=torch.uint8, device="cuda")
+    sc = torch.empty((N, K // BLOCK_LEN), dtype=torch.int16, device="cuda")
+    bias = torch.empty((N,), dtype=torch.float32, device="cuda") if want_bias else None
+    _check(lib().w4a32_unpack_native(_ptr(packed), N, K, _ptr(u4), _ptr(sc), _ptr(bias), _stream()),
+           "w4a32_unpack_native")
+    return u4, sc, bias
+
+
+def dequant(packed, N, K):
+    import torch
+
+    out = torch.empty((N, K), dtype=torch.float32, device="cuda")
+    _check(lib().w4a32_dequant(_ptr(packed), N, K, _ptr(out), _stream()), "w4a32_dequant")
+    return out
+
+
+def quant_lhs(x, ws=None):
+    M, K = x.shape
+    if ws is None:
+        ws = _dev_empty(workspace_bytes(M, K))
+    _check(lib().w4a32_quant_lhs(_ptr(x), M, K, x.stride(0), _ptr(ws), _stream()), "w4a32_quant_lhs")
+    return ws
+
+
+def export_lhs(ws, M, K):
+    import torch
+
+    aq = torch.empty((M, K), dtype=torch.int8, device="cuda")
+    recip = torch.empty((M,), dtype=torch.float32, device="cuda")
+    neg_zp = torch.empty((M,), dtype=torch.int32, device="cuda")
+    _check(lib().w4a32_export_lhs(_ptr(ws), M, K, _ptr(aq), _ptr(recip), _ptr(neg_zp), _stream()),
+           "w4a32_export_lhs")
+    return aq, recip, neg_zp
+
+
+def matmul_quantized(ws, packed, M, K, N, out=None):
+    import torch
+
+    y = out if out is not None else torch.empty((M, N), dtype=torch.float32, device="cuda")
+    _check(lib().w4a32_matmul_quantized(_ptr(y), _ptr(ws), _ptr(packed), M, K, N, _stream()),
+           "w4a32_matmul_quantized")
+    return y
+
+
+def matmul(x, packed, N, ws=None, out=None):
+    """The whole op on a contiguous f32 cuda tensor x [M,K]."""
+    import torch
+
+    M, K = x.shape
+    assert x.is_cuda and x.dtype == torch.float32 and x.is_contiguous()
+    if ws is None:
+        ws = _dev_empty(workspace_bytes(M, K))
+    y = out if out is not None else torch.empty((M, N), dtype=torch.float32, device="cuda")
+    _check(lib().w4a32_matmul(_ptr(y), _ptr(x), _ptr(packed), _ptr(ws), M, K, N, _stream()),
+           "w4a32_matmul")
+    return y

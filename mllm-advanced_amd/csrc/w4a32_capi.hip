@@ -1,0 +1,146 @@
+// The extern "C" surface declared in include/w4a32_hip.h: argument checks, geometry,
+// dispatch to the launchers. Nothing here allocates, frees or synchronises.
+#include "w4a32_hip.h"
+
+#include "w4a32_internal.h"
+
+namespace {
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+inline int shape_ok(int N, int K) {
+  if (N <= 0 || K <= 0) return W4A32_EINVAL;
+  if (K % w4::kBlockLen != 0) return W4A32_ESHAPE;
+  return W4A32_OK;
+}
+
+inline int from_hip(hipError_t e) { return e == hipSuccess ? W4A32_OK : W4A32_ELAUNCH; }
+
+}  // namespace
+
+extern "C" {
+
+const char* w4a32_error_string(int code) {
+  switch (code) {
+    case W4A32_OK: return "ok";
+    case W4A32_EINVAL: return "invalid argument (null/misaligned pointer or non-positive size)";
+    case W4A32_ESHAPE: return "unsupported shape (K must be a multiple of 32; M must fit the kernel)";
+    case W4A32_ELAUNCH: return "HIP launch failed";
+    case W4A32_ENOTSUP: return "not supported by this build";
+    default: return "unknown error";
+  }
+}
+
+int w4a32_abi_version(void) { return 1; }
+
+size_t w4a32_packed_bytes(int N, int K) {
+  if (shape_ok(N, K) != W4A32_OK) return 0;
+  return w4::weight_geom(N, K).total_bytes;
+}
+
+size_t w4a32_workspace_bytes(int M, int K) {
+  if (M <= 0 || shape_ok(1, K) != W4A32_OK) return 0;
+  return w4::ws_geom(M, K).total_bytes;
+}
+
+size_t w4a32_native_u4_bytes(int N, int K) {
+  if (shape_ok(N, K) != W4A32_OK) return 0;
+  return (size_t)N * (K / 2);
+}
+
+size_t w4a32_native_scale_bytes(int N, int K) {
+  if (shape_ok(N, K) != W4A32_OK) return 0;
+  return (size_t)N * (K / w4::kBlockLen) * sizeof(uint16_t);
+}
+
+int w4a32_quant_rhs_native(const float* d_w, int N, int K, uint8_t* d_u4, uint16_t* d_scales,
+                           int bf16_mode, void* stream) {
+  if (int e = shape_ok(N, K)) return e;
+  if (!d_w || !d_u4 || !d_scales) return W4A32_EINVAL;
+  if (!aligned(d_w, 16) || !aligned(d_u4, 16) || !aligned(d_scales, 2)) return W4A32_EINVAL;
+  if (bf16_mode != W4A32_BF16_TRUNC && bf16_mode != W4A32_BF16_RNE) return W4A32_EINVAL;
+  return from_hip(w4::launch_quant_rhs(d_w, N, K, d_u4, d_scales, bf16_mode,
+                                       static_cast<hipStream_t>(stream)));
+}
+
+int w4a32_repack_native(const uint8_t* d_u4, const uint16_t* d_scales, const float* d_bias, int N,
+                        int K, void* d_packed, void* stream) {
+  if (int e = shape_ok(N, K)) return e;
+  if (!d_u4 || !d_scales || !d_packed) return W4A32_EINVAL;
+  if (!aligned(d_u4, 16) || !aligned(d_scales, 2) || !aligned(d_packed, 16)) return W4A32_EINVAL;
+  return from_hip(w4::launch_repack(d_u4, d_scales, d_bias, N, K, static_cast<uint8_t*>(d_packed),
+                                    static_cast<hipStream_t>(stream)));
+}
+
+int w4a32_quant_pack_rhs(const float* d_w, const float* d_bias, int N, int K, void* d_packed,
+                         void* d_tmp, int bf16_mode, void* stream) {
+  if (int e = shape_ok(N, K)) return e;
+  if (!d_tmp || !aligned(d_tmp, 16)) return W4A32_EINVAL;
+  uint8_t* u4 = static_cast<uint8_t*>(d_tmp);
+  uint16_t* sc = reinterpret_cast<uint16_t*>(u4 + w4a32_native_u4_bytes(N, K));
+  if (int e = w4a32_quant_rhs_native(d_w, N, K, u4, sc, bf16_mode, stream)) return e;
+  return w4a32_repack_native(u4, sc, d_bias, N, K, d_packed, stream);
+}
+
+int w4a32_unpack_native(const void* d_packed, int N, int K, uint8_t* d_u4, uint16_t* d_scales,
+                        float* d_bias, void* stream) {
+  if (int e = shape_ok(N, K)) return e;
+  if (!d_packed || !d_u4 || !d_scales) return W4A32_EINVAL;
+  if (!aligned(d_packed, 16) || !aligned(d_u4, 4) || !aligned(d_scales, 2)) return W4A32_EINVAL;
+  return from_hip(w4::launch_unpack(static_cast<const uint8_t*>(d_packed), N, K, d_u4, d_scales,
+                                    d_bias, static_cast<hipStream_t>(stream)));
+}
+
+int w4a32_dequant(const void* d_packed, int N, int K, float* d_out, void* stream) {
+  if (int e = shape_ok(N, K)) return e;
+  if (!d_packed || !d_out) return W4A32_EINVAL;
+  if (!aligned(d_packed, 16) || !aligned(d_out, 16)) return W4A32_EINVAL;
+  return from_hip(w4::launch_dequant(static_cast<const uint8_t*>(d_packed), N, K, d_out,
+                                     static_cast<hipStream_t>(stream)));
+}
+
+int w4a32_quant_lhs(const float* d_x, int M, int K, int ldx, void* d_ws, void* stream) {
+  if (M <= 0) return W4A32_EINVAL;
+  if (int e = shape_ok(1, K)) return e;
+  if (!d_x || !d_ws || ldx < K) return W4A32_EINVAL;
+  if (!aligned(d_x, 16) || (ldx % 4) != 0 || !aligned(d_ws, 256)) return W4A32_EINVAL;
+  return from_hip(w4::launch_quant_lhs(d_x, M, K, ldx, static_cast<uint8_t*>(d_ws),
+                                       static_cast<hipStream_t>(stream)));
+}
+
+int w4a32_export_lhs(const void* d_ws, int M, int K, int8_t* d_aq, float* d_recip_scale,
+                     int32_t* d_neg_zero_point, void* stream) {
+  if (M <= 0) return W4A32_EINVAL;
+  if (int e = shape_ok(1, K)) return e;
+  if (!d_ws || !d_aq || !d_recip_scale || !d_neg_zero_point) return W4A32_EINVAL;
+  const w4::WsGeom g = w4::ws_geom(M, K);
+  const uint8_t* ws = static_cast<const uint8_t*>(d_ws);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipError_t e = hipMemcpyAsync(d_aq, ws + g.aq_off, (size_t)M * K, hipMemcpyDeviceToDevice, s);
+  if (e == hipSuccess)
+    e = hipMemcpyAsync(d_recip_scale, ws + g.scale_off, (size_t)M * 4, hipMemcpyDeviceToDevice, s);
+  if (e == hipSuccess)
+    e = hipMemcpyAsync(d_neg_zero_point, ws + g.off_off, (size_t)M * 4, hipMemcpyDeviceToDevice, s);
+  return from_hip(e);
+}
+
+int w4a32_matmul_quantized(float* d_y, const void* d_ws, const void* d_packed, int M, int K, int N,
+                           void* stream) {
+  if (M <= 0) return W4A32_EINVAL;
+  if (int e = shape_ok(N, K)) return e;
+  if (!d_y || !d_ws || !d_packed) return W4A32_EINVAL;
+  if (!aligned(d_ws, 256) || !aligned(d_packed, 16) || !aligned(d_y, 4)) return W4A32_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const uint8_t* ws = static_cast<const uint8_t*>(d_ws);
+  const uint8_t* pk = static_cast<const uint8_t*>(d_packed);
+  if (M <= w4::kGemvMaxM) return from_hip(w4::launch_gemv(d_y, ws, pk, M, K, N, s));
+  return from_hip(w4::launch_gemm(d_y, ws, pk, M, K, N, s));
+}
+
+int w4a32_matmul(float* d_y, const float* d_x, const void* d_packed, void* d_ws, int M, int K,
+                 int N, void* stream) {
+  if (int e = w4a32_quant_lhs(d_x, M, K, K, d_ws, stream)) return e;
+  return w4a32_matmul_quantized(d_y, d_ws, d_packed, M, K, N, stream);
+}
+
+}  // extern "C"

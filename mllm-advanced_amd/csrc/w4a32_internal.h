@@ -1,0 +1,31 @@
+// Launchers behind the C ABI. Each returns hipError_t of the launch; arguments are already
+// validated by the caller (w4a32_capi.hip).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "w4a32_layout.h"
+
+namespace w4 {
+
+// weights (offline)
+hipError_t launch_quant_rhs(const float* w, int N, int K, uint8_t* u4, uint16_t* scales, int rne,
+                            hipStream_t s);
+hipError_t launch_repack(const uint8_t* u4, const uint16_t* scales, const float* bias, int N, int K,
+                         uint8_t* packed, hipStream_t s);
+hipError_t launch_unpack(const uint8_t* packed, int N, int K, uint8_t* u4, uint16_t* scales,
+                         float* bias, hipStream_t s);
+hipError_t launch_dequant(const uint8_t* packed, int N, int K, float* out, hipStream_t s);
+
+// activations (every forward)
+hipError_t launch_quant_lhs(const float* x, int M, int K, int ldx, uint8_t* ws, hipStream_t s);
+
+// products
+hipError_t launch_gemv(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
+                       hipStream_t s);
+hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
+                       hipStream_t s);
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+
+}  // namespace w4

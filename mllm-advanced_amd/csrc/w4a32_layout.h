@@ -1,0 +1,98 @@
+// Device data layouts of the W4A32 Linear on MI355X, shared by host and kernels.
+//
+// WEIGHT BLOB ("tiles | rsum | bias"), for an [N][K] Linear, K % 32 == 0:
+//
+//   Np = N rounded up to 16, Kp = K rounded up to 128 (padding holds q = 0, scale = +0).
+//   tiles: tile (nt, kc) covers rows 16*nt .. +15 and k 128*kc .. +127 (four scale blocks)
+//          and occupies kTileBytes = 1152 contiguous bytes at ((nt * KC) + kc) * 1152:
+//
+//     [0, 1024)    64 lanes x 16 B. Lane l = 16*g + j  (g = k-group 0..3, j = row in tile)
+//                  holds four dwords; dword d belongs to scale block 4*kc + d and carries the
+//                  8 weights of row 16*nt + j at k = 128*kc + 32*d + 8*g + (0..7).
+//                  One wavefront-wide 128-bit load therefore reads 1 KiB contiguous, and
+//                  dword d of all 64 lanes is exactly the B operand of one 16x16x32 MFMA
+//                  (n = j, k-slice = g) that stays inside ONE scale block.
+//                  Inside a dword, nibble position 2e holds k offset e, position 2e+1 holds
+//                  k offset 4+e (e = 0..3), each as 4-bit two's complement of q = u4 - 8.
+//                  So (w << 4) & 0xF0F0F0F0 are the int8 values 16*q of k offsets 0..3 and
+//                  w & 0xF0F0F0F0 those of offsets 4..7: two ops per 8 weights, no sign fix.
+//     [1024, 1152) 16 rows x 4 bf16 scales: scale of (row j, block 4*kc + d) at 1024 + 8*j + 2*d.
+//
+//   rsum:  f32 [Np] at tiles_bytes: sum_b f32(scale_b) * (float)(sum_{k in b} q), accumulated
+//          in block order. Lets the int8 kernels add the activation offset once per output:
+//          sum_k (a_q + off) q s = sum_k a_q q s + off * rsum.
+//   bias:  f32 [Np] after rsum (zeros when the layer has none).
+//
+// ACTIVATION WORKSPACE for M rows (Mp = M rounded up to 16):
+//
+//   [0, 4*Mp)            f32  recip_scale[m]   (the "lhs scale" applied to the output)
+//   [4*Mp, 8*Mp)         i32  neg_zp[m]        (the "lhs offset" = -zero_point)
+//   hdr = round_up(8*Mp, 256)
+//   [hdr, hdr + Mp*K)    i8   a_q[m][k] row-major
+//   then, 256-aligned    f16  a_h[m][k] = (a_q + neg_zp) exactly, only written when M > 8
+#pragma once
+
+#include <stddef.h>
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define W4_HD __host__ __device__ inline
+#else
+#define W4_HD inline
+#endif
+
+namespace w4 {
+
+constexpr int kBlockLen = 32;
+constexpr int kTileRows = 16;
+constexpr int kTileK = 128;
+constexpr int kTileQBytes = 1024;
+constexpr int kTileScaleBytes = 128;
+constexpr int kTileBytes = kTileQBytes + kTileScaleBytes;
+constexpr int kGemvMaxM = 8;
+
+W4_HD int round_up(int v, int m) { return (v + m - 1) / m * m; }
+W4_HD size_t round_up_sz(size_t v, size_t m) { return (v + m - 1) / m * m; }
+
+struct WeightGeom {
+  int N, K, Np, Kp, NT, KC;
+  size_t tiles_bytes, rsum_off, bias_off, total_bytes;
+};
+
+W4_HD WeightGeom weight_geom(int N, int K) {
+  WeightGeom g;
+  g.N = N;
+  g.K = K;
+  g.Np = round_up(N, kTileRows);
+  g.Kp = round_up(K, kTileK);
+  g.NT = g.Np / kTileRows;
+  g.KC = g.Kp / kTileK;
+  g.tiles_bytes = (size_t)g.NT * g.KC * kTileBytes;
+  g.rsum_off = g.tiles_bytes;
+  g.bias_off = g.rsum_off + (size_t)g.Np * 4;
+  g.total_bytes = g.bias_off + (size_t)g.Np * 4;
+  return g;
+}
+
+struct WsGeom {
+  int M, K, Mp;
+  size_t scale_off, off_off, aq_off, ah_off, total_bytes;
+};
+
+W4_HD WsGeom ws_geom(int M, int K) {
+  WsGeom g;
+  g.M = M;
+  g.K = K;
+  g.Mp = round_up(M, 16);
+  g.scale_off = 0;
+  g.off_off = (size_t)4 * g.Mp;
+  g.aq_off = round_up_sz((size_t)8 * g.Mp, 256);
+  g.ah_off = g.aq_off + round_up_sz((size_t)g.Mp * K, 256);
+  g.total_bytes = g.ah_off + (M > kGemvMaxM ? (size_t)g.Mp * K * 2 : 0);
+  return g;
+}
+
+// Nibble position (0..7) inside a tile dword of the weight at k offset e (0..7) in its 8-group.
+W4_HD int nibble_pos(int e) { return e < 4 ? 2 * e : 2 * (e - 4) + 1; }
+
+}  // namespace w4

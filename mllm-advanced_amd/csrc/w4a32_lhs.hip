@@ -1,0 +1,111 @@
+// Per-row asymmetric int8 quantisation of the activations (runs in every forward).
+//
+// Bit-exact with the scalar model the reference's test holds
+// (tests/Arm/KaiLinearTest.hpp:166-228): range always contains 0, scale = 255 / (rmax - rmin),
+// the zero point is taken from the side with the smaller error, clamped, rounded to nearest
+// even; values are round_half_away(x * scale) + zero_point, clamped to int8. Every f32 product
+// and sum is an explicitly rounded intrinsic so no compiler flag can fuse them.
+#include "w4a32_internal.h"
+
+namespace w4 {
+
+__device__ __forceinline__ float wave_min(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+constexpr int kLhsThreads = 256;
+
+// One workgroup per row. Pass 1 reads the row for min/max, pass 2 re-reads it (it is L2/L1
+// resident: at most 35 KB) and writes 4 int8 per thread per step, plus the f16 copy of
+// (a_q - zp) that the f16 MFMA prefill kernel consumes.
+__global__ __launch_bounds__(kLhsThreads) void quant_lhs_kernel(
+    const float* __restrict__ x, int K, int ldx, float* __restrict__ recip_out,
+    int32_t* __restrict__ negzp_out, int8_t* __restrict__ aq, _Float16* __restrict__ ah) {
+  const int m = blockIdx.x;
+  const int t = threadIdx.x;
+  const float* row = x + (size_t)m * ldx;
+
+  float lo = 3.402823466e+38f, hi = -3.402823466e+38f;
+  for (int i = 4 * t; i < K; i += 4 * kLhsThreads) {
+    const float4 v = *reinterpret_cast<const float4*>(row + i);
+    lo = fminf(fminf(lo, v.x), fminf(v.y, fminf(v.z, v.w)));
+    hi = fmaxf(fmaxf(hi, v.x), fmaxf(v.y, fmaxf(v.z, v.w)));
+  }
+  lo = wave_min(lo);
+  hi = wave_max(hi);
+  __shared__ float s_lo[kLhsThreads / 64], s_hi[kLhsThreads / 64];
+  if ((t & 63) == 0) {
+    s_lo[t >> 6] = lo;
+    s_hi[t >> 6] = hi;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < kLhsThreads / 64; ++w) {
+    lo = fminf(lo, s_lo[w]);
+    hi = fmaxf(hi, s_hi[w]);
+  }
+
+  const float qmin = -128.0f, qmax = 127.0f;
+  const float rmin = (lo < 0.0f) ? lo : 0.0f;
+  const float rmax = (hi > 0.0f) ? hi : 0.0f;
+  const float scale = (rmin == rmax) ? 1.0f : __fdiv_rn(255.0f, __fsub_rn(rmax, rmin));
+  const float recip = (scale != 0.0f) ? __fdiv_rn(1.0f, scale) : 0.0f;
+  const float dmin = __fmul_rn(rmin, scale);
+  const float dmax = __fmul_rn(rmax, scale);
+  const float err_min = __fadd_rn(qmin, dmin);
+  const float err_max = __fadd_rn(qmax, dmax);
+  float zpf = (__fadd_rn(err_min, err_max) > 0.0f) ? __fsub_rn(qmin, dmin) : __fsub_rn(qmax, dmax);
+  zpf = fminf(fmaxf(zpf, qmin), qmax);
+  const int zp = __float2int_rn(zpf);  // nearest even, as lrintf in the default mode
+
+  if (t == 0) {
+    recip_out[m] = recip;
+    negzp_out[m] = -zp;
+  }
+
+  int8_t* dst = aq + (size_t)m * K;
+  for (int i = 4 * t; i < K; i += 4 * kLhsThreads) {
+    const float4 v = *reinterpret_cast<const float4*>(row + i);
+    const float f[4] = {v.x, v.y, v.z, v.w};
+    int q[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      int r = (int)roundf(__fmul_rn(f[e], scale)) + zp;  // |x*scale| <= 255: the cast is safe
+      r = r < -128 ? -128 : r;
+      r = r > 127 ? 127 : r;
+      q[e] = r;
+    }
+    const uint32_t packed = (uint32_t)(q[0] & 0xFF) | ((uint32_t)(q[1] & 0xFF) << 8) |
+                            ((uint32_t)(q[2] & 0xFF) << 16) | ((uint32_t)(q[3] & 0xFF) << 24);
+    *reinterpret_cast<uint32_t*>(dst + i) = packed;
+    if (ah) {
+      // a_q - zp lies in [-255, 255]: exact in f16
+      typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+      h4 hv;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) hv[e] = (_Float16)(float)(q[e] - zp);
+      *reinterpret_cast<h4*>(ah + (size_t)m * K + i) = hv;
+    }
+  }
+}
+
+hipError_t launch_quant_lhs(const float* x, int M, int K, int ldx, uint8_t* ws, hipStream_t s) {
+  const WsGeom g = ws_geom(M, K);
+  float* recip = reinterpret_cast<float*>(ws + g.scale_off);
+  int32_t* negzp = reinterpret_cast<int32_t*>(ws + g.off_off);
+  int8_t* aq = reinterpret_cast<int8_t*>(ws + g.aq_off);
+  _Float16* ah = (M > kGemvMaxM) ? reinterpret_cast<_Float16*>(ws + g.ah_off) : nullptr;
+  hipLaunchKernelGGL(quant_lhs_kernel, dim3(M), dim3(kLhsThreads), 0, s, x, K, ldx, recip, negzp,
+                     aq, ah);
+  return hipGetLastError();
+}
+
+}  // namespace w4

@@ -1,0 +1,288 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle on the same inputs.
+
+Integer/byte results (weight nibbles, bf16 scales, int8 activations, zero points, the
+repacked blob's round trip, dequantised weights) must be bit-exact. f32 outputs must be
+within max|y - ref| / max|ref| <= 1e-3 for the decode kernels (M <= 8) and <= 2e-3 for the
+prefill kernels, the tolerances the target states; since the block sums are exact integers
+on both sides the observed error is near 1e-6, and the tests also hold it to 2e-5.
+"""
+import numpy as np
+import pytest
+import torch
+
+from conftest import make_acts, make_weights, max_abs_rel
+
+pytestmark = pytest.mark.gpu
+
+GEMV_TOL = 1e-3
+GEMM_TOL = 2e-3
+TIGHT = 2e-5
+
+# (name, K, N, has_bias) - the Qwen2-1.5B linears, lm_head, and the Qwen2-VL ViT linears
+DECODER_SHAPES = [
+    ("q_proj", 1536, 1536, True),
+    ("kv_proj", 1536, 256, True),
+    ("o_proj", 1536, 1536, False),
+    ("gate_up", 1536, 8960, False),
+    ("down", 8960, 1536, False),
+]
+LM_HEAD = ("lm_head", 1536, 151936, False)
+VIT_SHAPES = [
+    ("vit_qkv", 1280, 3840, True),
+    ("vit_proj", 1280, 1280, True),
+    ("vit_fc1", 1280, 5120, True),
+    ("vit_fc2", 5120, 1280, True),
+]
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def bias_for(n, has_bias, seed=2):
+    if not has_bias:
+        return None
+    return (np.random.default_rng(seed).standard_normal(n) * 0.02).astype(np.float32)
+
+
+# ------------------------------------------------------------------- weights (offline)
+
+SPECIAL_W = "special"
+
+
+def special_weights():
+    """Blocks that exercise the quantizer's corner rules."""
+    w = make_weights(32, 256, seed=13)
+    w[0, :32] = 0.0                       # zero block -> scale -0.0, bytes 0x88
+    w[1, :32] = 0.5                       # constant block -> all -8
+    w[2, :32] = 0.0
+    w[2, 3], w[2, 7] = 2.0, -2.0          # tie: the first maximum wins, q[7] clamps to 7
+    w[3, :32] = 0.0
+    w[3, 0] = -1.0                        # scale 2^-3; exact .5 ties round away from zero
+    w[3, 1:8] = np.array([0.5, 1.5, 2.5, -0.5, -2.5, 6.5, 7.5], np.float32) * 0.125
+    w[4, 32:64] = -w[5, 32:64]            # negated block: same nibbles, flipped scale
+    return w
+
+
+@pytest.mark.parametrize("n,k,seed", [(32, 256, SPECIAL_W), (64, 128, 0), (1536, 1536, 1),
+                                      (256, 8960, 2), (50, 96, 3)])
+@pytest.mark.parametrize("mode", [0, 1])
+def test_quant_rhs_bit_exact(pkg, orc, n, k, seed, mode):
+    w = special_weights() if seed == SPECIAL_W else make_weights(n, k, seed=seed)
+    u4_ref, sc_ref = orc.quant_rhs(w, bf16_rne_mode=bool(mode))
+    u4, sc = pkg.quant_rhs_native(dev(w), bf16_mode=mode)
+    assert np.array_equal(host(u4), u4_ref)
+    assert np.array_equal(host(sc).view(np.uint16), sc_ref)
+
+
+@pytest.mark.parametrize("n,k", [(16, 128), (50, 96), (1536, 1536), (256, 8960), (3, 32)])
+def test_repack_round_trip_and_dequant_bit_exact(pkg, orc, n, k):
+    rng = np.random.default_rng(n * 7 + k)
+    u4 = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)           # any byte pattern
+    sc = (rng.standard_normal((n, k // 32)).astype(np.float32) * 0.01).view(np.uint32) >> 16
+    sc = sc.astype(np.uint16)
+    bias = rng.standard_normal(n).astype(np.float32)
+    packed = pkg.repack_native(dev(u4), dev(sc.view(np.int16)), dev(bias), n, k)
+    assert packed.numel() == pkg.packed_bytes(n, k)
+    u4_b, sc_b, bias_b = pkg.unpack_native(packed, n, k)
+    assert np.array_equal(host(u4_b), u4)
+    assert np.array_equal(host(sc_b).view(np.uint16), sc)
+    assert np.array_equal(host(bias_b), bias)
+    deq = host(pkg.dequant(packed, n, k))
+    assert np.array_equal(deq.view(np.uint32), orc.dequant(u4, sc, k).view(np.uint32))
+
+
+def test_quant_pack_equals_two_steps(pkg, orc):
+    w = make_weights(48, 256, seed=4)
+    b = bias_for(48, True)
+    one = pkg.quant_pack_rhs(dev(w), dev(b))
+    u4, sc = pkg.quant_rhs_native(dev(w))
+    two = pkg.repack_native(u4, sc, dev(b), 48, 256)
+    assert torch.equal(one, two)
+    u4_ref, sc_ref = orc.quant_rhs(w)
+    deq = host(pkg.dequant(one, 48, 256))
+    assert np.array_equal(deq.view(np.uint32), orc.dequant(u4_ref, sc_ref, 256).view(np.uint32))
+
+
+# ------------------------------------------------------------ activations (every forward)
+
+def special_acts(k):
+    x = make_acts(12, k, seed=5)
+    x[0] = 0.0                                   # zero row: scale 1, zp 127
+    x[1] = 0.0
+    x[1, 5] = 4.0                                # one-sided positive: zp -128
+    x[2] = 0.0
+    x[2, 9] = -4.0                               # one-sided negative: zp 127
+    x[3] = 0.0
+    x[3, 0], x[3, 1] = 2.0, -2.0                 # symmetric: zp -0.5 -> nearest even -> 0
+    x[4] = 0.0
+    x[4, :6] = [-100.0, 155.0, 0.5, 1.5, -0.5, -2.5]   # scale 1: .5 ties round away from zero
+    x[5] *= 20.0                                 # outlier row
+    x[6] = np.abs(x[6])                          # all positive
+    x[7] = -np.abs(x[7])                         # all negative
+    x[8] *= 1e-6                                 # tiny
+    x[9] *= 1e6                                  # huge
+    return x
+
+
+@pytest.mark.parametrize("m,k,seed", [(12, 1536, "special"), (12, 32, "special"), (1, 1536, 1),
+                                      (8, 8960, 2), (64, 1280, 3), (300, 5120, 4)])
+def test_quant_lhs_bit_exact(pkg, orc, m, k, seed):
+    x = special_acts(k) if seed == "special" else make_acts(m, k, seed=seed, outlier_frac=0.05)
+    aq_ref, recip_ref, negzp_ref, _ = orc.quant_lhs(x)
+    ws = pkg.quant_lhs(dev(x))
+    aq, recip, negzp = pkg.export_lhs(ws, x.shape[0], k)
+    assert np.array_equal(host(negzp), negzp_ref)
+    assert np.array_equal(host(recip).view(np.uint32), recip_ref.view(np.uint32))
+    assert np.array_equal(host(aq), aq_ref)
+
+
+# ------------------------------------------------------------------------- products
+
+def run_linear(pkg, orc, m, k, n, has_bias, wseed=0, xseed=1, outliers=0.0, threads=8, rows=None):
+    w = make_weights(n, k, seed=wseed)
+    x = make_acts(m, k, seed=xseed, outlier_frac=outliers)
+    bias = bias_for(n, has_bias)
+    u4, sc = orc.quant_rhs(w)
+    packed = pkg.repack_native(dev(u4), dev(sc.view(np.int16)), None if bias is None else dev(bias),
+                               n, k)
+    y = host(pkg.matmul(dev(x), packed, n))
+    if rows is None:
+        ref = orc.linear(x, u4, sc, bias=bias, threads=threads)
+        return y, ref
+    ref = orc.linear(x[rows], u4, sc, bias=bias, threads=threads)   # rows are independent
+    return y[rows], ref
+
+
+@pytest.mark.parametrize("name,k,n,has_bias", DECODER_SHAPES + VIT_SHAPES)
+@pytest.mark.parametrize("m", [1, 4, 8])
+def test_gemv_matches_oracle(pkg, orc, name, k, n, has_bias, m):
+    y, ref = run_linear(pkg, orc, m, k, n, has_bias)
+    err = max_abs_rel(y, ref)
+    assert err <= GEMV_TOL and err <= TIGHT, (name, m, err)
+
+
+@pytest.mark.parametrize("m", [2, 3, 5, 6, 7])
+def test_gemv_every_m(pkg, orc, m):
+    y, ref = run_linear(pkg, orc, m, 1536, 256, True, outliers=0.3)
+    assert max_abs_rel(y, ref) <= TIGHT
+
+
+@pytest.mark.parametrize("m", [1, 8])
+def test_gemv_lm_head(pkg, orc, m):
+    name, k, n, has_bias = LM_HEAD
+    y, ref = run_linear(pkg, orc, m, k, n, has_bias)
+    err = max_abs_rel(y, ref)
+    assert err <= GEMV_TOL and err <= TIGHT, err
+
+
+@pytest.mark.parametrize("m,k,n", [(1, 32, 16), (3, 64, 5), (8, 96, 50), (1, 1024, 1024)])
+def test_gemv_ragged_shapes(pkg, orc, m, k, n):
+    # N not a multiple of 16, K not a multiple of 128: padding inside the tiles must be inert
+    y, ref = run_linear(pkg, orc, m, k, n, True, wseed=m + k, xseed=n)
+    assert max_abs_rel(y, ref) <= TIGHT
+
+
+def exact_case(m, n, k, seed):
+    rng = np.random.default_rng(seed)
+    x = rng.integers(-100, 156, size=(m, k)).astype(np.float32)
+    x[:, 0], x[:, 1] = -100.0, 155.0
+    q = rng.integers(-8, 8, size=(n, k)).astype(np.int64)
+    e = rng.integers(-7, -1, size=(n, k // 32))
+    for r in range(n):
+        for b in range(k // 32):
+            q[r, 32 * b + int(rng.integers(0, 32))] = -8
+    return x, (q * np.exp2(np.repeat(e, 32, axis=1))).astype(np.float32)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 48, 256), (8, 33, 512), (40, 64, 256), (130, 20, 128)])
+def test_lossless_inputs_give_the_exact_dense_product(pkg, m, n, k):
+    # Inputs both quantizers represent exactly, with every partial sum below 2^24: the op
+    # must equal a float64 matmul bit for bit. Fails on any wrong index, sign, nibble order,
+    # scale pairing or operand layout, independently of the oracle.
+    x, w = exact_case(m, n, k, seed=m + n)
+    packed = pkg.quant_pack_rhs(dev(w))
+    y = host(pkg.matmul(dev(x), packed, n)).astype(np.float64)
+    assert np.array_equal(y, x.astype(np.float64) @ w.astype(np.float64).T)
+
+
+@pytest.mark.parametrize("name,k,n,has_bias", DECODER_SHAPES)
+@pytest.mark.parametrize("m", [128, 512])
+def test_gemm_matches_oracle(pkg, orc, name, k, n, has_bias, m):
+    # 1 % of rows scaled x20 stresses the per-row activation scales
+    rows = None if m * n * k <= 2 ** 31 else np.unique(
+        np.concatenate([np.arange(0, m, 37), [m - 1]]))
+    y, ref = run_linear(pkg, orc, m, k, n, has_bias, outliers=0.01, rows=rows)
+    err = max_abs_rel(y, ref)
+    assert err <= GEMM_TOL and err <= TIGHT, (name, m, err)
+
+
+@pytest.mark.parametrize("name,k,n,has_bias", DECODER_SHAPES + VIT_SHAPES)
+def test_gemm_large_m_on_sampled_rows(pkg, orc, name, k, n, has_bias):
+    # M = 2048 (ViT: 1024): rows are independent, so the oracle checks a sample of them
+    m = 1024 if name.startswith("vit") else 2048
+    rows = np.unique(np.concatenate([np.arange(0, m, 101), [m - 1, m - 2, 63, 64, 65]]))
+    y, ref = run_linear(pkg, orc, m, k, n, has_bias, outliers=0.01, rows=rows)
+    err = max_abs_rel(y, ref)
+    assert err <= GEMM_TOL and err <= TIGHT, (name, err)
+
+
+@pytest.mark.parametrize("m", [9, 15, 16, 17, 63, 65, 100])
+def test_gemm_ragged_m(pkg, orc, m):
+    y, ref = run_linear(pkg, orc, m, 256, 50, True, outliers=0.1)
+    assert max_abs_rel(y, ref) <= TIGHT
+
+
+def test_gemm_rows_agree_with_gemv(pkg):
+    # size-independent property at a full prefill size: each row of the M=512 product equals
+    # the M=1 product of that row (different kernels, same integer block sums)
+    k, n, m = 1536, 8960, 512
+    w = make_weights(n, k, seed=0)
+    x = dev(make_acts(m, k, seed=1, outlier_frac=0.01))
+    packed = pkg.quant_pack_rhs(dev(w))
+    big = pkg.matmul(x, packed, n)
+    for r in (0, 5, 255, 511):
+        one = pkg.matmul(x[r:r + 1].contiguous(), packed, n)
+        assert max_abs_rel(host(one), host(big[r:r + 1])) <= TIGHT
+
+
+def test_weight_row_permutation_permutes_outputs(pkg):
+    k, n = 1536, 1536
+    w = make_weights(n, k, seed=3)
+    perm = np.random.default_rng(0).permutation(n)
+    x = dev(make_acts(4, k, seed=2))
+    y = host(pkg.matmul(x, pkg.quant_pack_rhs(dev(w)), n))
+    yp = host(pkg.matmul(x, pkg.quant_pack_rhs(dev(w[perm])), n))
+    assert np.array_equal(yp, y[:, perm])
+
+
+def test_golden_fixture(pkg):
+    g = np.load(__import__("os").path.join(__import__("os").path.dirname(__file__), "golden",
+                                           "w4a32_small.npz"))
+    packed = pkg.repack_native(dev(g["u4"]), dev(g["scales"].view(np.int16)), dev(g["bias"]),
+                               int(g["n"]), int(g["k"]))
+    ws = pkg.quant_lhs(dev(g["x"]))
+    aq, recip, negzp = pkg.export_lhs(ws, int(g["m"]), int(g["k"]))
+    assert np.array_equal(host(aq), g["aq"])
+    assert np.array_equal(host(negzp), g["neg_zp"])
+    assert np.array_equal(host(recip), g["recip"])
+    u4, sc = pkg.quant_rhs_native(dev(g["w"]))
+    assert np.array_equal(host(u4), g["u4"]) and np.array_equal(host(sc).view(np.uint16), g["scales"])
+    y = host(pkg.matmul(dev(g["x"]), packed, int(g["n"])))
+    assert max_abs_rel(y, g["y"]) <= TIGHT
+
+
+def test_bad_arguments_return_error_codes(pkg):
+    L = pkg.lib()
+    x = torch.zeros((1, 48), device="cuda")
+    assert L.w4a32_packed_bytes(16, 48) == 0                      # K % 32 != 0
+    assert L.w4a32_quant_lhs(x.data_ptr(), 1, 48, 48, x.data_ptr(), None) == -2
+    assert L.w4a32_quant_lhs(None, 1, 64, 64, x.data_ptr(), None) == -1
+    assert L.w4a32_matmul_quantized(None, None, None, 1, 64, 16, None) == -1
+    with pytest.raises(pkg.W4A32Error):
+        pkg._check(-2, "probe")
