@@ -98,8 +98,9 @@ __global__ __launch_bounds__(1024) void gemv_dot4_kernel(
   }
   __syncthreads();
 
-  if (threadIdx.x < 16 * M) {
-    const int m = threadIdx.x >> 4, jj = threadIdx.x & 15;
+  // 16*M outputs; a workgroup may have as few as 64 threads, so stride over them.
+  for (int o = threadIdx.x; o < 16 * M; o += blockDim.x) {
+    const int m = o >> 4, jj = o & 15;
     const int n = kTileRows * nt + jj;
     if (n < N) {
       float s = 0.0f;
