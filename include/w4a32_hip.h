@@ -109,6 +109,16 @@ int w4a32_export_lhs(const void* d_ws, int M, int K, int8_t* d_aq, float* d_reci
 int w4a32_matmul_quantized(float* d_y, const void* d_ws, const void* d_packed, int M, int K, int N,
                            void* stream);
 
+/* Same product with the kernel named by the caller (tests and benchmarks compare them).
+ * The reference picks its micro-kernel the same way, by a tile id argument
+ * (KaiLinear_f32_qai8dxp_qsi4c32p_mxk_nxk::Tiles, kai_linear.hpp:76-118). */
+#define W4A32_KERNEL_AUTO 0       /* M <= 8: GEMV, M <= 32: int8 MFMA, else f16 MFMA */
+#define W4A32_KERNEL_GEMV 1       /* v_dot4 decode kernel, M <= 8 */
+#define W4A32_KERNEL_GEMM_I8 2    /* int8 MFMA, exact int32 block sums, any M */
+#define W4A32_KERNEL_GEMM_F16 3   /* f16 MFMA on exact f16 operands, M > 8 */
+int w4a32_matmul_quantized_ex(float* d_y, const void* d_ws, const void* d_packed, int M, int K,
+                              int N, int kernel, void* stream);
+
 /* The whole op = ...::matmul (kai_linear.cpp:350-398): quantise rows of d_x into d_ws,
  * then multiply. d_ws must hold w4a32_workspace_bytes(M, K). */
 int w4a32_matmul(float* d_y, const float* d_x, const void* d_packed, void* d_ws, int M, int K,

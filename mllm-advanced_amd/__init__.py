@@ -18,6 +18,7 @@ BLOCK_LEN = 32
 GEMV_MAX_M = 8
 BF16_TRUNC = 0
 BF16_RNE = 1
+KERNEL_AUTO, KERNEL_GEMV, KERNEL_GEMM_I8, KERNEL_GEMM_F16 = 0, 1, 2, 3
 
 #: every symbol include/w4a32_hip.h declares, with (restype, argtypes)
 _vp, _ci, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
@@ -36,6 +37,7 @@ ABI = {
     "w4a32_quant_lhs": (_ci, [_vp, _ci, _ci, _ci, _vp, _vp]),
     "w4a32_export_lhs": (_ci, [_vp, _ci, _ci, _vp, _vp, _vp, _vp]),
     "w4a32_matmul_quantized": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp]),
+    "w4a32_matmul_quantized_ex": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp]),
     "w4a32_matmul": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
 }
 
@@ -169,12 +171,12 @@ def export_lhs(ws, M, K):
     return aq, recip, neg_zp
 
 
-def matmul_quantized(ws, packed, M, K, N, out=None):
+def matmul_quantized(ws, packed, M, K, N, out=None, kernel=KERNEL_AUTO):
     import torch
 
     y = out if out is not None else torch.empty((M, N), dtype=torch.float32, device="cuda")
-    _check(lib().w4a32_matmul_quantized(_ptr(y), _ptr(ws), _ptr(packed), M, K, N, _stream()),
-           "w4a32_matmul_quantized")
+    _check(lib().w4a32_matmul_quantized_ex(_ptr(y), _ptr(ws), _ptr(packed), M, K, N, kernel,
+                                           _stream()), "w4a32_matmul_quantized_ex")
     return y
 
 

@@ -124,8 +124,8 @@ int w4a32_export_lhs(const void* d_ws, int M, int K, int8_t* d_aq, float* d_reci
   return from_hip(e);
 }
 
-int w4a32_matmul_quantized(float* d_y, const void* d_ws, const void* d_packed, int M, int K, int N,
-                           void* stream) {
+int w4a32_matmul_quantized_ex(float* d_y, const void* d_ws, const void* d_packed, int M, int K,
+                              int N, int kernel, void* stream) {
   if (M <= 0) return W4A32_EINVAL;
   if (int e = shape_ok(N, K)) return e;
   if (!d_y || !d_ws || !d_packed) return W4A32_EINVAL;
@@ -133,8 +133,26 @@ int w4a32_matmul_quantized(float* d_y, const void* d_ws, const void* d_packed, i
   hipStream_t s = static_cast<hipStream_t>(stream);
   const uint8_t* ws = static_cast<const uint8_t*>(d_ws);
   const uint8_t* pk = static_cast<const uint8_t*>(d_packed);
-  if (M <= w4::kGemvMaxM) return from_hip(w4::launch_gemv(d_y, ws, pk, M, K, N, s));
-  return from_hip(w4::launch_gemm(d_y, ws, pk, M, K, N, s));
+  switch (kernel) {
+    case W4A32_KERNEL_AUTO:
+      if (M <= w4::kGemvMaxM) return from_hip(w4::launch_gemv(d_y, ws, pk, M, K, N, s));
+      return from_hip(w4::launch_gemm(d_y, ws, pk, M, K, N, w4::kKernelAuto, s));
+    case W4A32_KERNEL_GEMV:
+      if (M > w4::kGemvMaxM) return W4A32_ESHAPE;
+      return from_hip(w4::launch_gemv(d_y, ws, pk, M, K, N, s));
+    case W4A32_KERNEL_GEMM_I8:
+      return from_hip(w4::launch_gemm(d_y, ws, pk, M, K, N, w4::kKernelGemmI8, s));
+    case W4A32_KERNEL_GEMM_F16:
+      if (M <= w4::kGemvMaxM) return W4A32_ESHAPE;  // the f16 activation copy exists only for M > 8
+      return from_hip(w4::launch_gemm(d_y, ws, pk, M, K, N, w4::kKernelGemmF16, s));
+    default:
+      return W4A32_EINVAL;
+  }
+}
+
+int w4a32_matmul_quantized(float* d_y, const void* d_ws, const void* d_packed, int M, int K, int N,
+                           void* stream) {
+  return w4a32_matmul_quantized_ex(d_y, d_ws, d_packed, M, K, N, W4A32_KERNEL_AUTO, stream);
 }
 
 int w4a32_matmul(float* d_y, const float* d_x, const void* d_packed, void* d_ws, int M, int K,

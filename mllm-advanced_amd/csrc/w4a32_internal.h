@@ -24,7 +24,13 @@ hipError_t launch_quant_lhs(const float* x, int M, int K, int ldx, uint8_t* ws, 
 hipError_t launch_gemv(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                        hipStream_t s);
 hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
-                       hipStream_t s);
+                       int kernel, hipStream_t s);
+
+// kernel selectors of w4a32_matmul_quantized_ex (0 = the library's own choice)
+constexpr int kKernelAuto = 0;
+constexpr int kKernelGemv = 1;
+constexpr int kKernelGemmI8 = 2;
+constexpr int kKernelGemmF16 = 3;
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
 

@@ -22,6 +22,12 @@
 //          in block order. Lets the int8 kernels add the activation offset once per output:
 //          sum_k (a_q + off) q s = sum_k a_q q s + off * rsum.
 //   bias:  f32 [Np] after rsum (zeros when the layer has none).
+//   rowmul: f32 [Np] after bias: 2^E_n, where E_n puts the row's largest |scale| in [2^11, 2^12).
+//   hscale: per tile 64 x f16 (128 B, same order as the bf16 scales in the tile) after rowmul:
+//          scale * 2^-E_n. A bf16 scale has 8 significant bits, so this is exact whenever it is
+//          a normal f16, i.e. for every block whose scale is within 2^-25 of the row's largest;
+//          then q * hscale (4 + 8 bits) is exact in f16 too. The f16 MFMA prefill kernel uses
+//          this plane and multiplies its f32 accumulators by rowmul.
 //
 // ACTIVATION WORKSPACE for M rows (Mp = M rounded up to 16):
 //
@@ -29,7 +35,9 @@
 //   [4*Mp, 8*Mp)         i32  neg_zp[m]        (the "lhs offset" = -zero_point)
 //   hdr = round_up(8*Mp, 256)
 //   [hdr, hdr + Mp*K)    i8   a_q[m][k] row-major
-//   then, 256-aligned    f16  a_h[m][k] = (a_q + neg_zp) exactly, only written when M > 8
+//   then, 256-aligned    f16  a_h = (a_q + neg_zp) exactly (|.| <= 255), only written when M > 8;
+//                        inside each aligned group of 8 k the order is k0,k2,k4,k6,k1,k3,k5,k7,
+//                        the order in which a tile dword unpacks to f16 pairs (see kHalfOrder)
 #pragma once
 
 #include <stddef.h>
@@ -56,7 +64,7 @@ W4_HD size_t round_up_sz(size_t v, size_t m) { return (v + m - 1) / m * m; }
 
 struct WeightGeom {
   int N, K, Np, Kp, NT, KC;
-  size_t tiles_bytes, rsum_off, bias_off, total_bytes;
+  size_t tiles_bytes, rsum_off, bias_off, rowmul_off, hscale_off, total_bytes;
 };
 
 W4_HD WeightGeom weight_geom(int N, int K) {
@@ -70,7 +78,9 @@ W4_HD WeightGeom weight_geom(int N, int K) {
   g.tiles_bytes = (size_t)g.NT * g.KC * kTileBytes;
   g.rsum_off = g.tiles_bytes;
   g.bias_off = g.rsum_off + (size_t)g.Np * 4;
-  g.total_bytes = g.bias_off + (size_t)g.Np * 4;
+  g.rowmul_off = g.bias_off + (size_t)g.Np * 4;
+  g.hscale_off = g.rowmul_off + (size_t)g.Np * 4;
+  g.total_bytes = g.hscale_off + (size_t)g.NT * g.KC * kTileScaleBytes;
   return g;
 }
 
@@ -94,5 +104,10 @@ W4_HD WsGeom ws_geom(int M, int K) {
 
 // Nibble position (0..7) inside a tile dword of the weight at k offset e (0..7) in its 8-group.
 W4_HD int nibble_pos(int e) { return e < 4 ? 2 * e : 2 * (e - 4) + 1; }
+
+// Masking a tile dword with 0x000F000F after shifting right by 0, 4, 8, 12 bits yields the
+// nibble pairs (0,4), (1,5), (2,6), (3,7) = k offsets (0,2), (4,6), (1,3), (5,7).
+// kHalfOrder[i] is the k offset stored at position i of an 8-group of a_h.
+constexpr int kHalfOrder[8] = {0, 2, 4, 6, 1, 3, 5, 7};
 
 }  // namespace w4

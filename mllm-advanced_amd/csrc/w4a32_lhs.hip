@@ -72,27 +72,31 @@ __global__ __launch_bounds__(kLhsThreads) void quant_lhs_kernel(
   }
 
   int8_t* dst = aq + (size_t)m * K;
-  for (int i = 4 * t; i < K; i += 4 * kLhsThreads) {
-    const float4 v = *reinterpret_cast<const float4*>(row + i);
-    const float f[4] = {v.x, v.y, v.z, v.w};
-    int q[4];
+  for (int i = 8 * t; i < K; i += 8 * kLhsThreads) {  // K % 32 == 0: whole groups of 8
+    const float4 v0 = *reinterpret_cast<const float4*>(row + i);
+    const float4 v1 = *reinterpret_cast<const float4*>(row + i + 4);
+    const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+    int q[8];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
+    for (int e = 0; e < 8; ++e) {
       int r = (int)roundf(__fmul_rn(f[e], scale)) + zp;  // |x*scale| <= 255: the cast is safe
       r = r < -128 ? -128 : r;
       r = r > 127 ? 127 : r;
       q[e] = r;
     }
-    const uint32_t packed = (uint32_t)(q[0] & 0xFF) | ((uint32_t)(q[1] & 0xFF) << 8) |
-                            ((uint32_t)(q[2] & 0xFF) << 16) | ((uint32_t)(q[3] & 0xFF) << 24);
-    *reinterpret_cast<uint32_t*>(dst + i) = packed;
+    uint2 packed;
+    packed.x = (uint32_t)(q[0] & 0xFF) | ((uint32_t)(q[1] & 0xFF) << 8) |
+               ((uint32_t)(q[2] & 0xFF) << 16) | ((uint32_t)(q[3] & 0xFF) << 24);
+    packed.y = (uint32_t)(q[4] & 0xFF) | ((uint32_t)(q[5] & 0xFF) << 8) |
+               ((uint32_t)(q[6] & 0xFF) << 16) | ((uint32_t)(q[7] & 0xFF) << 24);
+    *reinterpret_cast<uint2*>(dst + i) = packed;
     if (ah) {
-      // a_q - zp lies in [-255, 255]: exact in f16
-      typedef _Float16 h4 __attribute__((ext_vector_type(4)));
-      h4 hv;
+      // a_q - zp lies in [-255, 255]: exact in f16. Stored in the order a weight dword unpacks.
+      typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+      h8 hv;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) hv[e] = (_Float16)(float)(q[e] - zp);
-      *reinterpret_cast<h4*>(ah + (size_t)m * K + i) = hv;
+      for (int e = 0; e < 8; ++e) hv[e] = (_Float16)(float)(q[kHalfOrder[e]] - zp);
+      *reinterpret_cast<h8*>(ah + (size_t)m * K + i) = hv;
     }
   }
 }

@@ -117,15 +117,27 @@ __global__ __launch_bounds__(64) void repack_kernel(const uint8_t* __restrict__ 
   *reinterpret_cast<uint16_t*>(base + kTileQBytes + 2 * l) = s;
 }
 
-// Per-row sum_b f32(scale_b) * (float)(sum_{k in b} q) in block order, and the bias plane.
+// E_n such that (largest |scale| of the row) * 2^-E_n lies in [2^11, 2^12); 0 for an all-zero row.
+// mag = bf16 bits of that scale without the sign. bf16 subnormals count as exponent -126.
+__device__ __forceinline__ int row_exponent(uint32_t mag) {
+  if (mag == 0) return 0;
+  int e = (int)(mag >> 7) - 127;
+  if ((mag >> 7) == 0) e = -126;
+  return e - 11;
+}
+
+// Per-row sum_b f32(scale_b) * (float)(sum_{k in b} q) in block order, the bias plane, and the
+// power of two that normalises the row's scales for the f16 copy.
 __global__ __launch_bounds__(256) void rsum_bias_kernel(const uint8_t* __restrict__ u4,
                                                         const uint16_t* __restrict__ scales,
                                                         const float* __restrict__ bias, int N,
                                                         int K, int Np, float* __restrict__ rsum,
-                                                        float* __restrict__ bias_out) {
+                                                        float* __restrict__ bias_out,
+                                                        float* __restrict__ rowmul) {
   const int n = blockIdx.x * blockDim.x + threadIdx.x;
   if (n >= Np) return;
   float r = 0.0f, bv = 0.0f;
+  uint32_t max_mag = 0;  // largest |scale| of the row, as bf16 bits without the sign
   if (n < N) {
     const int nb = K / kBlockLen;
     const uint4* row = reinterpret_cast<const uint4*>(u4 + (size_t)n * (K / 2));
@@ -141,12 +153,34 @@ __global__ __launch_bounds__(256) void rsum_bias_kernel(const uint8_t* __restric
         s += (int)((t & 0xFFFFu) + (t >> 16));
       }
       s -= 8 * kBlockLen;
-      r = __fadd_rn(r, __fmul_rn((float)s, bf16_bits_to_f32(scales[(size_t)n * nb + b])));
+      const uint32_t sbits = scales[(size_t)n * nb + b];
+      r = __fadd_rn(r, __fmul_rn((float)s, bf16_bits_to_f32(sbits)));
+      const uint32_t mag = sbits & 0x7FFFu;
+      if (mag < 0x7F80u && mag > max_mag) max_mag = mag;  // ignore inf/nan scales
     }
     if (bias) bv = bias[n];
   }
   rsum[n] = r;
   bias_out[n] = bv;
+  rowmul[n] = ldexpf(1.0f, row_exponent(max_mag));
+}
+
+// f16 copy of the block scales, each row divided by its rowmul (a power of two).
+__global__ __launch_bounds__(64) void hscale_kernel(const uint16_t* __restrict__ scales, int N,
+                                                    int K, int KC, const float* __restrict__ rowmul,
+                                                    _Float16* __restrict__ hscale) {
+  const int tile = blockIdx.x;
+  const int nt = tile / KC, kc = tile % KC;
+  const int l = threadIdx.x;
+  const int nb = K / kBlockLen;
+  const int sn = kTileRows * nt + (l >> 2), sb = 4 * kc + (l & 3);
+  float v = 0.0f;
+  if (sn < N && sb < nb) {
+    int e;
+    (void)frexpf(rowmul[sn], &e);  // rowmul = 2^(e-1)
+    v = ldexpf(bf16_bits_to_f32(scales[(size_t)sn * nb + sb]), -(e - 1));
+  }
+  hscale[(size_t)tile * 64 + l] = (_Float16)v;
 }
 
 __global__ __launch_bounds__(64) void unpack_kernel(const uint8_t* __restrict__ packed, int N,
@@ -229,7 +263,13 @@ hipError_t launch_repack(const uint8_t* u4, const uint16_t* scales, const float*
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(rsum_bias_kernel, dim3((g.Np + 255) / 256), dim3(256), 0, s, u4, scales, bias,
                      N, K, g.Np, reinterpret_cast<float*>(packed + g.rsum_off),
-                     reinterpret_cast<float*>(packed + g.bias_off));
+                     reinterpret_cast<float*>(packed + g.bias_off),
+                     reinterpret_cast<float*>(packed + g.rowmul_off));
+  e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(hscale_kernel, dim3(g.NT * g.KC), dim3(64), 0, s, scales, N, K, g.KC,
+                     reinterpret_cast<const float*>(packed + g.rowmul_off),
+                     reinterpret_cast<_Float16*>(packed + g.hscale_off));
   return hipGetLastError();
 }
 

@@ -33,9 +33,11 @@ def test_library_exports_every_declared_symbol(pkg):
 
 def test_size_functions(pkg):
     L = pkg.lib()
-    # tiles of 16 rows x 128 k = 1024 B nibbles + 128 B scales, then rsum and bias planes
-    assert L.w4a32_packed_bytes(8960, 1536) == (8960 // 16) * (1536 // 128) * 1152 + 2 * 8960 * 4
-    assert L.w4a32_packed_bytes(50, 96) == 4 * 1 * 1152 + 2 * 64 * 4       # padded to 64 x 128
+    # tiles of 16 rows x 128 k = 1024 B nibbles + 128 B scales; then the rsum, bias and rowmul
+    # planes (f32 per row) and the f16 copy of the scales (128 B per tile)
+    tiles = (8960 // 16) * (1536 // 128)
+    assert L.w4a32_packed_bytes(8960, 1536) == tiles * 1152 + 3 * 8960 * 4 + tiles * 128
+    assert L.w4a32_packed_bytes(50, 96) == 4 * 1152 + 3 * 64 * 4 + 4 * 128   # padded to 64 x 128
     assert L.w4a32_packed_bytes(16, 48) == 0 and L.w4a32_packed_bytes(0, 32) == 0
     assert L.w4a32_native_u4_bytes(256, 1536) == 256 * 768
     assert L.w4a32_native_scale_bytes(256, 1536) == 256 * 48 * 2
@@ -45,10 +47,11 @@ def test_size_functions(pkg):
 
 
 def test_nibbles_and_scales_are_the_algorithmic_bytes(pkg):
-    # the blob adds nothing to the format's own bytes when N % 16 == 0 and K % 128 == 0
+    # when N % 16 == 0 and K % 128 == 0 the tiles hold exactly the format's own bytes (what the
+    # decode kernels stream); the rest of the blob is three f32 planes and the f16 scale copy
     for n, k in [(1536, 1536), (256, 1536), (8960, 1536), (1536, 8960), (151936, 1536)]:
         fmt = n * k // 2 + n * (k // 32) * 2
-        assert pkg.packed_bytes(n, k) == fmt + 2 * 4 * n
+        assert pkg.packed_bytes(n, k) == fmt + 3 * 4 * n + n * (k // 32) * 2
 
 
 def test_fixture_matches_oracle(orc):

@@ -232,10 +232,50 @@ def test_gemm_large_m_on_sampled_rows(pkg, orc, name, k, n, has_bias):
     assert err <= GEMM_TOL and err <= TIGHT, (name, err)
 
 
-@pytest.mark.parametrize("m", [9, 15, 16, 17, 63, 65, 100])
+@pytest.mark.parametrize("m", [9, 15, 16, 17, 32, 33, 63, 65, 100, 129, 257, 300])
 def test_gemm_ragged_m(pkg, orc, m):
     y, ref = run_linear(pkg, orc, m, 256, 50, True, outliers=0.1)
     assert max_abs_rel(y, ref) <= TIGHT
+
+
+@pytest.mark.parametrize("kernel", ["i8", "f16"])
+@pytest.mark.parametrize("m,k,n", [(9, 32, 16), (40, 96, 50), (128, 1536, 256), (300, 1280, 3840),
+                                   (512, 8960, 1536), (1024, 5120, 1280)])
+def test_gemm_each_kernel_matches_oracle(pkg, orc, kernel, m, k, n):
+    # both prefill kernels on the same inputs; K = 32 and 96 leave padding inside a stage
+    w = make_weights(n, k, seed=k)
+    x = make_acts(m, k, seed=m, outlier_frac=0.02)
+    bias = bias_for(n, True)
+    u4, sc = orc.quant_rhs(w)
+    packed = pkg.repack_native(dev(u4), dev(sc.view(np.int16)), dev(bias), n, k)
+    ws = pkg.quant_lhs(dev(x))
+    sel = pkg.KERNEL_GEMM_I8 if kernel == "i8" else pkg.KERNEL_GEMM_F16
+    y = host(pkg.matmul_quantized(ws, packed, m, k, n, kernel=sel))
+    rows = np.unique(np.concatenate([np.arange(0, m, 41), [m - 1]]))
+    ref = orc.linear(x[rows], u4, sc, bias=bias, threads=8)
+    err = max_abs_rel(y[rows], ref)
+    assert err <= GEMM_TOL and err <= TIGHT, (kernel, err)
+
+
+def test_f16_kernel_with_wide_scale_range(pkg, orc):
+    # rows whose block scales differ by many octaves, and rows that are tiny or huge overall:
+    # the per-row power-of-two normalisation must keep the f16 operands exact
+    n, k, m = 64, 256, 48
+    rng = np.random.default_rng(8)
+    w = make_weights(n, k, seed=8)
+    for r in range(n):
+        w[r] *= np.float32(2.0) ** rng.integers(-30, 30)
+        for b in range(k // 32):
+            w[r, 32 * b:32 * b + 32] *= np.float32(2.0) ** rng.integers(-12, 1)
+    x = make_acts(m, k, seed=9)
+    u4, sc = orc.quant_rhs(w)
+    packed = pkg.repack_native(dev(u4), dev(sc.view(np.int16)), None, n, k)
+    ws = pkg.quant_lhs(dev(x))
+    y = host(pkg.matmul_quantized(ws, packed, m, k, n, kernel=pkg.KERNEL_GEMM_F16))
+    ref = orc.linear(x, u4, sc, threads=4)
+    # per output column (its own row of weights), relative to that column's largest output
+    col_err = np.abs(y - ref).max(axis=0) / np.abs(ref).max(axis=0)
+    assert col_err.max() <= TIGHT, col_err.max()
 
 
 def test_gemm_rows_agree_with_gemv(pkg):
@@ -284,5 +324,12 @@ def test_bad_arguments_return_error_codes(pkg):
     assert L.w4a32_quant_lhs(x.data_ptr(), 1, 48, 48, x.data_ptr(), None) == -2
     assert L.w4a32_quant_lhs(None, 1, 64, 64, x.data_ptr(), None) == -1
     assert L.w4a32_matmul_quantized(None, None, None, 1, 64, 16, None) == -1
+    ws = torch.zeros(pkg.workspace_bytes(4, 64), dtype=torch.uint8, device="cuda")
+    pk = torch.zeros(pkg.packed_bytes(16, 64), dtype=torch.uint8, device="cuda")
+    y = torch.zeros((16, 16), device="cuda")
+    args = (y.data_ptr(), ws.data_ptr(), pk.data_ptr())
+    assert L.w4a32_matmul_quantized_ex(*args, 4, 64, 16, pkg.KERNEL_GEMM_F16, None) == -2
+    assert L.w4a32_matmul_quantized_ex(*args, 16, 64, 16, pkg.KERNEL_GEMV, None) == -2
+    assert L.w4a32_matmul_quantized_ex(*args, 4, 64, 16, 99, None) == -1
     with pytest.raises(pkg.W4A32Error):
         pkg._check(-2, "probe")
