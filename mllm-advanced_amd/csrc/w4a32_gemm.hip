@@ -2,7 +2,7 @@
 //
 // Two kernels:
 //
-//  * gemm_f16_kernel (M > 32): v_mfma_f32_16x16x32_f16 on EXACT f16 operands. The activation
+//  * gemm_f16_kernel (M > 32): v_mfma_f32_32x32x16_f16 on EXACT f16 operands. The activation
 //    operand is a_q - zp (an integer in [-255, 255]); the weight operand is q * scale / 2^E_n
 //    (4 + 8 significant bits), dequantised ONCE per workgroup from the 4-bit tiles into LDS,
 //    already in MFMA fragment order. Every product is exact in f32; only the order of the f32
@@ -108,169 +108,249 @@ typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 // 8 weights of one tile dword -> 8 f16 (q * s), in the order k0,k2,k4,k6,k1,k3,k5,k7.
-// 0x6400 | u4 is the f16 number 1024 + u4; subtracting 1032 leaves q exactly.
-__device__ __forceinline__ uint4 dequant8(uint32_t w, h2 s) {
+// 0x6400 | u4 is the f16 number 1024 + u4, and 0x6400 | (u4 << 4) is 1024 + 16*u4, so the
+// nibbles at bits 0-3 and 4-7 of each half-word need no shift: subtract 1032 (resp. 1152) to
+// get q (resp. 16*q) exactly, then multiply by s (resp. s/16). `s` holds {s, s} and `s16`
+// holds {s/16, s/16}; s/16 is exact unless s is already a subnormal f16.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t m, uint32_t o) {
+  return (a & m) | o;  // one v_and_or_b32
+}
+__device__ __forceinline__ uint4 dequant8(uint32_t w, h2 s, h2 s16) {
   const uint32_t x = w ^ 0x88888888u;  // two's complement nibbles -> offset-8 nibbles
-  uint32_t p[4];
-  p[0] = (x & 0x000F000Fu) | 0x64006400u;
-  p[1] = ((x >> 4) & 0x000F000Fu) | 0x64006400u;
-  p[2] = ((x >> 8) & 0x000F000Fu) | 0x64006400u;
-  p[3] = ((x >> 12) & 0x000F000Fu) | 0x64006400u;
-  const h2 bias = {(_Float16)1032.0f, (_Float16)1032.0f};
-  uint32_t o[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    h2 v = __builtin_bit_cast(h2, p[i]);
-    v = (v - bias) * s;
-    o[i] = __builtin_bit_cast(uint32_t, v);
-  }
-  return make_uint4(o[0], o[1], o[2], o[3]);
+  const uint32_t xh = x >> 8;
+  const h2 b1 = {(_Float16)1032.0f, (_Float16)1032.0f};
+  const h2 b16 = {(_Float16)1152.0f, (_Float16)1152.0f};
+  const h2 p0 = __builtin_bit_cast(h2, and_or(x, 0x000F000Fu, 0x64006400u));   // nibbles 0,4
+  const h2 p1 = __builtin_bit_cast(h2, and_or(x, 0x00F000F0u, 0x64006400u));   // nibbles 1,5
+  const h2 p2 = __builtin_bit_cast(h2, and_or(xh, 0x000F000Fu, 0x64006400u));  // nibbles 2,6
+  const h2 p3 = __builtin_bit_cast(h2, and_or(xh, 0x00F000F0u, 0x64006400u));  // nibbles 3,7
+  const h2 o0 = (p0 - b1) * s;
+  const h2 o1 = (p1 - b16) * s16;
+  const h2 o2 = (p2 - b1) * s;
+  const h2 o3 = (p3 - b16) * s16;
+  return make_uint4(__builtin_bit_cast(uint32_t, o0), __builtin_bit_cast(uint32_t, o1),
+                    __builtin_bit_cast(uint32_t, o2), __builtin_bit_cast(uint32_t, o3));
 }
 
-constexpr int kF16BK = 64;  // k per LDS stage (two scale blocks, half of a weight tile chunk)
+constexpr int kF16BK = 64;    // k per stage (two scale blocks, half of a weight tile chunk)
+constexpr int kF16Depth = 2;  // stages in flight between a global load and its use
 
-// Workgroup = 4 wavefronts arranged 2 (M) x 2 (N) over a BM x BN output tile.
-// LDS holds one stage: A as [2 k-blocks][BM/16 fragments][16 rows][32 k] f16 and B likewise;
-// a fragment is 1 KiB contiguous, and lane (g, j) reads its 16 bytes at j*64 + g*16.
-// The next stage travels global -> registers while the current one is multiplied.
-template <int BM, int BN>
-__global__ __launch_bounds__(256, 2) void gemm_f16_kernel(
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// v_mfma_f32_32x32x16_f16 (measured on MI355X: 2.1-2.2 PFLOP/s, twice the 16x16x32 shape).
+// Operands: lane l = 32*h + i holds 8 f16 of row/column i at "k-slot" h. Which k values a slot
+// stands for is free as long as A and B agree; here, inside a 32-k scale block, slice 0 is
+// k {0..7 | 16..23} for h = {0 | 1} and slice 1 is k {8..15 | 24..31}, so that one lane's two A
+// operands of a block are 32 contiguous bytes of its activation row.
+//
+// Workgroup = 4 wavefronts stacked along M; wavefront w owns rows [32*WM*w, 32*WM*(w+1)) of
+// the BM x BN tile (BM = 128*WM, BN = 32*WN) and all BN columns.
+//
+//  * A (f16 activations) never touches LDS: the row quantiser already wrote it as 2 KiB chunks
+//    of 32 rows x 32 k, so the two operand loads of a block read one contiguous chunk (instead
+//    of 32 rows that lie K*2 bytes apart), into a register ring kF16Depth stages deep (a load
+//    has that many stages of MFMA work to land).
+//  * B (4-bit weights) is shared by the four wavefronts: its packed bytes are prefetched into
+//    a small register ring, dequantised once per workgroup to f16 and double-buffered in LDS
+//    as 1 KiB fragments in lane order (lane l at l*16: conflict-free 128-bit accesses).
+//  * One barrier per stage: it publishes the B buffer written during the previous stage and
+//    frees the one read during it.
+template <int WAVES_M, int WAVES_N, int WM, int WN>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_f16_kernel(
     float* __restrict__ y, const _Float16* __restrict__ ah, const float* __restrict__ recip,
     const uint8_t* __restrict__ packed, const uint8_t* __restrict__ hscale,
     const float* __restrict__ rowmul, const float* __restrict__ bias, int M, int N, int K, int NT,
     int KC) {
-  constexpr int MT = BM / 16, NTW = BN / 16;
-  constexpr int WMT = MT / 2, WNT = NTW / 2;
-  constexpr int A_UNITS = BM * 8 / 256;    // 16-byte pieces of A per thread per stage
-  constexpr int B_UNITS = NTW * 64 / 256;  // 8-byte pieces of packed B per thread per stage
-  static_assert(B_UNITS >= 1, "BN too small");
+  constexpr int D = kF16Depth;
+  constexpr int NWAVES = WAVES_M * WAVES_N;
+  constexpr int BM = 32 * WM * WAVES_M;
+  constexpr int BN32 = WN * WAVES_N;           // 32-column fragments per workgroup and k-slice
+  constexpr int WNT = 2 * BN32;                // 16-row weight tile rows per workgroup
+  static_assert(WNT % NWAVES == 0, "each wavefront dequantises WNT/NWAVES tile rows per stage");
+  constexpr int B_UNITS = WNT / NWAVES;        // 8-byte pieces of packed B per thread per stage
+  constexpr int kBufBytes = 4 * BN32 * 1024;   // one B stage: [4 k-slices][BN32 fragments]
 
-  __shared__ __align__(16) uint8_t lds[(BM + BN) * kF16BK * 2];
-  uint8_t* sA = lds;
-  uint8_t* sB = lds + BM * kF16BK * 2;
+  __shared__ __align__(16) uint8_t sB[2 * kBufBytes];
 
   const int t = threadIdx.x;
   const int wave = t >> 6, lane = t & 63;
-  const int g = lane >> 4, j = lane & 15;
-  const int wm = wave >> 1, wn = wave & 1;
-  const int m0 = blockIdx.y * BM;
-  const int nt0 = blockIdx.x * NTW;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int g = lane >> 4, j = lane & 15;     // position inside a weight tile
+  const int h = lane >> 5, i32 = lane & 31;   // position inside an MFMA operand / C tile
+  const int m0 = blockIdx.y * BM + 32 * WM * wm;
+  const int nt0 = blockIdx.x * WNT;
+  const int nstages = (K + kF16BK - 1) / kF16BK;
 
-  uint4 ra[A_UNITS];
-  uint2 rb[B_UNITS];
-  uint32_t rs[B_UNITS];
+  uint4 areg[D][2][WM][2];  // [ring slot][k-block][32-row tile][slice of the block]
+  uint2 breg[D][B_UNITS];
+  uint32_t sreg[D][B_UNITS];
 
-  auto load_stage = [&](int s) {
-    const int k0 = s * kF16BK;
+  // Per-lane base pointers; everything that changes from stage to stage is a wavefront-uniform
+  // offset (scalar registers), so issuing a load costs no vector address arithmetic.
+  const int KB = K >> 5;  // 32-k blocks per row
+  const uint8_t* a_ptr[WM];
 #pragma unroll
-    for (int u = 0; u < A_UNITS; ++u) {
-      const int unit = t + 256 * u;
-      const int row = unit >> 3, kseg = unit & 7;
-      int gr = m0 + row;
-      gr = gr < M ? gr : M - 1;  // rows past M repeat the last row; their outputs are not stored
-      const int kk = k0 + 8 * kseg;
-      ra[u] = make_uint4(0, 0, 0, 0);
-      if (kk < K) ra[u] = *reinterpret_cast<const uint4*>(ah + (size_t)gr * K + kk);
-    }
-    const int kc = s >> 1, half = s & 1;
+  for (int a = 0; a < WM; ++a) {
+    int mt = (m0 >> 5) + a;
+    const int mt_last = (M - 1) >> 5;
+    mt = mt < mt_last ? mt : mt_last;  // tiles past M repeat the last one; never stored
+    a_ptr[a] = reinterpret_cast<const uint8_t*>(ah) + (size_t)mt * KB * 2048 + 64 * i32 + 32 * h;
+  }
+  const uint8_t* bq_ptr[B_UNITS];
+  const uint8_t* bs_ptr[B_UNITS];
 #pragma unroll
-    for (int u = 0; u < B_UNITS; ++u) {
-      const int unit = t + 256 * u;
-      const int ntl = unit >> 6, ln = unit & 63;
-      const int nt = nt0 + ntl;
-      rb[u] = make_uint2(0, 0);
-      rs[u] = 0;
-      if (nt < NT) {
-        const size_t tile = (size_t)nt * KC + kc;
-        rb[u] = *reinterpret_cast<const uint2*>(packed + tile * kTileBytes + 16 * ln + 8 * half);
-        rs[u] = *reinterpret_cast<const uint32_t*>(hscale + tile * kTileScaleBytes + 8 * (ln & 15) +
-                                                   4 * half);
+  for (int u = 0; u < B_UNITS; ++u) {
+    int nt = nt0 + wave + NWAVES * u;
+    nt = nt < NT ? nt : NT - 1;  // tile rows past the matrix: their columns are never stored
+    bq_ptr[u] = packed + (size_t)nt * KC * kTileBytes + 16 * lane;
+    bs_ptr[u] = hscale + (size_t)nt * KC * kTileScaleBytes + 8 * j;
+  }
+
+  // The steady-state loop must stay ONE basic block (the compiler can then wait for exactly
+  // the load it needs instead of draining all of them), so nothing below branches: stage
+  // numbers and k-blocks are clamped to valid addresses, and what must not contribute is
+  // multiplied by a zero scale (padded stages) or meets the zero nibbles and zero scales that
+  // pad every weight tile (k >= K).
+  auto load_a = [&](int s, uint4 (&dst)[2][WM][2]) {
+    const int sc = s < nstages ? s : nstages - 1;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      int blk = 2 * sc + kb;
+      blk = blk < KB ? blk : KB - 1;
+      const int off = blk * 2048;
+#pragma unroll
+      for (int a = 0; a < WM; ++a) {
+        dst[kb][a][0] = *reinterpret_cast<const uint4*>(a_ptr[a] + off);
+        dst[kb][a][1] = *reinterpret_cast<const uint4*>(a_ptr[a] + off + 16);
       }
     }
   };
 
-  auto store_stage = [&]() {
-#pragma unroll
-    for (int u = 0; u < A_UNITS; ++u) {
-      const int unit = t + 256 * u;
-      const int row = unit >> 3, kseg = unit & 7;
-      const int kb = kseg >> 2, gg = kseg & 3;
-      const int off = (((kb * MT + (row >> 4)) * 16 + (row & 15)) * 64) + gg * 16;
-      *reinterpret_cast<uint4*>(sA + off) = ra[u];
-    }
+  auto load_b = [&](int s, uint2 (&q)[B_UNITS], uint32_t (&sc)[B_UNITS]) {
+    const int st = s < nstages ? s : nstages - 1;
+    const int kc = st >> 1, half = st & 1;
+    const int offq = kc * kTileBytes + 8 * half;
+    const int offs = kc * kTileScaleBytes + 4 * half;
 #pragma unroll
     for (int u = 0; u < B_UNITS; ++u) {
-      const int unit = t + 256 * u;
-      const int ntl = unit >> 6, ln = unit & 63;
-      const int lane_off = (ln & 15) * 64 + (ln >> 4) * 16;
-      const h2 s2 = __builtin_bit_cast(h2, rs[u]);
-      const h2 s_lo = {s2[0], s2[0]};
-      const h2 s_hi = {s2[1], s2[1]};
-      *reinterpret_cast<uint4*>(sB + (0 * NTW + ntl) * 1024 + lane_off) = dequant8(rb[u].x, s_lo);
-      *reinterpret_cast<uint4*>(sB + (1 * NTW + ntl) * 1024 + lane_off) = dequant8(rb[u].y, s_hi);
+      q[u] = *reinterpret_cast<const uint2*>(bq_ptr[u] + offq);
+      sc[u] = *reinterpret_cast<const uint32_t*>(bs_ptr[u] + offs);
     }
   };
 
-  v4f acc[WMT][WNT];
+  // Tile lane (g, j) of tile row ntl, block dd -> fragment (slice 2*dd + (g & 1), column tile
+  // ntl / 2), operand lane 32*(g >> 1) + 16*(ntl & 1) + j.
+  // `s` is the stage the registers hold; a stage past the end (loaded from clamped addresses)
+  // gets scale 0. The mask is applied here, at use, so that the load itself has no consumer
+  // until D stages later.
+  auto store_b = [&](int s, int buf, const uint2 (&q)[B_UNITS], const uint32_t (&sc)[B_UNITS]) {
+    const uint32_t keep = s < nstages ? 0xFFFFFFFFu : 0u;
+    const h2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
 #pragma unroll
-  for (int a = 0; a < WMT; ++a)
-#pragma unroll
-    for (int b = 0; b < WNT; ++b) acc[a][b] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int u = 0; u < B_UNITS; ++u) {
+      const int ntl = wave + NWAVES * u;
+      const h2 s2 = __builtin_bit_cast(h2, sc[u] & keep);
+      const h2 s2_16 = s2 * sixteenth;
+      const h2 s_lo = {s2[0], s2[0]}, s_lo16 = {s2_16[0], s2_16[0]};
+      const h2 s_hi = {s2[1], s2[1]}, s_hi16 = {s2_16[1], s2_16[1]};
+      const int op_lane = 32 * (g >> 1) + 16 * (ntl & 1) + j;
+      uint8_t* base = sB + buf * kBufBytes + ((g & 1) * BN32 + (ntl >> 1)) * 1024 + 16 * op_lane;
+      *reinterpret_cast<uint4*>(base) = dequant8(q[u].x, s_lo, s_lo16);                    // block 0
+      *reinterpret_cast<uint4*>(base + 2 * BN32 * 1024) = dequant8(q[u].y, s_hi, s_hi16);  // block 1
+    }
+  };
 
-  const int nstages = (K + kF16BK - 1) / kF16BK;
-  const int frag_off = j * 64 + g * 16;
-  load_stage(0);
-  for (int s = 0; s < nstages; ++s) {
-    __syncthreads();  // every wavefront has finished reading the previous stage
-    store_stage();
-    __syncthreads();
-    if (s + 1 < nstages) load_stage(s + 1);
+  v16f acc[WM][WN];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      h8 af[WMT], bf[WNT];
+  for (int a = 0; a < WM; ++a)
 #pragma unroll
-      for (int a = 0; a < WMT; ++a)
-        af[a] = *reinterpret_cast<const h8*>(sA + (kb * MT + wm * WMT + a) * 1024 + frag_off);
+    for (int b = 0; b < WN; ++b)
 #pragma unroll
-      for (int b = 0; b < WNT; ++b)
-        bf[b] = *reinterpret_cast<const h8*>(sB + (kb * NTW + wn * WNT + b) * 1024 + frag_off);
+      for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
+
+  // Prologue: A stages 0..D-1 and B stages 0..D in flight; B stage 0 goes to LDS buffer 0.
 #pragma unroll
-      for (int a = 0; a < WMT; ++a)
+  for (int p = 0; p < D; ++p) load_a(p, areg[p]);
+  {
+    uint2 q0[B_UNITS];
+    uint32_t s0[B_UNITS];
+    load_b(0, q0, s0);
 #pragma unroll
-        for (int b = 0; b < WNT; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[a], bf[b], acc[a][b], 0, 0, 0);
+    for (int p = 0; p < D; ++p) load_b(p + 1, breg[p], sreg[p]);  // ring slot p holds stage p+1
+    store_b(0, 0, q0, s0);
+  }
+
+  // Stages are processed D at a time (ring slot u and LDS buffer u & 1 are then compile-time
+  // constants); the stage count is rounded up to a multiple of D, extra stages multiply by 0.
+  for (int s_base = 0; s_base < nstages; s_base += D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      const int s = s_base + u;
+      __syncthreads();
+      // B of stage s+1 (ring slot u) -> the LDS buffer not being read; refill the slot
+      store_b(s + 1, (u + 1) & 1, breg[u], sreg[u]);
+      load_b(s + 1 + D, breg[u], sreg[u]);
+
+      // B fragments come from LDS one k-slice ahead of the MFMAs that use them.
+      const uint8_t* bbuf = sB + (u & 1) * kBufBytes + 16 * lane;
+      h8 bf[2][WN];
+#pragma unroll
+      for (int b = 0; b < WN; ++b)
+        bf[0][b] = *reinterpret_cast<const h8*>(bbuf + (wn * WN + b) * 1024);
+#pragma unroll
+      for (int sl = 0; sl < 4; ++sl) {
+        if (sl < 3) {
+#pragma unroll
+          for (int b = 0; b < WN; ++b)
+            bf[(sl + 1) & 1][b] =
+                *reinterpret_cast<const h8*>(bbuf + ((sl + 1) * BN32 + wn * WN + b) * 1024);
+        }
+#pragma unroll
+        for (int b = 0; b < WN; ++b) {
+#pragma unroll
+          for (int a = 0; a < WM; ++a) {
+            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                __builtin_bit_cast(h8, areg[u][sl >> 1][a][sl & 1]), bf[sl & 1][b], acc[a][b], 0, 0,
+                0);
+          }
+        }
+      }
+      load_a(s + D, areg[u]);
     }
   }
 
-  // C layout: lane (g, j) holds column j, rows 4*g + r of each 16x16 tile.
+  // C layout of a 32x32 tile: lane (h, i32) holds column i32; register v holds row
+  // 8*(v/4) + 4*h + v%4.
 #pragma unroll
-  for (int b = 0; b < WNT; ++b) {
-    const int n = 16 * (nt0 + wn * WNT + b) + j;
+  for (int b = 0; b < WN; ++b) {
+    const int n = 16 * nt0 + 32 * (wn * WN + b) + i32;
     if (n >= N) continue;
     const float rm = rowmul[n], bs = bias[n];
 #pragma unroll
-    for (int a = 0; a < WMT; ++a) {
+    for (int a = 0; a < WM; ++a) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int m = m0 + 16 * (wm * WMT + a) + 4 * g + r;
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + 32 * a + 8 * (v >> 2) + 4 * h + (v & 3);
         if (m < M) {
-          float v = acc[a][b][r] * rm;
-          v = __fmaf_rn(v, recip[m], bs);
-          v = fminf(fmaxf(v, -3.402823466e+38f), 3.402823466e+38f);
-          y[(size_t)m * N + n] = v;
+          float val = acc[a][b][v] * rm;
+          val = __fmaf_rn(val, recip[m], bs);
+          val = fminf(fmaxf(val, -3.402823466e+38f), 3.402823466e+38f);
+          y[(size_t)m * N + n] = val;
         }
       }
     }
   }
 }
 
-template <int BM, int BN>
+template <int WAVES_M, int WAVES_N, int WM, int WN>
 static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                              hipStream_t s) {
+  constexpr int BM = 32 * WM * WAVES_M, WNT = 2 * WN * WAVES_N;
   const WeightGeom g = weight_geom(N, K);
   const WsGeom w = ws_geom(M, K);
-  dim3 grid((g.NT + BN / 16 - 1) / (BN / 16), (M + BM - 1) / BM);
-  hipLaunchKernelGGL((gemm_f16_kernel<BM, BN>), grid, dim3(256), 0, s, y,
+  dim3 grid((g.NT + WNT - 1) / WNT, (M + BM - 1) / BM);
+  hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN>), grid,
+                     dim3(64 * WAVES_M * WAVES_N), 0, s, y,
                      reinterpret_cast<const _Float16*>(ws + w.ah_off),
                      reinterpret_cast<const float*>(ws + w.scale_off), packed,
                      packed + g.hscale_off, reinterpret_cast<const float*>(packed + g.rowmul_off),
@@ -293,27 +373,13 @@ static hipError_t launch_gemm_i8(float* y, const uint8_t* ws, const uint8_t* pac
   return hipGetLastError();
 }
 
-// Tile choice: the chip has 256 CUs with two workgroups resident each. Prefer the largest tile
-// that still yields enough workgroups; a tile with a larger wavefront tile reuses each LDS
-// fragment more often, so it is weighted up.
-static int pick_f16_tile(int M, int NT) {
-  struct Cand { int bm, bn; double w; };
-  const Cand cands[3] = {{256, 128, 1.0}, {128, 128, 0.8}, {128, 64, 0.6}};
-  const double slots = 512.0;
-  int best = 0;
-  double best_score = -1.0;
-  for (int i = 0; i < 3; ++i) {
-    const long tiles = (long)((M + cands[i].bm - 1) / cands[i].bm) *
-                       ((NT + cands[i].bn / 16 - 1) / (cands[i].bn / 16));
-    const double rounds = (double)((tiles + (long)slots - 1) / (long)slots);
-    const double useful = ((double)M * NT * 16) / ((double)tiles * cands[i].bm * cands[i].bn);
-    const double score = cands[i].w * useful * (double)tiles / (rounds * slots);
-    if (score > best_score) {
-      best_score = score;
-      best = i;
-    }
-  }
-  return best;
+// All f16 configurations use a 128 x 128 output tile (1 KiB weight fragments shared through
+// LDS by the whole workgroup). With many tiles, 4 wavefronts per workgroup and three workgroups
+// per CU did best on MI355X; with few tiles, 8 wavefronts per workgroup (smaller wavefront
+// tiles, more wavefronts per SIMD to hide each other's stalls) did.
+static bool many_tiles(int M, int NT) {
+  const long tiles = (long)((M + 127) / 128) * ((NT + 7) / 8);
+  return tiles >= 1024;
 }
 
 hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
@@ -322,11 +388,8 @@ hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M
     return launch_gemm_i8(y, ws, packed, M, K, N, s);
   }
   const WeightGeom g = weight_geom(N, K);
-  switch (pick_f16_tile(M, g.NT)) {
-    case 0: return launch_f16<256, 128>(y, ws, packed, M, K, N, s);
-    case 1: return launch_f16<128, 128>(y, ws, packed, M, K, N, s);
-    default: return launch_f16<128, 64>(y, ws, packed, M, K, N, s);
-  }
+  if (many_tiles(M, g.NT)) return launch_f16<4, 1, 1, 4>(y, ws, packed, M, K, N, s);
+  return launch_f16<4, 2, 1, 2>(y, ws, packed, M, K, N, s);
 }
 
 }  // namespace w4

@@ -29,15 +29,20 @@
 //          then q * hscale (4 + 8 bits) is exact in f16 too. The f16 MFMA prefill kernel uses
 //          this plane and multiplies its f32 accumulators by rowmul.
 //
-// ACTIVATION WORKSPACE for M rows (Mp = M rounded up to 16):
+// ACTIVATION WORKSPACE for M rows (Mp = M rounded up to 32):
 //
 //   [0, 4*Mp)            f32  recip_scale[m]   (the "lhs scale" applied to the output)
 //   [4*Mp, 8*Mp)         i32  neg_zp[m]        (the "lhs offset" = -zero_point)
 //   hdr = round_up(8*Mp, 256)
 //   [hdr, hdr + Mp*K)    i8   a_q[m][k] row-major
-//   then, 256-aligned    f16  a_h = (a_q + neg_zp) exactly (|.| <= 255), only written when M > 8;
-//                        inside each aligned group of 8 k the order is k0,k2,k4,k6,k1,k3,k5,k7,
-//                        the order in which a tile dword unpacks to f16 pairs (see kHalfOrder)
+//   then, 256-aligned    f16  a_h = (a_q + neg_zp) exactly (|.| <= 255), only written when M > 8,
+//                        stored as 2 KiB chunks so that the f16 MFMA kernel reads whole
+//                        chunks instead of 32 rows lying K*2 bytes apart:
+//                          chunk (mt, kb) = rows 32*mt..+31, k 32*kb..+31, at
+//                          (mt * K/32 + kb) * 2048, row-major inside: row i at i*64, its four
+//                          groups of 8 k at 16 bytes each; inside a group the order is
+//                          k0,k2,k4,k6,k1,k3,k5,k7 - the order in which a weight tile dword
+//                          unpacks to f16 pairs (see kHalfOrder).
 #pragma once
 
 #include <stddef.h>
@@ -93,7 +98,7 @@ W4_HD WsGeom ws_geom(int M, int K) {
   WsGeom g;
   g.M = M;
   g.K = K;
-  g.Mp = round_up(M, 16);
+  g.Mp = round_up(M, 32);
   g.scale_off = 0;
   g.off_off = (size_t)4 * g.Mp;
   g.aq_off = round_up_sz((size_t)8 * g.Mp, 256);

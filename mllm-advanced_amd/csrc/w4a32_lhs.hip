@@ -24,8 +24,8 @@ __device__ __forceinline__ float wave_max(float v) {
 constexpr int kLhsThreads = 256;
 
 // One workgroup per row. Pass 1 reads the row for min/max, pass 2 re-reads it (it is L2/L1
-// resident: at most 35 KB) and writes 4 int8 per thread per step, plus the f16 copy of
-// (a_q - zp) that the f16 MFMA prefill kernel consumes.
+// resident: at most 35 KB) and writes 8 int8 per thread per step, plus the f16 copy of
+// (a_q - zp), tiled in MFMA operand order, that the f16 MFMA prefill kernel consumes.
 __global__ __launch_bounds__(kLhsThreads) void quant_lhs_kernel(
     const float* __restrict__ x, int K, int ldx, float* __restrict__ recip_out,
     int32_t* __restrict__ negzp_out, int8_t* __restrict__ aq, _Float16* __restrict__ ah) {
@@ -96,7 +96,10 @@ __global__ __launch_bounds__(kLhsThreads) void quant_lhs_kernel(
       h8 hv;
 #pragma unroll
       for (int e = 0; e < 8; ++e) hv[e] = (_Float16)(float)(q[kHalfOrder[e]] - zp);
-      *reinterpret_cast<h8*>(ah + (size_t)m * K + i) = hv;
+      // chunk (m / 32, k-block) holds 32 rows x 32 k, 64 bytes per row (see w4a32_layout.h)
+      const int kb = i >> 5, grp = (i >> 3) & 3;
+      const size_t chunk = (size_t)(m >> 5) * (K >> 5) + kb;
+      *reinterpret_cast<h8*>(ah + chunk * 1024 + (m & 31) * 32 + grp * 8) = hv;
     }
   }
 }

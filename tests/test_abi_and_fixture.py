@@ -41,7 +41,7 @@ def test_size_functions(pkg):
     assert L.w4a32_packed_bytes(16, 48) == 0 and L.w4a32_packed_bytes(0, 32) == 0
     assert L.w4a32_native_u4_bytes(256, 1536) == 256 * 768
     assert L.w4a32_native_scale_bytes(256, 1536) == 256 * 48 * 2
-    assert L.w4a32_workspace_bytes(1, 1536) == 256 + 16 * 1536            # header + 16 padded rows
+    assert L.w4a32_workspace_bytes(1, 1536) == 256 + 32 * 1536            # header + 32 padded rows
     assert L.w4a32_workspace_bytes(512, 1536) == 4096 + 512 * 1536 * 3    # + the f16 copy
     assert L.w4a32_workspace_bytes(1, 100) == 0
 
