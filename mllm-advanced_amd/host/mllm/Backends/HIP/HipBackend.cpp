@@ -1,0 +1,124 @@
+#include "mllm/Backends/HIP/HipBackend.hpp"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdlib>
+#include <cstring>
+
+#include "mllm/Backends/HIP/Ops/LinearOp.hpp"
+#include "mllm/Engine/Context.hpp"
+#include "mllm/Utils/Log.hpp"
+
+#define MLLM_CHECK_HIP(expr)                                                                    \
+  do {                                                                                          \
+    hipError_t e_ = (expr);                                                                     \
+    if (e_ != hipSuccess)                                                                       \
+      MLLM_ERROR_EXIT(::mllm::kHipError, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), \
+                      __FILE__, __LINE__);                                                      \
+  } while (0)
+
+namespace mllm::hip {
+
+namespace {
+size_t roundUp(size_t v, size_t a) { return (v + a - 1) / a * a; }
+}  // namespace
+
+bool HipAllocator::alloc(const std::shared_ptr<Storage>& storage) {
+  void* p = nullptr;
+  if (!generalAlloc(&p, storage->size_, alignSize()) || !p) return false;
+  storage->ptr_ = p;
+  return true;
+}
+
+void HipAllocator::free(Storage* storage) { generalFree(storage->ptr_); }
+
+bool HipAllocator::generalAlloc(void** ptr, size_t cap, size_t align) {
+  const size_t bytes = roundUp(cap ? cap : 1, align);
+  MLLM_CHECK_HIP(hipMalloc(ptr, bytes));  // hipMalloc returns memory aligned to 256 bytes or more
+  return *ptr != nullptr;
+}
+
+void HipAllocator::generalFree(void* ptr) {
+  if (!ptr) return;
+  MLLM_CHECK_HIP(hipDeviceSynchronize());  // the stream may still be using it
+  MLLM_CHECK_HIP(hipFree(ptr));
+}
+
+size_t HipAllocator::allocSize(Storage* storage) { return roundUp(storage->size_, alignSize()); }
+
+bool HostAllocator::alloc(const std::shared_ptr<Storage>& storage) {
+  void* p = nullptr;
+  if (!generalAlloc(&p, storage->size_, alignSize())) return false;
+  storage->ptr_ = p;
+  return true;
+}
+
+void HostAllocator::free(Storage* storage) { generalFree(storage->ptr_); }
+
+bool HostAllocator::generalAlloc(void** ptr, size_t cap, size_t align) {
+  *ptr = std::aligned_alloc(align, roundUp(cap ? cap : 1, align));
+  return *ptr != nullptr;
+}
+
+void HostAllocator::generalFree(void* ptr) { std::free(ptr); }
+
+size_t HostAllocator::allocSize(Storage* storage) { return roundUp(storage->size_, alignSize()); }
+
+HostBackend::HostBackend() : BackendBase(kCPU) { allocator_ = std::make_shared<HostAllocator>(); }
+
+HipBackend::HipBackend() : BackendBase(kHIP) {
+  int count = 0;
+  MLLM_CHECK_HIP(hipGetDeviceCount(&count));
+  if (count < 1) MLLM_ERROR_EXIT(kHipError, "no HIP device is visible");
+  MLLM_CHECK_HIP(hipSetDevice(0));
+  hipDeviceProp_t prop{};
+  MLLM_CHECK_HIP(hipGetDeviceProperties(&prop, 0));
+  MLLM_INFO("Found device: %s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+  hipStream_t s = nullptr;
+  MLLM_CHECK_HIP(hipStreamCreate(&s));  // default priority
+  stream_ = s;
+  allocator_ = std::make_shared<HipAllocator>();
+  regOpFactory<HipLinearOpFactory, HipD2HOpFactory>();
+}
+
+HipBackend::~HipBackend() {
+  if (stream_) {
+    (void)hipStreamSynchronize(static_cast<hipStream_t>(stream_));
+    (void)hipStreamDestroy(static_cast<hipStream_t>(stream_));
+  }
+}
+
+void HipBackend::synchronize() const {
+  MLLM_CHECK_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream_)));
+}
+
+std::shared_ptr<HipBackend> createHipBackend() { return std::make_shared<HipBackend>(); }
+std::shared_ptr<HostBackend> createHostBackend() { return std::make_shared<HostBackend>(); }
+
+HipBackend& currentHipBackend() {
+  auto b = std::dynamic_pointer_cast<HipBackend>(MllmEngineCtx::instance().getBackend(kHIP));
+  if (!b) MLLM_ERROR_EXIT(kCoreError, "the backend registered for HIP is not a HipBackend");
+  return *b;
+}
+
+Tensor toDevice(const Tensor& host) {
+  MLLM_RT_ASSERT(host.device() == kCPU);
+  Tensor d = Tensor::empty(host.shape(), host.dtype(), kHIP).alloc();
+  d.setName(host.name());
+  auto s = static_cast<hipStream_t>(currentHipBackend().stream());
+  MLLM_CHECK_HIP(hipMemcpyAsync(d.ptr<void>(), host.ptr<void>(), host.bytes(), hipMemcpyHostToDevice, s));
+  MLLM_CHECK_HIP(hipStreamSynchronize(s));  // the source may be pageable or go away
+  return d;
+}
+
+Tensor toHost(const Tensor& device) {
+  MLLM_RT_ASSERT(device.device() == kHIP);
+  Tensor h = Tensor::empty(device.shape(), device.dtype(), kCPU).alloc();
+  h.setName(device.name());
+  auto s = static_cast<hipStream_t>(currentHipBackend().stream());
+  MLLM_CHECK_HIP(hipMemcpyAsync(h.ptr<void>(), device.ptr<void>(), device.bytes(), hipMemcpyDeviceToHost, s));
+  MLLM_CHECK_HIP(hipStreamSynchronize(s));
+  return h;
+}
+
+}  // namespace mllm::hip

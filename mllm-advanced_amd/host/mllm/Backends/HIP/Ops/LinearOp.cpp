@@ -1,0 +1,170 @@
+#include "mllm/Backends/HIP/Ops/LinearOp.hpp"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstring>
+
+#include "mllm/Backends/HIP/HipBackend.hpp"
+#include "mllm/Engine/Context.hpp"
+#include "mllm/Engine/ParameterReader.hpp"
+#include "mllm/Utils/Log.hpp"
+#include "w4a32_hip.h"
+
+namespace mllm::hip {
+
+namespace {
+
+void check(int rc, const char* what) {
+  if (rc != W4A32_OK) MLLM_ERROR_EXIT(kHipError, "%s failed: %s", what, w4a32_error_string(rc));
+}
+
+void checkHip(hipError_t e, const char* what) {
+  if (e != hipSuccess) MLLM_ERROR_EXIT(kHipError, "%s failed: %s", what, hipGetErrorString(e));
+}
+
+// [KAI-recall, unpinned] size of the blob the reference's Arm quantizer writes for nr | N:
+// per row K/2 nibble bytes + K/32 bf16 scales + f32 row sum + f32 bias.
+size_t kleidiaiBlobBytes(int N, int K) { return (size_t)N * (K / 2 + K / 32 * 2 + 8); }
+
+}  // namespace
+
+HipLinearOp::HipLinearOp(const LinearOpCargo& cargo) : LinearOp(cargo) {}
+
+size_t HipLinearOp::nativeBlobBytes(int N, int K) {
+  return w4a32_native_u4_bytes(N, K) + w4a32_native_scale_bytes(N, K) + (size_t)N * sizeof(float);
+}
+
+void HipLinearOp::load(const std::shared_ptr<ParameterLoader>& ploader) {
+  const int N = cargo_.out_channels, K = cargo_.in_channels;
+  if (!isW4A32ImplType(cargo_.impl_type_)) {
+    MLLM_ERROR_EXIT(kCoreError, "%s: the HIP backend implements the W4A32 Linear family only "
+                    "(KaiLinear_f32_qai8dxp_qsi4c32p_mxk_nxk:*), impl type %d asked",
+                    name().c_str(), static_cast<int>(cargo_.impl_type_));
+    return;
+  }
+  const size_t packed_bytes = w4a32_packed_bytes(N, K);
+  if (packed_bytes == 0) {
+    MLLM_ERROR_EXIT(kShapeError, "%s: in_channels %d must be a positive multiple of 32", name().c_str(), K);
+    return;
+  }
+  LinearOp::load(ploader);  // weight_/bias_ now alias the (host) parameter file
+  auto& hb = currentHipBackend();
+  void* stream = hb.stream();
+  Tensor packed = Tensor::empty({static_cast<int32_t>(packed_bytes)}, kInt8, kHIP).alloc();
+
+  if (weight_.dtype() == kFp32 && weight_.shape().size() == 2 && weight_.shape()[0] == N &&
+      weight_.shape()[1] == K) {
+    Tensor w_dev = toDevice(weight_);
+    Tensor b_dev;
+    if (cargo_.bias) {
+      if (bias_.dtype() != kFp32 || static_cast<int>(bias_.numel()) != N) {
+        MLLM_ERROR_EXIT(kShapeError, "%s.bias must be f32 [%d]", name().c_str(), N);
+        return;
+      }
+      b_dev = toDevice(bias_);
+    }
+    const size_t tmp_bytes = w4a32_native_u4_bytes(N, K) + w4a32_native_scale_bytes(N, K);
+    Tensor tmp = Tensor::empty({static_cast<int32_t>(tmp_bytes)}, kInt8, kHIP).alloc();
+    check(w4a32_quant_pack_rhs(w_dev.ptr<float>(), b_dev.isNil() ? nullptr : b_dev.ptr<float>(), N, K,
+                               packed.ptr<void>(), tmp.ptr<void>(), W4A32_BF16_TRUNC, stream),
+          "w4a32_quant_pack_rhs");
+    hb.synchronize();  // tmp, w_dev, b_dev are released on return
+  } else if (weight_.dtype() == kInt8 && weight_.numel() == nativeBlobBytes(N, K)) {
+    Tensor blob = toDevice(weight_);
+    const uint8_t* u4 = blob.ptr<uint8_t>();
+    const auto* sc = reinterpret_cast<const uint16_t*>(u4 + w4a32_native_u4_bytes(N, K));
+    const auto* bias = reinterpret_cast<const float*>(u4 + w4a32_native_u4_bytes(N, K) +
+                                                      w4a32_native_scale_bytes(N, K));
+    check(w4a32_repack_native(u4, sc, bias, N, K, packed.ptr<void>(), stream), "w4a32_repack_native");
+    hb.synchronize();
+  } else if (weight_.dtype() == kInt8 && weight_.numel() == kleidiaiBlobBytes(N, K)) {
+    MLLM_ERROR_EXIT(kCoreError, "%s.weight looks like a KleidiAI-packed blob (%zu bytes). Its byte "
+                    "layout depends on the Arm tile and is not defined by the reference's own "
+                    "sources; re-quantize from the f32 model with this backend's quantizer.",
+                    name().c_str(), weight_.numel());
+    return;
+  } else {
+    MLLM_ERROR_EXIT(kShapeError, "%s.weight: expected f32 [%d,%d] or an int8 W4 blob of %zu bytes, "
+                    "got %s with %zu elements", name().c_str(), N, K, nativeBlobBytes(N, K),
+                    dataTypes2Str(weight_.dtype()), weight_.numel());
+    return;
+  }
+  packed.setName(name() + ".weight");
+  weight_ = packed;  // the op now holds the device blob; the host tensors are dropped
+  bias_ = Tensor::nil();
+}
+
+void HipLinearOp::reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
+  const auto& i = inputs[0];
+  auto o_shape = i.shape();
+  MLLM_RT_ASSERT_EQ(o_shape[o_shape.size() - 1], cargo_.in_channels);
+  o_shape[o_shape.size() - 1] = cargo_.out_channels;
+  // the W4A32 family always produces f32 (reference Arm/Ops/LinearOp.cpp:253-260)
+  outputs.emplace_back(Tensor::empty(o_shape, kFp32, i.device()));
+}
+
+void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
+  const auto& x = inputs[0];
+  auto& y = outputs[0];
+  if (x.device() != kHIP || x.dtype() != kFp32) {
+    MLLM_ERROR_EXIT(kCoreError, "%s: input must be an f32 tensor on the HIP device", name().c_str());
+    return;
+  }
+  if (weight_.isNil() || weight_.device() != kHIP) {
+    MLLM_ERROR_EXIT(kCoreError, "%s: forward before load", name().c_str());
+    return;
+  }
+  const int K = cargo_.in_channels, N = cargo_.out_channels;
+  // Every leading dimension is a row. (The reference reads M = shape[-2] and ignores the others,
+  // Arm/Ops/LinearOp.cpp:68; the engine only ever runs batch 1, where the two agree.)
+  const int M = static_cast<int>(x.numel() / static_cast<size_t>(K));
+  const size_t need = w4a32_workspace_bytes(M, K);
+  if (workspace_.isNil() || workspace_.bytes() < need) {
+    workspace_ = Tensor::empty({static_cast<int32_t>(need)}, kInt8, kHIP).alloc();
+  }
+  check(w4a32_matmul(y.ptr<float>(), x.ptr<float>(), weight_.ptr<void>(), workspace_.ptr<void>(), M, K,
+                     N, currentHipBackend().stream()),
+        "w4a32_matmul");
+  // Stays asynchronous on the backend's stream: a host consumer goes through D2H, which waits.
+}
+
+void HipD2HOp::reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
+  outputs.emplace_back(Tensor::empty(inputs[0].shape(), inputs[0].dtype(), kCPU));
+}
+
+void HipD2HOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
+  auto s = static_cast<hipStream_t>(currentHipBackend().stream());
+  checkHip(hipMemcpyAsync(outputs[0].ptr<void>(), inputs[0].ptr<void>(), inputs[0].bytes(),
+                          hipMemcpyDeviceToHost, s), "hipMemcpyAsync(D2H)");
+  checkHip(hipStreamSynchronize(s), "hipStreamSynchronize");
+}
+
+Tensor quantizeLinearForFile(const Tensor& weight_f32, const Tensor& bias_f32_or_nil) {
+  MLLM_RT_ASSERT(weight_f32.dtype() == kFp32 && weight_f32.shape().size() == 2);
+  const int N = weight_f32.shape()[0], K = weight_f32.shape()[1];
+  const size_t u4_bytes = w4a32_native_u4_bytes(N, K), sc_bytes = w4a32_native_scale_bytes(N, K);
+  if (u4_bytes == 0) {
+    MLLM_ERROR_EXIT(kShapeError, "quantize: in_channels %d must be a positive multiple of 32", K);
+    return Tensor::nil();
+  }
+  auto& hb = currentHipBackend();
+  Tensor w_dev = toDevice(weight_f32);
+  Tensor planes = Tensor::empty({static_cast<int32_t>(u4_bytes + sc_bytes)}, kInt8, kHIP).alloc();
+  check(w4a32_quant_rhs_native(w_dev.ptr<float>(), N, K, planes.ptr<uint8_t>(),
+                               reinterpret_cast<uint16_t*>(planes.ptr<uint8_t>() + u4_bytes),
+                               W4A32_BF16_TRUNC, hb.stream()),
+        "w4a32_quant_rhs_native");
+  Tensor planes_host = toHost(planes);
+  Tensor blob = Tensor::empty({static_cast<int32_t>(HipLinearOp::nativeBlobBytes(N, K))}, kInt8, kCPU).alloc();
+  std::memcpy(blob.ptr<uint8_t>(), planes_host.ptr<uint8_t>(), u4_bytes + sc_bytes);
+  auto* bias_out = reinterpret_cast<float*>(blob.ptr<uint8_t>() + u4_bytes + sc_bytes);
+  if (bias_f32_or_nil.isNil()) {
+    std::memset(bias_out, 0, (size_t)N * sizeof(float));
+  } else {
+    MLLM_RT_ASSERT(bias_f32_or_nil.dtype() == kFp32 && static_cast<int>(bias_f32_or_nil.numel()) == N);
+    std::memcpy(bias_out, bias_f32_or_nil.ptr<float>(), (size_t)N * sizeof(float));
+  }
+  return blob;
+}
+
+}  // namespace mllm::hip
