@@ -8,10 +8,12 @@ they do in real decoding). Each Linear is the whole op (per-row int8 quantisatio
 activations + the product), exactly what the operator boundary runs per call.
 
 Prints ONE JSON line. `value` = algorithmic bytes of the step / time per step (GB/s), inputs
-resident in HBM. `roofline` = the decode product kernel alone over the same launches (HIP
-events on the launch stream), against 8 TB/s. `extra` carries the M=512 prefill TFLOP/s per
-shape and the per-shape decode figures. `cpu_baseline` = the scalar CPU restatement of the
-reference path on this host, on a bounded sample.
+resident in HBM. `roofline` = the decode kernel (gemv_fused_kernel: row quantisation + product
+in one launch, the only kernel in the step) over the same launches, timed with HIP events on
+the launch stream, against 8 TB/s. `extra` carries per-shape decode figures, the M=512 and
+M=2048 prefill TFLOP/s (whole op and product kernel alone) and the prefill kernel's MFMA
+roofline. `cpu_baseline` = the scalar CPU restatement of the reference path on this host, on a
+bounded sample.
 """
 import argparse
 import importlib
@@ -52,7 +54,10 @@ def parse():
     ap.add_argument("--no-gemm", action="store_true", help="skip the prefill (M=512) leg")
     ap.add_argument("--eager", action="store_true", help="launch from Python instead of a HIP graph")
     ap.add_argument("--roofline-only", action="store_true",
-                    help="only the product-kernel passes (the run profiled under rocprofv3)")
+                    help="only the decode passes (the run profiled under rocprofv3 --kernel-trace)")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="a 256 MiB copy, then the decode kernel on gate_proj and lm_head and the "
+                         "prefill kernel on gate_proj (the run profiled under rocprofv3 --pmc)")
     return ap.parse_args()
 
 
@@ -139,26 +144,58 @@ def main():
         return e0.elapsed_time(e1) / steps, wall * 1e3 / steps
 
     use_graph = not args.eager
-    # quantise the activations once so the product-only pass has valid inputs
-    with torch.cuda.stream(stream):
-        whole_op_pass()
-    stream.synchronize()
 
-    ms_prod, _ = timed(product_only_pass, args.steps, args.warmup, use_graph)
+    if args.traffic_probe:
+        # known traffic first: 256 MiB read + 256 MiB written by a plain copy kernel
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        with torch.cuda.stream(stream):
+            for _ in range(3):
+                dst.copy_(src)
+            gate, M = layers[0][4], 512
+            # three different gate_proj buffers (cold weights each time), then lm_head three times
+            for lin in (layers[1][4], layers[2][4], layers[3][4], lm_head, lm_head, lm_head):
+                L.w4a32_matmul(y_by_n[lin.N].data_ptr(), x_by_k[lin.K].data_ptr(),
+                               lin.packed.data_ptr(), ws_by_k[lin.K].data_ptr(), 1, lin.K, lin.N, sptr)
+            x = torch.randn((M, gate.K), generator=xgen, device="cuda")
+            ws = torch.empty(pkg.workspace_bytes(M, gate.K), dtype=torch.uint8, device="cuda")
+            y = torch.empty((M, gate.N), device="cuda")
+            for _ in range(3):
+                L.w4a32_matmul(y.data_ptr(), x.data_ptr(), gate.packed.data_ptr(), ws.data_ptr(), M,
+                               gate.K, gate.N, sptr)
+        torch.cuda.synchronize()
+        print(json.dumps({"traffic_probe": {
+            "copy_bytes_read": 256 << 20, "copy_bytes_written": 256 << 20,
+            "gate_proj_M1_algorithmic_bytes": gate.bytes[1], "lm_head_M1_algorithmic_bytes": lm_head.bytes[1],
+            "gate_proj_M512_weight_bytes": gate.bytes[1] - 1 * gate.K * 4 - 1 * gate.N * 4}}))
+        return
+
+    # The whole op per decoder Linear is ONE kernel (gemv_fused_kernel); the step is 196
+    # launches of it plus lm_head (row-quant kernel + product kernel).
+    ms_step, wall_ms = timed(whole_op_pass, args.steps, args.warmup, use_graph)
     n_launch = len(step_linears)
-    roof_avg_us = ms_prod * 1e3 / n_launch
+    roof_avg_us = ms_step * 1e3 / n_launch
     roof_bytes = step_bytes / n_launch
     achieved = roof_bytes / (roof_avg_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                "kernel": "gemv_dot4_kernel<1>", "launches_per_step": n_launch,
-                "avg_launch_us": round(roof_avg_us, 3), "algorithmic_bytes_per_launch": int(roof_bytes)}
+                "kernel": "gemv_fused_kernel<1,R> (R=1 for K=1536, R=2 for K=8960); lm_head runs "
+                          "quant_lhs_kernel + gemv_q_kernel<1>",
+                "launches_per_step": n_launch, "avg_launch_us": round(roof_avg_us, 3),
+                "algorithmic_bytes_per_launch": int(roof_bytes),
+                "note": "average over the step's 197 launches (28 x 7 decoder shapes + lm_head), "
+                        "launch period inside a HIP graph; per-shape figures are in extra"}
     if args.roofline_only:
         print(json.dumps({"roofline": roofline}))
         return
 
-    ms_step, wall_ms = timed(whole_op_pass, args.steps, args.warmup, use_graph)
     value = step_bytes / (ms_step * 1e-3) / 1e9
+    # the same products on activations quantised once (w4a32_quant_lhs + w4a32_matmul_quantized)
+    with torch.cuda.stream(stream):
+        for K in ws_by_k:
+            L.w4a32_quant_lhs(x_by_k[K].data_ptr(), 1, K, K, ws_by_k[K].data_ptr(), sptr)
+    stream.synchronize()
+    ms_prod, _ = timed(product_only_pass, args.steps, args.warmup, use_graph)
 
     extra = {"decode_linears_tokens_per_s": round(1e3 / ms_step, 1),
              "wall_ms_per_step": round(wall_ms, 4), "graph": use_graph,
@@ -172,53 +209,77 @@ def main():
             lins = [lm_head] if name == "lm_head" else [layer[idx] for layer in layers]
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             for l in lins:
-                L.w4a32_matmul_quantized(y_by_n[N].data_ptr(), ws_by_k[K].data_ptr(),
-                                         l.packed.data_ptr(), 1, K, N, sptr)
+                L.w4a32_matmul(y_by_n[N].data_ptr(), x_by_k[K].data_ptr(), l.packed.data_ptr(),
+                               ws_by_k[K].data_ptr(), 1, K, N, sptr)
             e0.record(stream)
             for _ in range(reps):
                 for l in lins:
-                    L.w4a32_matmul_quantized(y_by_n[N].data_ptr(), ws_by_k[K].data_ptr(),
-                                             l.packed.data_ptr(), 1, K, N, sptr)
+                    L.w4a32_matmul(y_by_n[N].data_ptr(), x_by_k[K].data_ptr(), l.packed.data_ptr(),
+                                   ws_by_k[K].data_ptr(), 1, K, N, sptr)
             e1.record(stream)
             stream.synchronize()
             us = e0.elapsed_time(e1) * 1e3 / (reps * len(lins))
-            per_shape[name] = {"us": round(us, 2),
-                               "GBps": round(lins[0].bytes[1] / (us * 1e-6) / 1e9, 1),
-                               "note": "cache-resident" if name == "lm_head" else "rotating 28 buffers"}
+            gbs = lins[0].bytes[1] / (us * 1e-6) / 1e9
+            per_shape[name] = {"us": round(us, 2), "GBps": round(gbs, 1),
+                               "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 3),
+                               "note": ("one buffer, 132 MB (half of the 256 MB Infinity Cache)"
+                                        if name == "lm_head" else "rotating over 28 weight buffers")}
     extra["decode_per_shape"] = per_shape
 
-    # ---- prefill leg: M=512 whole op per shape
+    # ---- prefill leg: whole op (row quant + product) and the product kernel alone
     if not args.no_gemm:
-        M = 512
-        gemm = {}
-        total_flop, total_ms = 0.0, 0.0
+        prefill = {}
         with torch.cuda.stream(stream):
-            for idx, (name, K, N, b) in enumerate(LAYER_LINEARS):
-                lin = layers[0][idx]
-                x = torch.randn((M, K), generator=xgen, device="cuda")
-                ws = torch.empty(pkg.workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
-                y = torch.empty((M, N), device="cuda")
+            for M in (512, 2048):
+                per, tot_flop, tot_ms, tot_kms = {}, 0.0, 0.0, 0.0
+                for idx, (name, K, N, b) in enumerate(LAYER_LINEARS):
+                    lin = layers[0][idx]
+                    x = torch.randn((M, K), generator=xgen, device="cuda")
+                    x[: max(1, M // 100)] *= 20.0      # 1 % of rows x20: per-row scales matter
+                    ws = torch.empty(pkg.workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
+                    y = torch.empty((M, N), device="cuda")
 
-                def call():
-                    rc = L.w4a32_matmul(y.data_ptr(), x.data_ptr(), lin.packed.data_ptr(),
-                                        ws.data_ptr(), M, K, N, sptr)
-                    if rc:
-                        raise pkg.W4A32Error(f"w4a32_matmul M=512 ({name}) -> {rc}")
-                for _ in range(3):
-                    call()
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record(stream)
-                for _ in range(10):
-                    call()
-                e1.record(stream)
-                stream.synchronize()
-                ms = e0.elapsed_time(e1) / 10
-                flop = 2.0 * M * N * K
-                gemm[name] = {"ms": round(ms, 4), "TFLOPs": round(flop / (ms * 1e-3) / 1e12, 2)}
-                total_flop += flop
-                total_ms += ms
-        extra["prefill_M512_per_shape"] = gemm
-        extra["prefill_M512_layer_TFLOPs"] = round(total_flop / (total_ms * 1e-3) / 1e12, 2)
+                    def whole():
+                        rc = L.w4a32_matmul(y.data_ptr(), x.data_ptr(), lin.packed.data_ptr(),
+                                            ws.data_ptr(), M, K, N, sptr)
+                        if rc:
+                            raise pkg.W4A32Error(f"w4a32_matmul M={M} ({name}) -> {rc}")
+
+                    def kernel_only():
+                        rc = L.w4a32_matmul_quantized(y.data_ptr(), ws.data_ptr(), lin.packed.data_ptr(),
+                                                      M, K, N, sptr)
+                        if rc:
+                            raise pkg.W4A32Error(f"w4a32_matmul_quantized M={M} ({name}) -> {rc}")
+                    times = []
+                    for fn in (whole, kernel_only):
+                        for _ in range(3):
+                            fn()
+                        e0 = torch.cuda.Event(enable_timing=True)
+                        e1 = torch.cuda.Event(enable_timing=True)
+                        e0.record(stream)
+                        for _ in range(20):
+                            fn()
+                        e1.record(stream)
+                        stream.synchronize()
+                        times.append(e0.elapsed_time(e1) / 20)
+                    flop = 2.0 * M * N * K
+                    per[name] = {"ms": round(times[0], 4), "TFLOPs": round(flop / (times[0] * 1e-3) / 1e12, 1),
+                                 "kernel_ms": round(times[1], 4),
+                                 "kernel_TFLOPs": round(flop / (times[1] * 1e-3) / 1e12, 1)}
+                    tot_flop += flop
+                    tot_ms += times[0]
+                    tot_kms += times[1]
+                prefill[f"M{M}"] = {"per_shape": per,
+                                    "layer_TFLOPs": round(tot_flop / (tot_ms * 1e-3) / 1e12, 1),
+                                    "layer_kernel_TFLOPs": round(tot_flop / (tot_kms * 1e-3) / 1e12, 1)}
+        extra["prefill"] = prefill
+        best = prefill["M2048"]["per_shape"]["gate_proj"]["kernel_TFLOPs"]
+        extra["prefill_roofline"] = {"bound": "mfma", "kernel": "gemm_f16_kernel (v_mfma_f32_32x32x16_f16)",
+                                     "workload": "gate_proj M=2048 K=1536 N=8960, product kernel alone",
+                                     "achieved": best, "peak": 2500.0, "unit": "TFLOP/s",
+                                     "frac": round(best / 2500.0, 4),
+                                     "M512_gate_proj_kernel_TFLOPs":
+                                         prefill["M512"]["per_shape"]["gate_proj"]["kernel_TFLOPs"]}
 
     # ---- CPU baseline: scalar restatement of the reference path, bounded sample
     cpu = None

@@ -157,6 +157,13 @@ int w4a32_matmul_quantized(float* d_y, const void* d_ws, const void* d_packed, i
 
 int w4a32_matmul(float* d_y, const float* d_x, const void* d_packed, void* d_ws, int M, int K,
                  int N, void* stream) {
+  if (M > 0 && shape_ok(N, K) == W4A32_OK && w4::gemv_fused_applies(M, K, N)) {
+    // decode sizes: one kernel quantises the rows and multiplies (the workspace stays unused)
+    if (!d_y || !d_x || !d_packed || !d_ws) return W4A32_EINVAL;
+    if (!aligned(d_x, 16) || !aligned(d_packed, 16) || !aligned(d_y, 4)) return W4A32_EINVAL;
+    return from_hip(w4::launch_gemv_fused(d_y, d_x, K, static_cast<const uint8_t*>(d_packed), M, K,
+                                          N, static_cast<hipStream_t>(stream)));
+  }
   if (int e = w4a32_quant_lhs(d_x, M, K, K, d_ws, stream)) return e;
   return w4a32_matmul_quantized(d_y, d_ws, d_packed, M, K, N, stream);
 }

@@ -1,58 +1,37 @@
-// Decode product (M = 1..8): y[M][N] from int8 activation rows and the tiled 4-bit weights.
+// Decode product (M = 1..8): y[M][N] from f32 or already-quantised activation rows and the
+// tiled 4-bit weights.
 //
 // HBM-bound: per output row the kernel must stream K/2 bytes of nibbles and K/16 bytes of
 // scales once; everything else (activations, rsum, bias) is a few KB that live in L2/LDS.
 //
 // Work split: one workgroup per 16-row weight tile row (nt); its W wavefronts take the
 // 128-k chunks round-robin, so a workgroup streams one contiguous KC*1152-byte run.
-// A wavefront's 128-bit-per-lane load is one whole 1 KiB tile. The next chunk is requested
-// before the current one is consumed. Activations are staged once per workgroup into LDS
-// (after the first weight loads are in flight) and read back as 64-bit broadcasts.
+// A wavefront's 128-bit-per-lane load is one whole 1 KiB tile. The first chunk is requested
+// before anything else happens, the next one before the current one is consumed.
+//
+// Two entry kernels share the loop:
+//   gemv_q_kernel      activations already quantised (workspace of w4a32_quant_lhs)
+//   gemv_fused_kernel  quantises the f32 rows itself: every workgroup recomputes the row
+//                      min/max (a few KB from L2, DPP reductions) and quantises into its own
+//                      LDS copy with the same arithmetic as the standalone kernel. This removes
+//                      one kernel launch per Linear, which at decode sizes costs more than the
+//                      product itself.
 //
 // Arithmetic per 8 weights (one dword): two mask ops give int8 vectors of 16*q, two
 // v_dot4_i32_i8 give 16 * sum a_q*q exactly, one cvt + one fma apply the block scale in f32.
 // The 1/16 and the activation offset (off * rsum[n]) are folded in once per output.
 #include "w4a32_internal.h"
+#include "w4a32_quant_math.h"
 
 namespace w4 {
 
+// Streams this wavefront's chunks of tile row `tiles` against the int8 rows in LDS and leaves
+// the per-(m, j) sums over the whole workgroup in s_red[m*16 + j] order via a final reduction.
 template <int M>
-__global__ __launch_bounds__(1024) void gemv_dot4_kernel(
-    float* __restrict__ y, const int8_t* __restrict__ aq, const float* __restrict__ recip,
-    const int32_t* __restrict__ negzp, const uint8_t* __restrict__ packed, int N, int K, int KC,
-    const float* __restrict__ rsum, const float* __restrict__ bias) {
-  extern __shared__ __align__(16) uint8_t smem[];
-  const int Kp = KC * kTileK;
-  int8_t* s_a = reinterpret_cast<int8_t*>(smem);                  // [M][Kp]
-  float* s_red = reinterpret_cast<float*>(smem + (size_t)M * Kp); // [W][M][16]
-
-  const int nt = blockIdx.x;
-  const int W = blockDim.x >> 6;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+__device__ __forceinline__ void gemv_accumulate(const uint8_t* __restrict__ tiles, int KC, int Kp,
+                                                const int8_t* s_a, uint4 wq, uint2 sc, int kc,
+                                                int W, int lane, float (&acc)[M]) {
   const int g = lane >> 4, j = lane & 15;
-
-  const uint8_t* tiles = packed + (size_t)nt * KC * kTileBytes;
-
-  // First chunk of this wavefront: in flight while the activations are staged.
-  int kc = wave;
-  uint4 wq = make_uint4(0, 0, 0, 0);
-  uint2 sc = make_uint2(0, 0);
-  if (kc < KC) {
-    wq = *reinterpret_cast<const uint4*>(tiles + (size_t)kc * kTileBytes + 16 * lane);
-    sc = *reinterpret_cast<const uint2*>(tiles + (size_t)kc * kTileBytes + kTileQBytes + 8 * j);
-  }
-
-  // Stage a_q into LDS, 16 bytes per thread per step; k >= K (tile padding) reads as 0.
-  const int vec_per_row = Kp / 16;
-  for (int v = threadIdx.x; v < M * vec_per_row; v += blockDim.x) {
-    const int m = v / vec_per_row, c = v % vec_per_row;
-    uint4 val = make_uint4(0, 0, 0, 0);
-    if (16 * c < K) val = *reinterpret_cast<const uint4*>(aq + (size_t)m * K + 16 * c);
-    *reinterpret_cast<uint4*>(s_a + (size_t)m * Kp + 16 * c) = val;
-  }
-  __syncthreads();
-
-  float acc[M];
 #pragma unroll
   for (int m = 0; m < M; ++m) acc[m] = 0.0f;
 
@@ -64,7 +43,6 @@ __global__ __launch_bounds__(1024) void gemv_dot4_kernel(
       wq_n = *reinterpret_cast<const uint4*>(tiles + (size_t)kn * kTileBytes + 16 * lane);
       sc_n = *reinterpret_cast<const uint2*>(tiles + (size_t)kn * kTileBytes + kTileQBytes + 8 * j);
     }
-
     const uint32_t wv[4] = {wq.x, wq.y, wq.z, wq.w};
     const float sv[4] = {__uint_as_float(sc.x << 16), __uint_as_float(sc.x & 0xFFFF0000u),
                          __uint_as_float(sc.y << 16), __uint_as_float(sc.y & 0xFFFF0000u)};
@@ -85,35 +63,241 @@ __global__ __launch_bounds__(1024) void gemv_dot4_kernel(
     wq = wq_n;
     sc = sc_n;
   }
-
-  // Sum the four k-groups of a row (lanes j, j+16, j+32, j+48), then the wavefronts.
+  // Sum the four k-groups of a row (lanes j, j+16, j+32, j+48).
 #pragma unroll
   for (int m = 0; m < M; ++m) {
     acc[m] += __shfl_xor(acc[m], 16, 64);
     acc[m] += __shfl_xor(acc[m], 32, 64);
   }
-  if (g == 0) {
+}
+
+// Cross-wavefront sum and the output transform
+//   y = (sum/16 + off * rsum[n]) * lhs_scale + bias[n], clamped to the finite f32 range.
+// When the workgroup has at least 16*M threads, thread o owns output o and already holds
+// rsum/bias of its column (rs, bs: requested at kernel start); smaller workgroups (K < 128*M/4)
+// stride over the outputs and fetch them here.
+template <int M>
+__device__ __forceinline__ void gemv_finish(float* __restrict__ y, int N, int nt, int W,
+                                            const float (&acc)[M], float* s_red,
+                                            const float (&recip_m)[M], const int (&negzp_m)[M],
+                                            const float* __restrict__ rsum,
+                                            const float* __restrict__ bias, float rs, float bs) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane < 16) {
 #pragma unroll
-    for (int m = 0; m < M; ++m) s_red[(wave * M + m) * 16 + j] = acc[m];
+    for (int m = 0; m < M; ++m) s_red[(wave * M + m) * 16 + lane] = acc[m];
   }
   __syncthreads();
-
-  // 16*M outputs; a workgroup may have as few as 64 threads, so stride over them.
+  const bool prefetched = blockDim.x >= 16 * M;
   for (int o = threadIdx.x; o < 16 * M; o += blockDim.x) {
     const int m = o >> 4, jj = o & 15;
     const int n = kTileRows * nt + jj;
     if (n < N) {
       float s = 0.0f;
       for (int w = 0; w < W; ++w) s += s_red[(w * M + m) * 16 + jj];
-      float v = __fmaf_rn((float)negzp[m], rsum[n], s * 0.0625f);
-      v = __fmaf_rn(v, recip[m], bias[n]);
+      float rcp = 0.0f;
+      int off = 0;
+#pragma unroll
+      for (int mm = 0; mm < M; ++mm) {  // compile-time indices keep the arrays in registers
+        if (mm == m) {
+          rcp = recip_m[mm];
+          off = negzp_m[mm];
+        }
+      }
+      const float rsn = prefetched ? rs : rsum[n];
+      const float bsn = prefetched ? bs : bias[n];
+      float v = __fmaf_rn((float)off, rsn, s * 0.0625f);
+      v = __fmaf_rn(v, rcp, bsn);
       v = fminf(fmaxf(v, -3.402823466e+38f), 3.402823466e+38f);
       y[(size_t)m * N + n] = v;
     }
   }
 }
 
+template <int M>
+__global__ __launch_bounds__(1024) void gemv_q_kernel(
+    float* __restrict__ y, const int8_t* __restrict__ aq, const float* __restrict__ recip,
+    const int32_t* __restrict__ negzp, const uint8_t* __restrict__ packed, int N, int K, int KC,
+    const float* __restrict__ rsum, const float* __restrict__ bias) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  const int Kp = KC * kTileK;
+  int8_t* s_a = reinterpret_cast<int8_t*>(smem);                    // [M][Kp]
+  float* s_red = reinterpret_cast<float*>(smem + (size_t)M * Kp);   // [W][M][16]
+  float* s_par = s_red + (blockDim.x >> 6) * M * 16;                // recip[M], negzp[M]
+
+  const int nt = blockIdx.x;
+  const int W = blockDim.x >> 6;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const uint8_t* tiles = packed + (size_t)nt * KC * kTileBytes;
+
+  // First chunk of this wavefront: in flight while the activations are staged.
+  uint4 wq = make_uint4(0, 0, 0, 0);
+  uint2 sc = make_uint2(0, 0);
+  if (wave < KC) {
+    wq = *reinterpret_cast<const uint4*>(tiles + (size_t)wave * kTileBytes + 16 * lane);
+    sc = *reinterpret_cast<const uint2*>(tiles + (size_t)wave * kTileBytes + kTileQBytes +
+                                         8 * (lane & 15));
+  }
+  // Output-transform operands, requested now so the epilogue does not wait on memory.
+  float rs = 0.0f, bs = 0.0f;
+  {
+    const int n = kTileRows * nt + (threadIdx.x & 15);
+    if (threadIdx.x < 16 * M && n < N) {
+      rs = rsum[n];
+      bs = bias[n];
+    }
+  }
+  if (threadIdx.x < M) {
+    s_par[threadIdx.x] = recip[threadIdx.x];
+    reinterpret_cast<int*>(s_par)[M + threadIdx.x] = negzp[threadIdx.x];
+  }
+
+  // Stage a_q into LDS, 16 bytes per thread per step; k >= K (tile padding) reads as 0.
+  const int vec_per_row = Kp / 16;
+  for (int v = threadIdx.x; v < M * vec_per_row; v += blockDim.x) {
+    const int m = v / vec_per_row, c = v % vec_per_row;
+    uint4 val = make_uint4(0, 0, 0, 0);
+    if (16 * c < K) val = *reinterpret_cast<const uint4*>(aq + (size_t)m * K + 16 * c);
+    *reinterpret_cast<uint4*>(s_a + (size_t)m * Kp + 16 * c) = val;
+  }
+  __syncthreads();
+
+  float acc[M];
+  gemv_accumulate<M>(tiles, KC, Kp, s_a, wq, sc, wave, W, lane, acc);
+  float recip_m[M];
+  int negzp_m[M];
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+    recip_m[m] = s_par[m];
+    negzp_m[m] = reinterpret_cast<const int*>(s_par)[M + m];
+  }
+  gemv_finish<M>(y, N, nt, W, acc, s_red, recip_m, negzp_m, rsum, bias, rs, bs);
+}
+
+// Whole op in one launch: x f32 [M][K] (row stride ldx) -> y.
+// kFusedR = groups of 8 k a thread may own per row: covers K <= 8 * kFusedR * blockDim.x.
+template <int M, int kFusedR>
+__global__ __launch_bounds__(1024) void gemv_fused_kernel(
+    float* __restrict__ y, const float* __restrict__ x, int ldx, const uint8_t* __restrict__ packed,
+    int N, int K, int KC, const float* __restrict__ rsum, const float* __restrict__ bias) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  const int Kp = KC * kTileK;
+  const int W = blockDim.x >> 6;
+  int8_t* s_a = reinterpret_cast<int8_t*>(smem);                    // [M][Kp]
+  float* s_red = reinterpret_cast<float*>(smem + (size_t)M * Kp);   // [W][M][16]
+  float* s_mm = s_red + W * M * 16;                                 // [W][M][2] min, max
+
+  const int nt = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const uint8_t* tiles = packed + (size_t)nt * KC * kTileBytes;
+
+  uint4 wq = make_uint4(0, 0, 0, 0);
+  uint2 sc = make_uint2(0, 0);
+  if (wave < KC) {
+    wq = *reinterpret_cast<const uint4*>(tiles + (size_t)wave * kTileBytes + 16 * lane);
+    sc = *reinterpret_cast<const uint2*>(tiles + (size_t)wave * kTileBytes + kTileQBytes +
+                                         8 * (lane & 15));
+  }
+  float rs = 0.0f, bs = 0.0f;
+  {
+    const int n = kTileRows * nt + (threadIdx.x & 15);
+    if (threadIdx.x < 16 * M && n < N) {
+      rs = rsum[n];
+      bs = bias[n];
+    }
+  }
+
+  // Each thread owns up to kFusedR groups of 8 consecutive k per row (group index
+  // threadIdx.x + r*blockDim.x) and keeps them in registers from the min/max pass to the
+  // quantise pass, so x is read once. Wavefronts reduce min/max with DPP; the W partial results
+  // meet in LDS.
+  const int groups = K >> 3;
+  float xv[M][kFusedR][8];
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+    const float* row = x + (size_t)m * ldx;
+    float lo = 3.402823466e+38f, hi = -3.402823466e+38f;
+#pragma unroll
+    for (int r = 0; r < kFusedR; ++r) {
+      const int c = threadIdx.x + r * blockDim.x;
+      if (c < groups) {
+        const float4 v0 = *reinterpret_cast<const float4*>(row + 8 * c);
+        const float4 v1 = *reinterpret_cast<const float4*>(row + 8 * c + 4);
+        const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          xv[m][r][e] = f[e];
+          lo = fminf(lo, f[e]);
+          hi = fmaxf(hi, f[e]);
+        }
+      }
+    }
+    lo = wave_minmax<false>(lo);
+    hi = wave_minmax<true>(hi);
+    if (lane == 0) {
+      s_mm[(wave * M + m) * 2 + 0] = lo;
+      s_mm[(wave * M + m) * 2 + 1] = hi;
+    }
+  }
+  __syncthreads();
+
+  RowQuant par[M];
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+    float lo = 3.402823466e+38f, hi = -3.402823466e+38f;
+    for (int w = 0; w < W; ++w) {
+      lo = fminf(lo, s_mm[(w * M + m) * 2 + 0]);
+      hi = fmaxf(hi, s_mm[(w * M + m) * 2 + 1]);
+    }
+    par[m] = row_quant_params(lo, hi);
+  }
+
+  // Quantise into the LDS copy; the tile padding (k >= K) is 0.
+  const int grp_per_row = Kp >> 3;
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+#pragma unroll
+    for (int r = 0; r < kFusedR; ++r) {
+      const int c = threadIdx.x + r * blockDim.x;
+      if (c < grp_per_row) {
+        uint2 out = make_uint2(0, 0);
+        if (c < groups) {
+          int q[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) q[e] = quant_one(xv[m][r][e], par[m]);
+          out.x = pack4(q);
+          out.y = pack4(q + 4);
+        }
+        *reinterpret_cast<uint2*>(s_a + (size_t)m * Kp + 8 * c) = out;
+      }
+    }
+  }
+  __syncthreads();
+
+  float acc[M];
+  gemv_accumulate<M>(tiles, KC, Kp, s_a, wq, sc, wave, W, lane, acc);
+  float recip_m[M];
+  int negzp_m[M];
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+    recip_m[m] = par[m].recip;
+    negzp_m[m] = -par[m].zp;
+  }
+  gemv_finish<M>(y, N, nt, W, acc, s_red, recip_m, negzp_m, rsum, bias, rs, bs);
+}
+
 static int pick_waves(int KC) { return KC < 16 ? KC : 16; }
+
+template <typename Kern>
+static hipError_t raise_lds_limit(Kern kern, size_t lds, bool* raised) {
+  if (lds > 64 * 1024 && !*raised) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) return e;
+    *raised = true;
+  }
+  return hipSuccess;
+}
 
 template <int M>
 static hipError_t launch_gemv_m(float* y, const uint8_t* ws, const uint8_t* packed, int K, int N,
@@ -121,21 +305,30 @@ static hipError_t launch_gemv_m(float* y, const uint8_t* ws, const uint8_t* pack
   const WeightGeom g = weight_geom(N, K);
   const WsGeom w = ws_geom(M, K);
   const int W = pick_waves(g.KC);
-  const size_t lds = (size_t)M * g.Kp + (size_t)W * M * 16 * sizeof(float);
-  auto kern = gemv_dot4_kernel<M>;
-  if (lds > 64 * 1024) {
-    static bool raised = false;  // one attribute call per instantiation is enough
-    if (!raised) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-      if (e != hipSuccess) return e;
-      raised = true;
-    }
-  }
+  const size_t lds = (size_t)M * g.Kp + (size_t)W * M * 16 * sizeof(float) + 2 * M * sizeof(float);
+  auto kern = gemv_q_kernel<M>;
+  static bool raised = false;
+  if (hipError_t e = raise_lds_limit(kern, lds, &raised); e != hipSuccess) return e;
   hipLaunchKernelGGL(kern, dim3(g.NT), dim3(64 * W), lds, s, y,
                      reinterpret_cast<const int8_t*>(ws + w.aq_off),
                      reinterpret_cast<const float*>(ws + w.scale_off),
                      reinterpret_cast<const int32_t*>(ws + w.off_off), packed, N, K, g.KC,
+                     reinterpret_cast<const float*>(packed + g.rsum_off),
+                     reinterpret_cast<const float*>(packed + g.bias_off));
+  return hipGetLastError();
+}
+
+template <int M, int R>
+static hipError_t launch_fused_m(float* y, const float* x, int ldx, const uint8_t* packed, int K,
+                                 int N, hipStream_t s) {
+  const WeightGeom g = weight_geom(N, K);
+  const int W = pick_waves(g.KC);
+  const size_t lds = (size_t)M * g.Kp + (size_t)W * M * 16 * sizeof(float) +
+                     (size_t)W * M * 2 * sizeof(float);
+  auto kern = gemv_fused_kernel<M, R>;
+  static bool raised = false;
+  if (hipError_t e = raise_lds_limit(kern, lds, &raised); e != hipSuccess) return e;
+  hipLaunchKernelGGL(kern, dim3(g.NT), dim3(64 * W), lds, s, y, x, ldx, packed, N, K, g.KC,
                      reinterpret_cast<const float*>(packed + g.rsum_off),
                      reinterpret_cast<const float*>(packed + g.bias_off));
   return hipGetLastError();
@@ -152,6 +345,43 @@ hipError_t launch_gemv(float* y, const uint8_t* ws, const uint8_t* packed, int M
     case 6: return launch_gemv_m<6>(y, ws, packed, K, N, s);
     case 7: return launch_gemv_m<7>(y, ws, packed, K, N, s);
     case 8: return launch_gemv_m<8>(y, ws, packed, K, N, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+// Row groups (of 8 k) per thread the fused kernel needs: 1 if the padded row fits one pass of
+// the workgroup, else 2.
+static int fused_groups_per_thread(int K) {
+  const int KC = (K + kTileK - 1) / kTileK;
+  const long per_pass = (long)8 * 64 * pick_waves(KC);
+  return (int)(((long)KC * kTileK + per_pass - 1) / per_pass);
+}
+
+bool gemv_fused_applies(int M, int K, int N) {
+  // Every workgroup re-reads and re-quantises the M rows. That is cheaper than a second kernel
+  // launch while the rows are small next to the workgroup's weights, each thread can hold its
+  // share of them in registers, and a CU runs only a few workgroups in a row (measured on
+  // MI355X: at N = 151936 the two-kernel path is 1.7x faster, at N <= 8960 the fused one wins).
+  if (M < 1 || M > kGemvMaxM || (long)M * K > 16384 || N > 32768) return false;
+  const int r = fused_groups_per_thread(K);
+  return r == 1 || (r == 2 && M == 1);
+}
+
+hipError_t launch_gemv_fused(float* y, const float* x, int ldx, const uint8_t* packed, int M, int K,
+                             int N, hipStream_t s) {
+  if (fused_groups_per_thread(K) == 2) {
+    if (M != 1) return hipErrorInvalidValue;
+    return launch_fused_m<1, 2>(y, x, ldx, packed, K, N, s);
+  }
+  switch (M) {
+    case 1: return launch_fused_m<1, 1>(y, x, ldx, packed, K, N, s);
+    case 2: return launch_fused_m<2, 1>(y, x, ldx, packed, K, N, s);
+    case 3: return launch_fused_m<3, 1>(y, x, ldx, packed, K, N, s);
+    case 4: return launch_fused_m<4, 1>(y, x, ldx, packed, K, N, s);
+    case 5: return launch_fused_m<5, 1>(y, x, ldx, packed, K, N, s);
+    case 6: return launch_fused_m<6, 1>(y, x, ldx, packed, K, N, s);
+    case 7: return launch_fused_m<7, 1>(y, x, ldx, packed, K, N, s);
+    case 8: return launch_fused_m<8, 1>(y, x, ldx, packed, K, N, s);
     default: return hipErrorInvalidValue;
   }
 }

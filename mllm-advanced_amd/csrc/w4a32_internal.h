@@ -23,6 +23,10 @@ hipError_t launch_quant_lhs(const float* x, int M, int K, int ldx, uint8_t* ws, 
 // products
 hipError_t launch_gemv(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                        hipStream_t s);
+// whole decode op in one launch (row quantisation inside the product kernel)
+bool gemv_fused_applies(int M, int K, int N);
+hipError_t launch_gemv_fused(float* y, const float* x, int ldx, const uint8_t* packed, int M, int K,
+                             int N, hipStream_t s);
 hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                        int kernel, hipStream_t s);
 

@@ -6,20 +6,9 @@
 // even; values are round_half_away(x * scale) + zero_point, clamped to int8. Every f32 product
 // and sum is an explicitly rounded intrinsic so no compiler flag can fuse them.
 #include "w4a32_internal.h"
+#include "w4a32_quant_math.h"
 
 namespace w4 {
-
-__device__ __forceinline__ float wave_min(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, 64));
-  return v;
-}
-
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
-}
 
 constexpr int kLhsThreads = 256;
 
@@ -39,8 +28,8 @@ __global__ __launch_bounds__(kLhsThreads) void quant_lhs_kernel(
     lo = fminf(fminf(lo, v.x), fminf(v.y, fminf(v.z, v.w)));
     hi = fmaxf(fmaxf(hi, v.x), fmaxf(v.y, fmaxf(v.z, v.w)));
   }
-  lo = wave_min(lo);
-  hi = wave_max(hi);
+  lo = wave_minmax<false>(lo);
+  hi = wave_minmax<true>(hi);
   __shared__ float s_lo[kLhsThreads / 64], s_hi[kLhsThreads / 64];
   if ((t & 63) == 0) {
     s_lo[t >> 6] = lo;
@@ -52,22 +41,11 @@ __global__ __launch_bounds__(kLhsThreads) void quant_lhs_kernel(
     lo = fminf(lo, s_lo[w]);
     hi = fmaxf(hi, s_hi[w]);
   }
-
-  const float qmin = -128.0f, qmax = 127.0f;
-  const float rmin = (lo < 0.0f) ? lo : 0.0f;
-  const float rmax = (hi > 0.0f) ? hi : 0.0f;
-  const float scale = (rmin == rmax) ? 1.0f : __fdiv_rn(255.0f, __fsub_rn(rmax, rmin));
-  const float recip = (scale != 0.0f) ? __fdiv_rn(1.0f, scale) : 0.0f;
-  const float dmin = __fmul_rn(rmin, scale);
-  const float dmax = __fmul_rn(rmax, scale);
-  const float err_min = __fadd_rn(qmin, dmin);
-  const float err_max = __fadd_rn(qmax, dmax);
-  float zpf = (__fadd_rn(err_min, err_max) > 0.0f) ? __fsub_rn(qmin, dmin) : __fsub_rn(qmax, dmax);
-  zpf = fminf(fmaxf(zpf, qmin), qmax);
-  const int zp = __float2int_rn(zpf);  // nearest even, as lrintf in the default mode
+  const RowQuant p = row_quant_params(lo, hi);
+  const int zp = p.zp;
 
   if (t == 0) {
-    recip_out[m] = recip;
+    recip_out[m] = p.recip;
     negzp_out[m] = -zp;
   }
 
@@ -78,17 +56,10 @@ __global__ __launch_bounds__(kLhsThreads) void quant_lhs_kernel(
     const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
     int q[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      int r = (int)roundf(__fmul_rn(f[e], scale)) + zp;  // |x*scale| <= 255: the cast is safe
-      r = r < -128 ? -128 : r;
-      r = r > 127 ? 127 : r;
-      q[e] = r;
-    }
+    for (int e = 0; e < 8; ++e) q[e] = quant_one(f[e], p);
     uint2 packed;
-    packed.x = (uint32_t)(q[0] & 0xFF) | ((uint32_t)(q[1] & 0xFF) << 8) |
-               ((uint32_t)(q[2] & 0xFF) << 16) | ((uint32_t)(q[3] & 0xFF) << 24);
-    packed.y = (uint32_t)(q[4] & 0xFF) | ((uint32_t)(q[5] & 0xFF) << 8) |
-               ((uint32_t)(q[6] & 0xFF) << 16) | ((uint32_t)(q[7] & 0xFF) << 24);
+    packed.x = pack4(q);
+    packed.y = pack4(q + 4);
     *reinterpret_cast<uint2*>(dst + i) = packed;
     if (ah) {
       // a_q - zp lies in [-255, 255]: exact in f16. Stored in the order a weight dword unpacks.

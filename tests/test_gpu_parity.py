@@ -173,6 +173,25 @@ def test_gemv_every_m(pkg, orc, m):
     assert max_abs_rel(y, ref) <= TIGHT
 
 
+@pytest.mark.parametrize("m,k,n", [(1, 1536, 8960), (8, 1536, 256), (1, 8960, 1536), (3, 5120, 1280),
+                                   (2, 64, 40), (8, 32, 16)])
+def test_fused_decode_kernel_equals_two_step_path(pkg, orc, m, k, n):
+    # w4a32_matmul quantises inside the decode kernel when M*K is small; the two-step path
+    # (w4a32_quant_lhs, then the GEMV on the workspace) must give the same bits, and the
+    # quantised rows it exports must be the oracle's
+    w = make_weights(n, k, seed=k + n)
+    x = make_acts(m, k, seed=m, outlier_frac=0.3)
+    bias = bias_for(n, True)
+    packed = pkg.quant_pack_rhs(dev(w), dev(bias))
+    xd = dev(x)
+    fused = host(pkg.matmul(xd, packed, n))
+    ws = pkg.quant_lhs(xd)
+    two_step = host(pkg.matmul_quantized(ws, packed, m, k, n, kernel=pkg.KERNEL_GEMV))
+    assert np.array_equal(fused, two_step)
+    u4, sc = orc.quant_rhs(w)
+    assert max_abs_rel(fused, orc.linear(x, u4, sc, bias=bias, threads=4)) <= TIGHT
+
+
 @pytest.mark.parametrize("m", [1, 8])
 def test_gemv_lm_head(pkg, orc, m):
     name, k, n, has_bias = LM_HEAD
