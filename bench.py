@@ -170,8 +170,8 @@ def main():
             "gate_proj_M512_weight_bytes": gate.bytes[1] - 1 * gate.K * 4 - 1 * gate.N * 4}}))
         return
 
-    # The whole op per decoder Linear is ONE kernel (gemv_fused_kernel); the step is 196
-    # launches of it plus lm_head (row-quant kernel + product kernel).
+    # The whole op per Linear is ONE kernel: gemv_fused_kernel for the 196 decoder Linears,
+    # gemv_wide_kernel (one wavefront per tile row) for lm_head.
     ms_step, wall_ms = timed(whole_op_pass, args.steps, args.warmup, use_graph)
     n_launch = len(step_linears)
     roof_avg_us = ms_step * 1e3 / n_launch
@@ -180,7 +180,7 @@ def main():
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                 "kernel": "gemv_fused_kernel<1,R> (R=1 for K=1536, R=2 for K=8960); lm_head runs "
-                          "quant_lhs_kernel + gemv_q_kernel<1>",
+                          "gemv_wide_kernel<1,true>",
                 "launches_per_step": n_launch, "avg_launch_us": round(roof_avg_us, 3),
                 "algorithmic_bytes_per_launch": int(roof_bytes),
                 "note": "average over the step's 197 launches (28 x 7 decoder shapes + lm_head), "
@@ -206,7 +206,12 @@ def main():
     reps = 20
     with torch.cuda.stream(stream):
         for idx, (name, K, N, b) in enumerate(LAYER_LINEARS + [LM_HEAD]):
-            lins = [lm_head] if name == "lm_head" else [layer[idx] for layer in layers]
+            if name == "lm_head":
+                # three copies, 396 MB in all, so that no repetition finds its weights in the
+                # 256 MB Infinity Cache
+                lins = [lm_head] + [Linear(pkg, torch, *LM_HEAD, gen) for _ in range(2)]
+            else:
+                lins = [layer[idx] for layer in layers]
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             for l in lins:
                 L.w4a32_matmul(y_by_n[N].data_ptr(), x_by_k[K].data_ptr(), l.packed.data_ptr(),
@@ -222,7 +227,7 @@ def main():
             gbs = lins[0].bytes[1] / (us * 1e-6) / 1e9
             per_shape[name] = {"us": round(us, 2), "GBps": round(gbs, 1),
                                "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 3),
-                               "note": ("one buffer, 132 MB (half of the 256 MB Infinity Cache)"
+                               "note": ("rotating over 3 weight buffers (396 MB)"
                                         if name == "lm_head" else "rotating over 28 weight buffers")}
     extra["decode_per_shape"] = per_shape
 

@@ -9,6 +9,11 @@
 // A wavefront's 128-bit-per-lane load is one whole 1 KiB tile. The first chunk is requested
 // before anything else happens, the next one before the current one is consumed.
 //
+// For very wide layers (N >= 32768, e.g. a vocabulary projection) gemv_wide_kernel gives every
+// WAVEFRONT whole tile rows instead: it keeps four chunk loads in flight, needs no cross-wavefront
+// reduction and therefore no barrier after the activations are staged - that is the shape where
+// the kernel is genuinely bandwidth-bound.
+//
 // Two entry kernels share the loop:
 //   gemv_q_kernel      activations already quantised (workspace of w4a32_quant_lhs)
 //   gemv_fused_kernel  quantises the f32 rows itself: every workgroup recomputes the row
@@ -20,6 +25,8 @@
 // Arithmetic per 8 weights (one dword): two mask ops give int8 vectors of 16*q, two
 // v_dot4_i32_i8 give 16 * sum a_q*q exactly, one cvt + one fma apply the block scale in f32.
 // The 1/16 and the activation offset (off * rsum[n]) are folded in once per output.
+#include <algorithm>
+
 #include "w4a32_internal.h"
 #include "w4a32_quant_math.h"
 
@@ -334,19 +341,207 @@ static hipError_t launch_fused_m(float* y, const float* x, int ldx, const uint8_
   return hipGetLastError();
 }
 
+// ----------------------------------------------------------------------------------------
+// Wide layers: one wavefront per tile row.
+// ----------------------------------------------------------------------------------------
+constexpr int kWideWaves = 4;        // wavefronts per workgroup
+constexpr int kWideMinTiles = 2048;  // tile rows from which this kernel is used (N >= 32768)
+constexpr int kWideDepth = 4;        // chunk loads a wavefront keeps in flight
+
+// kFused: quantise x (f32, K <= 8 * 64 * kWideWaves so one group of 8 per thread and row
+// suffices) into LDS first; otherwise copy the already quantised rows from the workspace.
+template <int M, bool kFused>
+__global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
+    float* __restrict__ y, const float* __restrict__ x, int ldx, const int8_t* __restrict__ aq,
+    const float* __restrict__ recip, const int32_t* __restrict__ negzp,
+    const uint8_t* __restrict__ packed, int N, int K, int NT, int KC, const float* __restrict__ rsum,
+    const float* __restrict__ bias) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  const int Kp = KC * kTileK;
+  int8_t* s_a = reinterpret_cast<int8_t*>(smem);                   // [M][Kp]
+  float* s_mm = reinterpret_cast<float*>(smem + (size_t)M * Kp);   // [kWideWaves][M][2] or params
+
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int g = lane >> 4, j = lane & 15;
+  const int wave_global = blockIdx.x * kWideWaves + wave;
+  const int wave_stride = gridDim.x * kWideWaves;
+
+  float recip_m[M];
+  int negzp_m[M];
+  if (kFused) {
+    const int groups = K >> 3;
+    float xv[M][8];
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      float lo = 3.402823466e+38f, hi = -3.402823466e+38f;
+      if ((int)threadIdx.x < groups) {
+        const float* src = x + (size_t)m * ldx + 8 * threadIdx.x;
+        const float4 v0 = *reinterpret_cast<const float4*>(src);
+        const float4 v1 = *reinterpret_cast<const float4*>(src + 4);
+        const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          xv[m][e] = f[e];
+          lo = fminf(lo, f[e]);
+          hi = fmaxf(hi, f[e]);
+        }
+      }
+      lo = wave_minmax<false>(lo);
+      hi = wave_minmax<true>(hi);
+      if (lane == 0) {
+        s_mm[(wave * M + m) * 2 + 0] = lo;
+        s_mm[(wave * M + m) * 2 + 1] = hi;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      float lo = 3.402823466e+38f, hi = -3.402823466e+38f;
+#pragma unroll
+      for (int w = 0; w < kWideWaves; ++w) {
+        lo = fminf(lo, s_mm[(w * M + m) * 2 + 0]);
+        hi = fmaxf(hi, s_mm[(w * M + m) * 2 + 1]);
+      }
+      const RowQuant p = row_quant_params(lo, hi);
+      recip_m[m] = p.recip;
+      negzp_m[m] = -p.zp;
+      if ((int)threadIdx.x < (Kp >> 3)) {
+        uint2 out = make_uint2(0, 0);
+        if ((int)threadIdx.x < groups) {
+          int q[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) q[e] = quant_one(xv[m][e], p);
+          out.x = pack4(q);
+          out.y = pack4(q + 4);
+        }
+        *reinterpret_cast<uint2*>(s_a + (size_t)m * Kp + 8 * threadIdx.x) = out;
+      }
+    }
+  } else {
+    const int vec_per_row = Kp / 16;
+    for (int v = threadIdx.x; v < M * vec_per_row; v += blockDim.x) {
+      const int m = v / vec_per_row, c = v % vec_per_row;
+      uint4 val = make_uint4(0, 0, 0, 0);
+      if (16 * c < K) val = *reinterpret_cast<const uint4*>(aq + (size_t)m * K + 16 * c);
+      *reinterpret_cast<uint4*>(s_a + (size_t)m * Kp + 16 * c) = val;
+    }
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      recip_m[m] = recip[m];
+      negzp_m[m] = negzp[m];
+    }
+  }
+  __syncthreads();
+
+  for (int nt = wave_global; nt < NT; nt += wave_stride) {
+    const uint8_t* tiles = packed + (size_t)nt * KC * kTileBytes;
+    const int n = kTileRows * nt + j;
+    float rs = 0.0f, bs = 0.0f;
+    if (lane < 16 && n < N) {
+      rs = rsum[n];
+      bs = bias[n];
+    }
+    float acc[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m) acc[m] = 0.0f;
+
+    for (int kc0 = 0; kc0 < KC; kc0 += kWideDepth) {
+      uint4 wq[kWideDepth];
+      uint2 sc[kWideDepth];
+#pragma unroll
+      for (int i = 0; i < kWideDepth; ++i) {
+        // chunks past the end re-read the last one; their contribution is masked below
+        const int kc = kc0 + i < KC ? kc0 + i : KC - 1;
+        wq[i] = *reinterpret_cast<const uint4*>(tiles + (size_t)kc * kTileBytes + 16 * lane);
+        sc[i] = *reinterpret_cast<const uint2*>(tiles + (size_t)kc * kTileBytes + kTileQBytes + 8 * j);
+      }
+#pragma unroll
+      for (int i = 0; i < kWideDepth; ++i) {
+        if (kc0 + i < KC) {
+          const uint32_t wv[4] = {wq[i].x, wq[i].y, wq[i].z, wq[i].w};
+          const float sv[4] = {__uint_as_float(sc[i].x << 16), __uint_as_float(sc[i].x & 0xFFFF0000u),
+                               __uint_as_float(sc[i].y << 16), __uint_as_float(sc[i].y & 0xFFFF0000u)};
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            const int lo = (int)((wv[d] << 4) & 0xF0F0F0F0u);
+            const int hi = (int)(wv[d] & 0xF0F0F0F0u);
+            const int8_t* a_base = s_a + kTileK * (kc0 + i) + kBlockLen * d + 8 * g;
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+              const int2 a = *reinterpret_cast<const int2*>(a_base + (size_t)m * Kp);
+              int dot = __builtin_amdgcn_sdot4(a.x, lo, 0, false);
+              dot = __builtin_amdgcn_sdot4(a.y, hi, dot, false);
+              acc[m] = __fmaf_rn((float)dot, sv[d], acc[m]);
+            }
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      acc[m] += __shfl_xor(acc[m], 16, 64);
+      acc[m] += __shfl_xor(acc[m], 32, 64);
+    }
+    if (lane < 16 && n < N) {
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        float v = __fmaf_rn((float)negzp_m[m], rs, acc[m] * 0.0625f);
+        v = __fmaf_rn(v, recip_m[m], bs);
+        v = fminf(fmaxf(v, -3.402823466e+38f), 3.402823466e+38f);
+        y[(size_t)m * N + n] = v;
+      }
+    }
+  }
+}
+
+template <int M, bool kFused>
+static hipError_t launch_wide(float* y, const float* x, int ldx, const uint8_t* ws,
+                              const uint8_t* packed, int K, int N, hipStream_t s) {
+  const WeightGeom g = weight_geom(N, K);
+  const WsGeom w = ws_geom(M, K);
+  const size_t lds = (size_t)M * g.Kp + (size_t)kWideWaves * M * 2 * sizeof(float);
+  auto kern = gemv_wide_kernel<M, kFused>;
+  static bool raised = false;
+  if (hipError_t e = raise_lds_limit(kern, lds, &raised); e != hipSuccess) return e;
+  // 4 workgroups of 4 wavefronts per CU; every wavefront then walks NT / 4096 tile rows
+  const int grid = std::min((g.NT + kWideWaves - 1) / kWideWaves, 1024);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * kWideWaves), lds, s, y, x, ldx,
+                     ws ? reinterpret_cast<const int8_t*>(ws + w.aq_off) : nullptr,
+                     ws ? reinterpret_cast<const float*>(ws + w.scale_off) : nullptr,
+                     ws ? reinterpret_cast<const int32_t*>(ws + w.off_off) : nullptr, packed, N, K,
+                     g.NT, g.KC, reinterpret_cast<const float*>(packed + g.rsum_off),
+                     reinterpret_cast<const float*>(packed + g.bias_off));
+  return hipGetLastError();
+}
+
+static bool wide_applies(int K, int N) {
+  (void)K;
+  return (N + kTileRows - 1) / kTileRows >= kWideMinTiles;
+}
+
+#define W4_DISPATCH_M(CALL)   \
+  switch (M) {               \
+    case 1: return CALL(1);  \
+    case 2: return CALL(2);  \
+    case 3: return CALL(3);  \
+    case 4: return CALL(4);  \
+    case 5: return CALL(5);  \
+    case 6: return CALL(6);  \
+    case 7: return CALL(7);  \
+    case 8: return CALL(8);  \
+    default: return hipErrorInvalidValue; \
+  }
+
 hipError_t launch_gemv(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                        hipStream_t s) {
-  switch (M) {
-    case 1: return launch_gemv_m<1>(y, ws, packed, K, N, s);
-    case 2: return launch_gemv_m<2>(y, ws, packed, K, N, s);
-    case 3: return launch_gemv_m<3>(y, ws, packed, K, N, s);
-    case 4: return launch_gemv_m<4>(y, ws, packed, K, N, s);
-    case 5: return launch_gemv_m<5>(y, ws, packed, K, N, s);
-    case 6: return launch_gemv_m<6>(y, ws, packed, K, N, s);
-    case 7: return launch_gemv_m<7>(y, ws, packed, K, N, s);
-    case 8: return launch_gemv_m<8>(y, ws, packed, K, N, s);
-    default: return hipErrorInvalidValue;
+  if (wide_applies(K, N)) {
+#define W4_CALL(m) (launch_wide<m, false>(y, nullptr, 0, ws, packed, K, N, s))
+    W4_DISPATCH_M(W4_CALL)
+#undef W4_CALL
   }
+#define W4_CALL(m) (launch_gemv_m<m>(y, ws, packed, K, N, s))
+  W4_DISPATCH_M(W4_CALL)
+#undef W4_CALL
 }
 
 // Row groups (of 8 k) per thread the fused kernel needs: 1 if the padded row fits one pass of
@@ -359,31 +554,28 @@ static int fused_groups_per_thread(int K) {
 
 bool gemv_fused_applies(int M, int K, int N) {
   // Every workgroup re-reads and re-quantises the M rows. That is cheaper than a second kernel
-  // launch while the rows are small next to the workgroup's weights, each thread can hold its
-  // share of them in registers, and a CU runs only a few workgroups in a row (measured on
-  // MI355X: at N = 151936 the two-kernel path is 1.7x faster, at N <= 8960 the fused one wins).
-  if (M < 1 || M > kGemvMaxM || (long)M * K > 16384 || N > 32768) return false;
+  // launch while the rows are small next to the workgroup's weights and each thread can hold its
+  // share of them in registers.
+  if (M < 1 || M > kGemvMaxM || (long)M * K > 16384) return false;
+  if (wide_applies(K, N)) return K <= 8 * 64 * kWideWaves;  // one group of 8 per thread and row
   const int r = fused_groups_per_thread(K);
   return r == 1 || (r == 2 && M == 1);
 }
 
 hipError_t launch_gemv_fused(float* y, const float* x, int ldx, const uint8_t* packed, int M, int K,
                              int N, hipStream_t s) {
+  if (wide_applies(K, N)) {
+#define W4_CALL(m) (launch_wide<m, true>(y, x, ldx, nullptr, packed, K, N, s))
+    W4_DISPATCH_M(W4_CALL)
+#undef W4_CALL
+  }
   if (fused_groups_per_thread(K) == 2) {
     if (M != 1) return hipErrorInvalidValue;
     return launch_fused_m<1, 2>(y, x, ldx, packed, K, N, s);
   }
-  switch (M) {
-    case 1: return launch_fused_m<1, 1>(y, x, ldx, packed, K, N, s);
-    case 2: return launch_fused_m<2, 1>(y, x, ldx, packed, K, N, s);
-    case 3: return launch_fused_m<3, 1>(y, x, ldx, packed, K, N, s);
-    case 4: return launch_fused_m<4, 1>(y, x, ldx, packed, K, N, s);
-    case 5: return launch_fused_m<5, 1>(y, x, ldx, packed, K, N, s);
-    case 6: return launch_fused_m<6, 1>(y, x, ldx, packed, K, N, s);
-    case 7: return launch_fused_m<7, 1>(y, x, ldx, packed, K, N, s);
-    case 8: return launch_fused_m<8, 1>(y, x, ldx, packed, K, N, s);
-    default: return hipErrorInvalidValue;
-  }
+#define W4_CALL(m) (launch_fused_m<m, 1>(y, x, ldx, packed, K, N, s))
+  W4_DISPATCH_M(W4_CALL)
+#undef W4_CALL
 }
 
 }  // namespace w4
