@@ -365,6 +365,23 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
   const int g = lane >> 4, j = lane & 15;
   const int wave_global = blockIdx.x * kWideWaves + wave;
   const int wave_stride = gridDim.x * kWideWaves;
+  const int batches = (KC + kWideDepth - 1) / kWideDepth;  // per tile row
+
+  // Batch (nt, b) = chunks b*kWideDepth .. +kWideDepth-1 of tile row nt; chunks past the end
+  // re-read the last one and are masked out when consumed.
+  auto load_batch = [&](int nt, int b, uint4 (&wq)[kWideDepth], uint2 (&sc)[kWideDepth]) {
+    const uint8_t* tiles = packed + (size_t)nt * KC * kTileBytes;
+#pragma unroll
+    for (int i = 0; i < kWideDepth; ++i) {
+      const int kc = b * kWideDepth + i < KC ? b * kWideDepth + i : KC - 1;
+      wq[i] = *reinterpret_cast<const uint4*>(tiles + (size_t)kc * kTileBytes + 16 * lane);
+      sc[i] = *reinterpret_cast<const uint2*>(tiles + (size_t)kc * kTileBytes + kTileQBytes + 8 * j);
+    }
+  };
+  // The first batch is requested before the activations are touched.
+  uint4 wq_cur[kWideDepth];
+  uint2 sc_cur[kWideDepth];
+  if (wave_global < NT) load_batch(wave_global, 0, wq_cur, sc_cur);
 
   float recip_m[M];
   int negzp_m[M];
@@ -434,7 +451,6 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
   __syncthreads();
 
   for (int nt = wave_global; nt < NT; nt += wave_stride) {
-    const uint8_t* tiles = packed + (size_t)nt * KC * kTileBytes;
     const int n = kTileRows * nt + j;
     float rs = 0.0f, bs = 0.0f;
     if (lane < 16 && n < N) {
@@ -445,27 +461,37 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
 #pragma unroll
     for (int m = 0; m < M; ++m) acc[m] = 0.0f;
 
-    for (int kc0 = 0; kc0 < KC; kc0 += kWideDepth) {
-      uint4 wq[kWideDepth];
-      uint2 sc[kWideDepth];
+    for (int b = 0; b < batches; ++b) {
+      // request the next batch (of this tile row, or the first of the next one) ...
+      uint4 wq_nxt[kWideDepth];
+      uint2 sc_nxt[kWideDepth];
+      const bool last = b + 1 == batches;
+      const int nt_n = last ? nt + wave_stride : nt;
+      const int b_n = last ? 0 : b + 1;
+      if (nt_n < NT) {
+        load_batch(nt_n, b_n, wq_nxt, sc_nxt);
+      } else {
 #pragma unroll
-      for (int i = 0; i < kWideDepth; ++i) {
-        // chunks past the end re-read the last one; their contribution is masked below
-        const int kc = kc0 + i < KC ? kc0 + i : KC - 1;
-        wq[i] = *reinterpret_cast<const uint4*>(tiles + (size_t)kc * kTileBytes + 16 * lane);
-        sc[i] = *reinterpret_cast<const uint2*>(tiles + (size_t)kc * kTileBytes + kTileQBytes + 8 * j);
+        for (int i = 0; i < kWideDepth; ++i) {
+          wq_nxt[i] = make_uint4(0, 0, 0, 0);
+          sc_nxt[i] = make_uint2(0, 0);
+        }
       }
+      // ... then multiply the current one
 #pragma unroll
       for (int i = 0; i < kWideDepth; ++i) {
-        if (kc0 + i < KC) {
-          const uint32_t wv[4] = {wq[i].x, wq[i].y, wq[i].z, wq[i].w};
-          const float sv[4] = {__uint_as_float(sc[i].x << 16), __uint_as_float(sc[i].x & 0xFFFF0000u),
-                               __uint_as_float(sc[i].y << 16), __uint_as_float(sc[i].y & 0xFFFF0000u)};
+        const int kc = b * kWideDepth + i;
+        if (kc < KC) {
+          const uint32_t wv[4] = {wq_cur[i].x, wq_cur[i].y, wq_cur[i].z, wq_cur[i].w};
+          const float sv[4] = {__uint_as_float(sc_cur[i].x << 16),
+                               __uint_as_float(sc_cur[i].x & 0xFFFF0000u),
+                               __uint_as_float(sc_cur[i].y << 16),
+                               __uint_as_float(sc_cur[i].y & 0xFFFF0000u)};
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
             const int lo = (int)((wv[d] << 4) & 0xF0F0F0F0u);
             const int hi = (int)(wv[d] & 0xF0F0F0F0u);
-            const int8_t* a_base = s_a + kTileK * (kc0 + i) + kBlockLen * d + 8 * g;
+            const int8_t* a_base = s_a + kTileK * kc + kBlockLen * d + 8 * g;
 #pragma unroll
             for (int m = 0; m < M; ++m) {
               const int2 a = *reinterpret_cast<const int2*>(a_base + (size_t)m * Kp);
@@ -475,6 +501,11 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
             }
           }
         }
+      }
+#pragma unroll
+      for (int i = 0; i < kWideDepth; ++i) {
+        wq_cur[i] = wq_nxt[i];
+        sc_cur[i] = sc_nxt[i];
       }
     }
 #pragma unroll
