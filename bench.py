@@ -5,7 +5,9 @@ A "step" is one decode token's worth of W4A32 Linears at M=1 on Qwen2-1.5B shape
 x {q, k, v, o, gate, up, down} + lm_head, every layer with its own weights (868 MB of
 nibbles+scales per step, more than the 256 MB Infinity Cache, so weights come from HBM as
 they do in real decoding). Each Linear is the whole op (per-row int8 quantisation of the
-activations + the product), exactly what the operator boundary runs per call.
+activations + the product); Linears that take the same input (q,k,v and gate,up) are issued
+as one grouped call, as a decoder would. `extra.one_launch_per_linear` is the same pass with
+one call per Linear.
 
 Prints ONE JSON line. `value` = algorithmic bytes of the step / time per step (GB/s), inputs
 resident in HBM. `roofline` = the decode kernel (gemv_fused_kernel: row quantisation + product
@@ -111,6 +113,32 @@ def main():
             if rc:
                 raise pkg.W4A32Error(f"w4a32_matmul({l.name}) -> {rc}")
 
+    # The same pass as the decoder issues it: Linears that take the same input go out together
+    # (q,k,v on the attention input; gate,up on the MLP input), the others alone.
+    import ctypes
+    y_extra = {("k", 256): torch.empty((1, 256), device="cuda"), ("up", 8960): torch.empty((1, 8960), device="cuda")}
+
+    def group_args(lins, ys):
+        cnt = len(lins)
+        return ((ctypes.c_void_p * cnt)(*[t.data_ptr() for t in ys]),
+                (ctypes.c_void_p * cnt)(*[l.packed.data_ptr() for l in lins]),
+                (ctypes.c_int * cnt)(*[l.N for l in lins]), cnt)
+
+    grouped_calls = []
+    for layer in layers:
+        q, k, v, o, gate, up, down = layer
+        grouped_calls.append((group_args([q, k, v], [y_by_n[1536], y_by_n[256], y_extra[("k", 256)]]), 1536))
+        grouped_calls.append((group_args([o], [y_by_n[1536]]), 1536))
+        grouped_calls.append((group_args([gate, up], [y_by_n[8960], y_extra[("up", 8960)]]), 1536))
+        grouped_calls.append((group_args([down], [y_by_n[1536]]), 8960))
+    grouped_calls.append((group_args([lm_head], [y_by_n[151936]]), 1536))
+
+    def grouped_pass():
+        for (ya, pa, na, cnt), K in grouped_calls:
+            rc = L.w4a32_matmul_grouped(ya, x_by_k[K].data_ptr(), pa, na, cnt, ws_by_k[K].data_ptr(), 1, K, sptr)
+            if rc:
+                raise pkg.W4A32Error(f"w4a32_matmul_grouped -> {rc}")
+
     def product_only_pass():
         for l in step_linears:
             rc = L.w4a32_matmul_quantized(y_by_n[l.N].data_ptr(), ws_by_k[l.K].data_ptr(),
@@ -170,10 +198,10 @@ def main():
             "gate_proj_M512_weight_bytes": gate.bytes[1] - 1 * gate.K * 4 - 1 * gate.N * 4}}))
         return
 
-    # The whole op per Linear is ONE kernel: gemv_fused_kernel for the 196 decoder Linears,
-    # gemv_wide_kernel (one wavefront per tile row) for lm_head.
-    ms_step, wall_ms = timed(whole_op_pass, args.steps, args.warmup, use_graph)
-    n_launch = len(step_linears)
+    # Every call is ONE kernel (row quantisation inside): gemv_fused_kernel for the decoder
+    # Linears (q,k,v in one launch, gate,up in one launch), gemv_wide_kernel for lm_head.
+    ms_step, wall_ms = timed(grouped_pass, args.steps, args.warmup, use_graph)
+    n_launch = len(grouped_calls)
     roof_avg_us = ms_step * 1e3 / n_launch
     roof_bytes = step_bytes / n_launch
     achieved = roof_bytes / (roof_avg_us * 1e-6) / 1e9
@@ -183,14 +211,16 @@ def main():
                           "gemv_wide_kernel<1,true>",
                 "launches_per_step": n_launch, "avg_launch_us": round(roof_avg_us, 3),
                 "algorithmic_bytes_per_launch": int(roof_bytes),
-                "note": "average over the step's 197 launches (28 x 7 decoder shapes + lm_head), "
+                "note": "average over the step's 113 launches (28 x {qkv, o, gate+up, down} + lm_head), "
                         "launch period inside a HIP graph; per-shape figures are in extra"}
     if args.roofline_only:
         print(json.dumps({"roofline": roofline}))
         return
 
     value = step_bytes / (ms_step * 1e-3) / 1e9
-    # the same products on activations quantised once (w4a32_quant_lhs + w4a32_matmul_quantized)
+    # the same Linears one launch each (what the per-op boundary does without grouping) ...
+    ms_single, _ = timed(whole_op_pass, args.steps, args.warmup, use_graph)
+    # ... and the products alone on activations quantised once
     with torch.cuda.stream(stream):
         for K in ws_by_k:
             L.w4a32_quant_lhs(x_by_k[K].data_ptr(), 1, K, K, ws_by_k[K].data_ptr(), sptr)
@@ -199,6 +229,8 @@ def main():
 
     extra = {"decode_linears_tokens_per_s": round(1e3 / ms_step, 1),
              "wall_ms_per_step": round(wall_ms, 4), "graph": use_graph,
+             "one_launch_per_linear": {"launches": len(step_linears), "ms_per_step": round(ms_single, 4),
+                                       "GBps": round(step_bytes / (ms_single * 1e-3) / 1e9, 1)},
              "product_only_ms_per_step": round(ms_prod, 4)}
 
     # ---- per-shape decode figures (product kernel, weights rotated over the 28 layers)
@@ -322,9 +354,11 @@ def main():
         "data": "synthetic (torch cuda generator seed 0, N(0,0.02^2) f32 weights quantised to 4-bit "
                 "block-32 by the library; activations N(0,1) seed 1)",
         "config": {"workload": "config 2 at M=1: Qwen2-1.5B decode Linears, 28 layers x "
-                               "{q,k,v,o,gate,up,down} + lm_head, distinct weights per layer, "
-                               "whole op per Linear (row quant + product)",
-                   "M": 1, "launched_linears": n_launch, "algorithmic_bytes_per_step": step_bytes},
+                               "{q,k,v,o,gate,up,down} + lm_head, distinct weights per layer, whole op "
+                               "(row quant + product) per Linear; Linears that share an input (q,k,v; "
+                               "gate,up) are issued as one grouped call",
+                   "M": 1, "linears": len(step_linears), "launches": n_launch,
+                   "algorithmic_bytes_per_step": step_bytes},
         "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
     }
     print(json.dumps(out))

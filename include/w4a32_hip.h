@@ -124,6 +124,17 @@ int w4a32_matmul_quantized_ex(float* d_y, const void* d_ws, const void* d_packed
 int w4a32_matmul(float* d_y, const float* d_x, const void* d_packed, void* d_ws, int M, int K,
                  int N, void* stream);
 
+/* Several Linears applied to the SAME activation rows, in one launch where the sizes allow:
+ * d_y, d_packed and N are HOST arrays of `count` (<= W4A32_MAX_GROUP) entries; Linear i has blob
+ * d_packed[i] for [N[i]][K] and writes d_y[i][M][N[i]]. Stands in for the consecutive matmul
+ * calls the model code makes on one input - q_proj/k_proj/v_proj and gate_proj/up_proj
+ * (mllm/Models/ds_qwen2/modeling_ds_qwen2.hpp:47-54, 106-155) - each of which would otherwise
+ * quantise the same rows again (kai_linear.cpp:358-362). Results are bit-identical to calling
+ * w4a32_matmul once per Linear. */
+#define W4A32_MAX_GROUP 4
+int w4a32_matmul_grouped(float* const* d_y, const float* d_x, const void* const* d_packed,
+                         const int* N, int count, void* d_ws, int M, int K, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

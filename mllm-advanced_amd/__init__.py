@@ -39,6 +39,7 @@ ABI = {
     "w4a32_matmul_quantized": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a32_matmul_quantized_ex": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp]),
     "w4a32_matmul": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
+    "w4a32_matmul_grouped": (_ci, [_vp, _vp, _vp, _vp, _ci, _vp, _ci, _ci, _vp]),
 }
 
 
@@ -192,3 +193,20 @@ def matmul(x, packed, N, ws=None, out=None):
     _check(lib().w4a32_matmul(_ptr(y), _ptr(x), _ptr(packed), _ptr(ws), M, K, N, _stream()),
            "w4a32_matmul")
     return y
+
+
+def matmul_grouped(x, packed_list, n_list, ws=None):
+    """Several Linears on the same rows x [M,K]; returns one output tensor per Linear."""
+    import torch
+
+    M, K = x.shape
+    cnt = len(packed_list)
+    if ws is None:
+        ws = _dev_empty(workspace_bytes(M, K))
+    ys = [torch.empty((M, n), dtype=torch.float32, device="cuda") for n in n_list]
+    y_arr = (ctypes.c_void_p * cnt)(*[y.data_ptr() for y in ys])
+    p_arr = (ctypes.c_void_p * cnt)(*[p.data_ptr() for p in packed_list])
+    n_arr = (ctypes.c_int * cnt)(*n_list)
+    _check(lib().w4a32_matmul_grouped(y_arr, _ptr(x), p_arr, n_arr, cnt, _ptr(ws), M, K, _stream()),
+           "w4a32_matmul_grouped")
+    return ys

@@ -168,4 +168,28 @@ int w4a32_matmul(float* d_y, const float* d_x, const void* d_packed, void* d_ws,
   return w4a32_matmul_quantized(d_y, d_ws, d_packed, M, K, N, stream);
 }
 
+int w4a32_matmul_grouped(float* const* d_y, const float* d_x, const void* const* d_packed,
+                         const int* N, int count, void* d_ws, int M, int K, void* stream) {
+  if (!d_y || !d_x || !d_packed || !N || !d_ws) return W4A32_EINVAL;
+  if (count < 1 || count > W4A32_MAX_GROUP || M <= 0) return W4A32_EINVAL;
+  for (int i = 0; i < count; ++i) {
+    if (int e = shape_ok(N[i], K)) return e;
+    if (!d_y[i] || !d_packed[i]) return W4A32_EINVAL;
+    if (!aligned(d_packed[i], 16) || !aligned(d_y[i], 4)) return W4A32_EINVAL;
+  }
+  if (!aligned(d_x, 16) || !aligned(d_ws, 256)) return W4A32_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (w4::gemv_group_applies(M, K, N, count)) {
+    const uint8_t* pk[W4A32_MAX_GROUP];
+    for (int i = 0; i < count; ++i) pk[i] = static_cast<const uint8_t*>(d_packed[i]);
+    return from_hip(w4::launch_gemv_group(d_y, d_x, K, pk, N, count, M, K, s));
+  }
+  // other sizes: quantise the rows once, then one product per Linear
+  if (int e = w4a32_quant_lhs(d_x, M, K, K, d_ws, stream)) return e;
+  for (int i = 0; i < count; ++i) {
+    if (int e = w4a32_matmul_quantized(d_y[i], d_ws, d_packed[i], M, K, N[i], stream)) return e;
+  }
+  return W4A32_OK;
+}
+
 }  // extern "C"

@@ -181,20 +181,63 @@ __global__ __launch_bounds__(1024) void gemv_q_kernel(
   gemv_finish<M>(y, N, nt, W, acc, s_red, recip_m, negzp_m, rsum, bias, rs, bs);
 }
 
+// Up to kMaxGroup Linears that share their activation rows (and therefore K), run by one launch:
+// workgroup b serves tile row b - first[i] of Linear i, where first[] are running sums of tile rows.
+constexpr int kMaxGroup = 4;
+struct GroupArgs {
+  const uint8_t* packed[kMaxGroup];
+  float* y[kMaxGroup];
+  int N[kMaxGroup];
+  int first[kMaxGroup + 1];  // first[i] = tile rows of Linears 0..i-1; first[count] = grid size
+  int count;
+};
+
 // Whole op in one launch: x f32 [M][K] (row stride ldx) -> y.
 // kFusedR = groups of 8 k a thread may own per row: covers K <= 8 * kFusedR * blockDim.x.
-template <int M, int kFusedR>
-__global__ __launch_bounds__(1024) void gemv_fused_kernel(
-    float* __restrict__ y, const float* __restrict__ x, int ldx, const uint8_t* __restrict__ packed,
-    int N, int K, int KC, const float* __restrict__ rsum, const float* __restrict__ bias) {
+// kGrouped = false: a single Linear, the group table is not consulted.
+template <int M, int kFusedR, bool kGrouped>
+__global__ __launch_bounds__(1024) void gemv_fused_kernel(const GroupArgs ga,
+                                                          const float* __restrict__ x, int ldx,
+                                                          int K, int KC) {
   extern __shared__ __align__(16) uint8_t smem[];
+  const uint8_t* packed = ga.packed[0];
+  float* y = ga.y[0];
+  int N = ga.N[0], nt_first = 0;
+  if (kGrouped) {
+    // Which Linear this workgroup belongs to. All four table entries are fetched first (the
+    // empty asm pins them in scalar registers) and then selected, so that the choice costs a
+    // few scalar ops instead of a second, dependent load from the argument segment.
+    const uint8_t* pk[kMaxGroup];
+    float* yy[kMaxGroup];
+    int nn[kMaxGroup], ff[kMaxGroup];
+#pragma unroll
+    for (int i = 0; i < kMaxGroup; ++i) {
+      pk[i] = ga.packed[i];
+      yy[i] = ga.y[i];
+      nn[i] = ga.N[i];
+      ff[i] = ga.first[i];
+      asm volatile("" : "+s"(pk[i]), "+s"(yy[i]), "+s"(nn[i]), "+s"(ff[i]));
+    }
+#pragma unroll
+    for (int i = 1; i < kMaxGroup; ++i) {
+      if (i < ga.count && (int)blockIdx.x >= ff[i]) {
+        packed = pk[i];
+        y = yy[i];
+        N = nn[i];
+        nt_first = ff[i];
+      }
+    }
+  }
+  const int Np = (N + kTileRows - 1) / kTileRows * kTileRows;
+  const float* rsum = reinterpret_cast<const float*>(packed + (size_t)(Np / kTileRows) * KC * kTileBytes);
+  const float* bias = rsum + Np;
   const int Kp = KC * kTileK;
   const int W = blockDim.x >> 6;
   int8_t* s_a = reinterpret_cast<int8_t*>(smem);                    // [M][Kp]
   float* s_red = reinterpret_cast<float*>(smem + (size_t)M * Kp);   // [W][M][16]
   float* s_mm = s_red + W * M * 16;                                 // [W][M][2] min, max
 
-  const int nt = blockIdx.x;
+  const int nt = (int)blockIdx.x - nt_first;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const uint8_t* tiles = packed + (size_t)nt * KC * kTileBytes;
 
@@ -326,18 +369,23 @@ static hipError_t launch_gemv_m(float* y, const uint8_t* ws, const uint8_t* pack
 }
 
 template <int M, int R>
-static hipError_t launch_fused_m(float* y, const float* x, int ldx, const uint8_t* packed, int K,
-                                 int N, hipStream_t s) {
-  const WeightGeom g = weight_geom(N, K);
-  const int W = pick_waves(g.KC);
-  const size_t lds = (size_t)M * g.Kp + (size_t)W * M * 16 * sizeof(float) +
+static hipError_t launch_fused_m(const GroupArgs& ga, const float* x, int ldx, int K, hipStream_t s) {
+  const int KC = (K + kTileK - 1) / kTileK;
+  const int Kp = KC * kTileK;
+  const int W = pick_waves(KC);
+  const size_t lds = (size_t)M * Kp + (size_t)W * M * 16 * sizeof(float) +
                      (size_t)W * M * 2 * sizeof(float);
-  auto kern = gemv_fused_kernel<M, R>;
-  static bool raised = false;
-  if (hipError_t e = raise_lds_limit(kern, lds, &raised); e != hipSuccess) return e;
-  hipLaunchKernelGGL(kern, dim3(g.NT), dim3(64 * W), lds, s, y, x, ldx, packed, N, K, g.KC,
-                     reinterpret_cast<const float*>(packed + g.rsum_off),
-                     reinterpret_cast<const float*>(packed + g.bias_off));
+  const dim3 grid(ga.first[ga.count]), block(64 * W);
+  static bool raised1 = false, raisedg = false;
+  if (ga.count == 1) {
+    auto kern = gemv_fused_kernel<M, R, false>;
+    if (hipError_t e = raise_lds_limit(kern, lds, &raised1); e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, grid, block, lds, s, ga, x, ldx, K, KC);
+  } else {
+    auto kern = gemv_fused_kernel<M, R, true>;
+    if (hipError_t e = raise_lds_limit(kern, lds, &raisedg); e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, grid, block, lds, s, ga, x, ldx, K, KC);
+  }
   return hipGetLastError();
 }
 
@@ -593,6 +641,17 @@ bool gemv_fused_applies(int M, int K, int N) {
   return r == 1 || (r == 2 && M == 1);
 }
 
+static hipError_t launch_fused_group(const GroupArgs& ga, const float* x, int ldx, int M, int K,
+                                     hipStream_t s) {
+  if (fused_groups_per_thread(K) == 2) {
+    if (M != 1) return hipErrorInvalidValue;
+    return launch_fused_m<1, 2>(ga, x, ldx, K, s);
+  }
+#define W4_CALL(m) (launch_fused_m<m, 1>(ga, x, ldx, K, s))
+  W4_DISPATCH_M(W4_CALL)
+#undef W4_CALL
+}
+
 hipError_t launch_gemv_fused(float* y, const float* x, int ldx, const uint8_t* packed, int M, int K,
                              int N, hipStream_t s) {
   if (wide_applies(K, N)) {
@@ -600,13 +659,36 @@ hipError_t launch_gemv_fused(float* y, const float* x, int ldx, const uint8_t* p
     W4_DISPATCH_M(W4_CALL)
 #undef W4_CALL
   }
-  if (fused_groups_per_thread(K) == 2) {
-    if (M != 1) return hipErrorInvalidValue;
-    return launch_fused_m<1, 2>(y, x, ldx, packed, K, N, s);
+  GroupArgs ga{};
+  ga.packed[0] = packed;
+  ga.y[0] = y;
+  ga.N[0] = N;
+  ga.first[0] = 0;
+  ga.first[1] = (N + kTileRows - 1) / kTileRows;
+  ga.count = 1;
+  return launch_fused_group(ga, x, ldx, M, K, s);
+}
+
+bool gemv_group_applies(int M, int K, const int* N, int count) {
+  if (count < 1 || count > kMaxGroup) return false;
+  for (int i = 0; i < count; ++i) {
+    if (!gemv_fused_applies(M, K, N[i]) || wide_applies(K, N[i])) return false;
   }
-#define W4_CALL(m) (launch_fused_m<m, 1>(y, x, ldx, packed, K, N, s))
-  W4_DISPATCH_M(W4_CALL)
-#undef W4_CALL
+  return true;
+}
+
+hipError_t launch_gemv_group(float* const* y, const float* x, int ldx, const uint8_t* const* packed,
+                             const int* N, int count, int M, int K, hipStream_t s) {
+  GroupArgs ga{};
+  ga.first[0] = 0;
+  for (int i = 0; i < count; ++i) {
+    ga.packed[i] = packed[i];
+    ga.y[i] = y[i];
+    ga.N[i] = N[i];
+    ga.first[i + 1] = ga.first[i] + (N[i] + kTileRows - 1) / kTileRows;
+  }
+  ga.count = count;
+  return launch_fused_group(ga, x, ldx, M, K, s);
 }
 
 }  // namespace w4

@@ -27,6 +27,10 @@ hipError_t launch_gemv(float* y, const uint8_t* ws, const uint8_t* packed, int M
 bool gemv_fused_applies(int M, int K, int N);
 hipError_t launch_gemv_fused(float* y, const float* x, int ldx, const uint8_t* packed, int M, int K,
                              int N, hipStream_t s);
+// several Linears on the same activation rows in one launch (decode sizes only)
+bool gemv_group_applies(int M, int K, const int* N, int count);
+hipError_t launch_gemv_group(float* const* y, const float* x, int ldx, const uint8_t* const* packed,
+                             const int* N, int count, int M, int K, hipStream_t s);
 hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                        int kernel, hipStream_t s);
 
