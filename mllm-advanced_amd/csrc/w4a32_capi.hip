@@ -179,6 +179,7 @@ int w4a32_matmul_grouped(float* const* d_y, const float* d_x, const void* const*
   }
   if (!aligned(d_x, 16) || !aligned(d_ws, 256)) return W4A32_EINVAL;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (count == 1) return w4a32_matmul(d_y[0], d_x, d_packed[0], d_ws, M, K, N[0], stream);
   if (w4::gemv_group_applies(M, K, N, count)) {
     const uint8_t* pk[W4A32_MAX_GROUP];
     for (int i = 0; i < count; ++i) pk[i] = static_cast<const uint8_t*>(d_packed[i]);

@@ -160,7 +160,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_f16_kernel(
     float* __restrict__ y, const _Float16* __restrict__ ah, const float* __restrict__ recip,
     const uint8_t* __restrict__ packed, const uint8_t* __restrict__ hscale,
     const float* __restrict__ rowmul, const float* __restrict__ bias, int M, int N, int K, int NT,
-    int KC) {
+    int KC, int MB, int NB, int n_major) {
   constexpr int D = kF16Depth;
   constexpr int NWAVES = WAVES_M * WAVES_N;
   constexpr int BM = 32 * WM * WAVES_M;
@@ -177,8 +177,19 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_f16_kernel(
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int g = lane >> 4, j = lane & 15;     // position inside a weight tile
   const int h = lane >> 5, i32 = lane & 31;   // position inside an MFMA operand / C tile
-  const int m0 = blockIdx.y * BM + 32 * WM * wm;
-  const int nt0 = blockIdx.x * WNT;
+  // Workgroup -> tile. The hardware deals consecutive workgroups round-robin to the 8 XCDs, each
+  // with its own L2. Workgroup b therefore takes tile (b % 8) * ceil(T / 8) + b / 8, so that an
+  // XCD owns one contiguous run of tiles; the run is ordered so that neighbours share the larger
+  // operand (n_major: all row blocks of a weight column block together, weights fetched by one
+  // XCD only; otherwise all column blocks of a row block together).
+  const int total = MB * NB;
+  const int per_xcd = (total + 7) >> 3;
+  const int tile = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+  if (tile >= total) return;  // whole workgroup: no barrier has been reached yet
+  const int mb = n_major ? tile % MB : tile / NB;
+  const int nb = n_major ? tile / MB : tile % NB;
+  const int m0 = mb * BM + 32 * WM * wm;
+  const int nt0 = nb * WNT;
   const int nstages = (K + kF16BK - 1) / kF16BK;
 
   uint4 areg[D][2][WM][2];  // [ring slot][k-block][32-row tile][slice of the block]
@@ -348,13 +359,18 @@ static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed,
   constexpr int BM = 32 * WM * WAVES_M, WNT = 2 * WN * WAVES_N;
   const WeightGeom g = weight_geom(N, K);
   const WsGeom w = ws_geom(M, K);
-  dim3 grid((g.NT + WNT - 1) / WNT, (M + BM - 1) / BM);
-  hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN>), grid,
+  const int NB = (g.NT + WNT - 1) / WNT, MB = (M + BM - 1) / BM;
+  const int grid = ((MB * NB + 7) / 8) * 8;
+  // keep together what is more expensive to fetch eight times: the f16 activations (2 bytes per
+  // element) or the packed weights (0.5625 bytes per element)
+  const int n_major = (double)M * 2.0 <= (double)N * 0.5625 ? 1 : 0;
+  hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN>), dim3(grid),
                      dim3(64 * WAVES_M * WAVES_N), 0, s, y,
                      reinterpret_cast<const _Float16*>(ws + w.ah_off),
                      reinterpret_cast<const float*>(ws + w.scale_off), packed,
                      packed + g.hscale_off, reinterpret_cast<const float*>(packed + g.rowmul_off),
-                     reinterpret_cast<const float*>(packed + g.bias_off), M, N, K, g.NT, g.KC);
+                     reinterpret_cast<const float*>(packed + g.bias_off), M, N, K, g.NT, g.KC, MB, NB,
+                     n_major);
   return hipGetLastError();
 }
 
