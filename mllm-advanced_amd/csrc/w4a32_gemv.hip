@@ -78,6 +78,8 @@ __device__ __forceinline__ void gemv_accumulate(const uint8_t* __restrict__ tile
   }
 }
 
+constexpr int kMaxWaves = 16;  // wavefronts per workgroup, at most
+
 // Cross-wavefront sum and the output transform
 //   y = (sum/16 + off * rsum[n]) * lhs_scale + bias[n], clamped to the finite f32 range.
 // When the workgroup has at least 16*M threads, thread o owns output o and already holds
@@ -100,8 +102,14 @@ __device__ __forceinline__ void gemv_finish(float* __restrict__ y, int N, int nt
     const int m = o >> 4, jj = o & 15;
     const int n = kTileRows * nt + jj;
     if (n < N) {
+      // All kMaxWaves reads are issued before the first add (a loop over W would wait for each
+      // LDS read in turn); wavefronts past W re-read the last one and add 0.
+      float part[kMaxWaves];
+#pragma unroll
+      for (int w = 0; w < kMaxWaves; ++w) part[w] = s_red[((w < W ? w : W - 1) * M + m) * 16 + jj];
       float s = 0.0f;
-      for (int w = 0; w < W; ++w) s += s_red[(w * M + m) * 16 + jj];
+#pragma unroll
+      for (int w = 0; w < kMaxWaves; ++w) s += w < W ? part[w] : 0.0f;
       float rcp = 0.0f;
       int off = 0;
 #pragma unroll
@@ -181,6 +189,17 @@ __global__ __launch_bounds__(1024) void gemv_q_kernel(
   gemv_finish<M>(y, N, nt, W, acc, s_red, recip_m, negzp_m, rsum, bias, rs, bs);
 }
 
+// Loads and stores through pointers picked from the group table must say that they address global
+// memory: the compiler no longer knows, would emit flat instructions and, because those may
+// complete out of order with global ones, wait for every outstanding load at the first use of any.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+#define W4_GLOBAL __attribute__((address_space(1)))
+template <typename T>
+__device__ __forceinline__ T load_global(const void* p) {
+  return *(const W4_GLOBAL T*)p;
+}
+
 // Up to kMaxGroup Linears that share their activation rows (and therefore K), run by one launch:
 // workgroup b serves tile row b - first[i] of Linear i, where first[] are running sums of tile rows.
 constexpr int kMaxGroup = 4;
@@ -193,10 +212,17 @@ struct GroupArgs {
 };
 
 // Whole op in one launch: x f32 [M][K] (row stride ldx) -> y.
-// kFusedR = groups of 8 k a thread may own per row: covers K <= 8 * kFusedR * blockDim.x.
+//
+// A workgroup of W wavefronts owns one tile row. Wavefront w holds its chunks w, w + W, ... (kCPW
+// of them, covering KC <= kCPW * W); all kCPW loads are requested at kernel start. Each thread owns kFusedR groups of 8 activations per row (covering
+// K <= 8 * kFusedR * blockDim.x), kept in registers from the min/max pass to the quantise pass.
 // kGrouped = false: a single Linear, the group table is not consulted.
-template <int M, int kFusedR, bool kGrouped>
-__global__ __launch_bounds__(1024) void gemv_fused_kernel(const GroupArgs ga,
+//
+// Nearly every instruction here is executed once per wavefront and depends on the one before, so
+// the kernel's duration at decode sizes is its instruction count times the issue latency: the
+// reductions use one DPP instruction per step and the quantiser four VALU instructions per value.
+template <int M, int kFusedR, bool kGrouped, int kCPW>
+__global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(const GroupArgs ga,
                                                           const float* __restrict__ x, int ldx,
                                                           int K, int KC) {
   extern __shared__ __align__(16) uint8_t smem[];
@@ -228,78 +254,81 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(const GroupArgs ga,
       }
     }
   }
-  const int Np = (N + kTileRows - 1) / kTileRows * kTileRows;
-  const float* rsum = reinterpret_cast<const float*>(packed + (size_t)(Np / kTileRows) * KC * kTileBytes);
-  const float* bias = rsum + Np;
+  const int NT = (N + kTileRows - 1) / kTileRows;
+  const float* rsum = reinterpret_cast<const float*>(packed + (size_t)NT * KC * kTileBytes);
+  const float* bias = rsum + NT * kTileRows;
   const int Kp = KC * kTileK;
   const int W = blockDim.x >> 6;
-  int8_t* s_a = reinterpret_cast<int8_t*>(smem);                    // [M][Kp]
-  float* s_red = reinterpret_cast<float*>(smem + (size_t)M * Kp);   // [W][M][16]
-  float* s_mm = s_red + W * M * 16;                                 // [W][M][2] min, max
+  int8_t* s_a = reinterpret_cast<int8_t*>(smem);                          // [M][Kp]
+  float* s_red = reinterpret_cast<float*>(smem + (size_t)M * Kp);         // [W][M][16]
+  float2* s_mm = reinterpret_cast<float2*>(s_red + W * M * 16);     // [W][M] (min, max)
 
   const int nt = (int)blockIdx.x - nt_first;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const uint8_t* tiles = packed + (size_t)nt * KC * kTileBytes;
+  const int g = lane >> 4, j = lane & 15;
 
-  uint4 wq = make_uint4(0, 0, 0, 0);
-  uint2 sc = make_uint2(0, 0);
-  if (wave < KC) {
-    wq = *reinterpret_cast<const uint4*>(tiles + (size_t)wave * kTileBytes + 16 * lane);
-    sc = *reinterpret_cast<const uint2*>(tiles + (size_t)wave * kTileBytes + kTileQBytes +
-                                         8 * (lane & 15));
-  }
-  float rs = 0.0f, bs = 0.0f;
-  {
-    const int n = kTileRows * nt + (threadIdx.x & 15);
-    if (threadIdx.x < 16 * M && n < N) {
-      rs = rsum[n];
-      bs = bias[n];
-    }
-  }
-
-  // Each thread owns up to kFusedR groups of 8 consecutive k per row (group index
-  // threadIdx.x + r*blockDim.x) and keeps them in registers from the min/max pass to the
-  // quantise pass, so x is read once. Wavefronts reduce min/max with DPP; the W partial results
-  // meet in LDS.
+  // x first (a few KB, normally in L2), then the weights, so that the min/max and quantise passes
+  // run while the weights are on their way from HBM.
   const int groups = K >> 3;
   float xv[M][kFusedR][8];
 #pragma unroll
   for (int m = 0; m < M; ++m) {
     const float* row = x + (size_t)m * ldx;
-    float lo = 3.402823466e+38f, hi = -3.402823466e+38f;
 #pragma unroll
     for (int r = 0; r < kFusedR; ++r) {
       const int c = threadIdx.x + r * blockDim.x;
-      if (c < groups) {
-        const float4 v0 = *reinterpret_cast<const float4*>(row + 8 * c);
-        const float4 v1 = *reinterpret_cast<const float4*>(row + 8 * c + 4);
-        const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+      const int cc = c < groups ? c : groups - 1;  // a duplicate of a real element: harmless for min/max
+      const float4 v0 = *reinterpret_cast<const float4*>(row + 8 * cc);
+      const float4 v1 = *reinterpret_cast<const float4*>(row + 8 * cc + 4);
+      const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          xv[m][r][e] = f[e];
-          lo = fminf(lo, f[e]);
-          hi = fmaxf(hi, f[e]);
-        }
+      for (int e = 0; e < 8; ++e) xv[m][r][e] = f[e];
+    }
+  }
+  u32x4 wq[kCPW];
+  u32x2 sc[kCPW];
+  const uint8_t* tiles = packed + (size_t)nt * KC * kTileBytes;
+#pragma unroll
+  for (int i = 0; i < kCPW; ++i) {
+    const int kc = wave + i * W < KC ? wave + i * W : KC - 1;  // masked where used
+    wq[i] = load_global<u32x4>(tiles + (size_t)kc * kTileBytes + 16 * lane);
+    sc[i] = load_global<u32x2>(tiles + (size_t)kc * kTileBytes + kTileQBytes + 8 * j);
+  }
+  // Output o = m * 16 + jj belongs to thread o when the workgroup has that many threads; its
+  // rsum / bias are requested now so the epilogue does not wait on memory.
+  constexpr int kOutputs = M * 16;
+  float rs = 0.0f, bs = 0.0f;
+  {
+    const int n = kTileRows * nt + j;
+    if (threadIdx.x < kOutputs && n < N) {
+      rs = load_global<float>(rsum + n);
+      bs = load_global<float>(bias + n);
+    }
+  }
+
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+    float lo = xv[m][0][0], hi = xv[m][0][0];
+#pragma unroll
+    for (int r = 0; r < kFusedR; ++r) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        lo = fminf(lo, xv[m][r][e]);
+        hi = fmaxf(hi, xv[m][r][e]);
       }
     }
-    lo = wave_minmax<false>(lo);
-    hi = wave_minmax<true>(hi);
-    if (lane == 0) {
-      s_mm[(wave * M + m) * 2 + 0] = lo;
-      s_mm[(wave * M + m) * 2 + 1] = hi;
-    }
+    wave_minmax_pair(lo, hi);
+    if (lane == 63) s_mm[wave * M + m] = make_float2(lo, hi);
   }
   __syncthreads();
 
   RowQuant par[M];
 #pragma unroll
   for (int m = 0; m < M; ++m) {
-    float lo = 3.402823466e+38f, hi = -3.402823466e+38f;
-    for (int w = 0; w < W; ++w) {
-      lo = fminf(lo, s_mm[(w * M + m) * 2 + 0]);
-      hi = fmaxf(hi, s_mm[(w * M + m) * 2 + 1]);
-    }
-    par[m] = row_quant_params(lo, hi);
+    // lane j of every 16-lane row fetches wavefront j's result (the last one again past W)
+    float2 v = s_mm[(j < W ? j : W - 1) * M + m];
+    row16_minmax_pair(v.x, v.y);
+    par[m] = row_quant_params(v.x, v.y);
   }
 
   // Quantise into the LDS copy; the tile padding (k >= K) is 0.
@@ -310,14 +339,8 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(const GroupArgs ga,
     for (int r = 0; r < kFusedR; ++r) {
       const int c = threadIdx.x + r * blockDim.x;
       if (c < grp_per_row) {
-        uint2 out = make_uint2(0, 0);
-        if (c < groups) {
-          int q[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) q[e] = quant_one(xv[m][r][e], par[m]);
-          out.x = pack4(q);
-          out.y = pack4(q + 4);
-        }
+        uint2 out = quant_group8(xv[m][r], par[m]);
+        if (c >= groups) out = make_uint2(0, 0);
         *reinterpret_cast<uint2*>(s_a + (size_t)m * Kp + 8 * c) = out;
       }
     }
@@ -325,15 +348,68 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(const GroupArgs ga,
   __syncthreads();
 
   float acc[M];
-  gemv_accumulate<M>(tiles, KC, Kp, s_a, wq, sc, wave, W, lane, acc);
-  float recip_m[M];
-  int negzp_m[M];
+#pragma unroll
+  for (int m = 0; m < M; ++m) acc[m] = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kCPW; ++i) {
+    const bool valid = wave + i * W < KC;
+    const int kc = valid ? wave + i * W : KC - 1;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const int8_t* a_base = s_a + kTileK * kc + kBlockLen * d + 8 * g;
+      int2 a[M];
+#pragma unroll
+      for (int m = 0; m < M; ++m) a[m] = *reinterpret_cast<const int2*>(a_base + (size_t)m * Kp);
+      const uint32_t wv = wq[i][d];
+      const uint32_t sw = sc[i][d >> 1];
+      const uint32_t sbits = valid ? ((d & 1) ? (sw & 0xFFFF0000u) : (sw << 16)) : 0u;
+      const float sv = __uint_as_float(sbits);
+      const int lo = (int)((wv << 4) & 0xF0F0F0F0u);  // 16*q at k offsets 0..3
+      const int hi = (int)(wv & 0xF0F0F0F0u);         // 16*q at k offsets 4..7
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        int dot = __builtin_amdgcn_sdot4(a[m].x, lo, 0, false);
+        dot = __builtin_amdgcn_sdot4(a[m].y, hi, dot, false);
+        acc[m] = __fmaf_rn((float)dot, sv, acc[m]);
+      }
+    }
+  }
+  // Sum the four k-groups of a row (lanes j, j+16, j+32, j+48), then across wavefronts via LDS.
 #pragma unroll
   for (int m = 0; m < M; ++m) {
-    recip_m[m] = par[m].recip;
-    negzp_m[m] = -par[m].zp;
+    float v = acc[m];
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    if (lane < 16) s_red[(wave * M + m) * 16 + lane] = v;
   }
-  gemv_finish<M>(y, N, nt, W, acc, s_red, recip_m, negzp_m, rsum, bias, rs, bs);
+  __syncthreads();
+
+  //   y = (sum/16 + off * rsum[n]) * lhs_scale + bias[n], clamped to the finite f32 range
+  const bool prefetched = blockDim.x >= kOutputs;
+  for (int o = threadIdx.x; o < kOutputs; o += blockDim.x) {
+    const int m = o >> 4;
+    const int n = kTileRows * nt + (o & 15);
+    if (n < N) {
+      float s = 0.0f;
+#pragma unroll 4
+      for (int w = 0; w < W; ++w) s += s_red[w * kOutputs + o];
+      float rcp = 0.0f;
+      int off = 0;
+#pragma unroll
+      for (int mm = 0; mm < M; ++mm) {  // compile-time indices keep the array in registers
+        if (mm == m) {
+          rcp = par[mm].recip;
+          off = -par[mm].zp;
+        }
+      }
+      const float rsn = prefetched ? rs : load_global<float>(rsum + n);
+      const float bsn = prefetched ? bs : load_global<float>(bias + n);
+      float v = __fmaf_rn((float)off, rsn, s * 0.0625f);
+      v = __fmaf_rn(v, rcp, bsn);
+      v = fminf(fmaxf(v, -3.402823466e+38f), 3.402823466e+38f);
+      *(W4_GLOBAL float*)(y + (size_t)m * N + n) = v;
+    }
+  }
 }
 
 static int pick_waves(int KC) { return KC < 16 ? KC : 16; }
@@ -368,21 +444,51 @@ static hipError_t launch_gemv_m(float* y, const uint8_t* ws, const uint8_t* pack
   return hipGetLastError();
 }
 
-template <int M, int R>
-static hipError_t launch_fused_m(const GroupArgs& ga, const float* x, int ldx, int K, hipStream_t s) {
+// Launch shape of the fused kernel: W wavefronts per workgroup, each holding CPW chunks; every
+// thread owns R groups of 8 activations per row.
+struct FusedPlan {
+  int W, CPW, R;
+};
+constexpr int kMaxCPW = 5;
+
+// Shapes that keep their chunks, activations and accumulators in registers without spilling.
+constexpr bool fused_shape_ok(int M, int cpw) { return cpw <= kMaxCPW && (M == 1 || M * cpw <= 24); }
+
+// About three chunks per wavefront: fewer wavefronts mean less dispatch time and fewer copies of
+// the activation pass competing for the SIMDs, more chunks a longer serial product (measured on
+// K = 1536: 4 wavefronts x 3 chunks beats 12 x 1, 6 x 2 and 3 x 4 at every grid size).
+static FusedPlan fused_plan(int M, int K) {
+  const int KC = (K + kTileK - 1) / kTileK;
+  const int groups = KC * kTileK / 8;
+  const int max_r = M == 1 ? 2 : 1;  // two groups per thread and row only fit the registers at M = 1
+  const int max_w = M == 1 ? kMaxWaves : 8;  // M > 1 is compiled for 512 threads (256 VGPRs each)
+  for (int cpw = 3; cpw <= kMaxCPW; ++cpw) {
+    int W = (KC + cpw - 1) / cpw;
+    if (W > max_w) continue;
+    const int c = (KC + W - 1) / W;  // chunks per wavefront with that many ...
+    W = (KC + c - 1) / c;            // ... and the fewest wavefronts that need no more
+    while (W <= max_w && (groups + 64 * W - 1) / (64 * W) > max_r) ++W;
+    if (W > max_w || !fused_shape_ok(M, (KC + W - 1) / W)) continue;
+    return FusedPlan{W, (KC + W - 1) / W, (groups + 64 * W - 1) / (64 * W)};
+  }
+  return FusedPlan{0, 0, 0};
+}
+
+template <int M, int R, int CPW>
+static hipError_t launch_fused_m(const GroupArgs& ga, const float* x, int ldx, int K, int W,
+                                 hipStream_t s) {
   const int KC = (K + kTileK - 1) / kTileK;
   const int Kp = KC * kTileK;
-  const int W = pick_waves(KC);
   const size_t lds = (size_t)M * Kp + (size_t)W * M * 16 * sizeof(float) +
                      (size_t)W * M * 2 * sizeof(float);
   const dim3 grid(ga.first[ga.count]), block(64 * W);
   static bool raised1 = false, raisedg = false;
   if (ga.count == 1) {
-    auto kern = gemv_fused_kernel<M, R, false>;
+    auto kern = gemv_fused_kernel<M, R, false, CPW>;
     if (hipError_t e = raise_lds_limit(kern, lds, &raised1); e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, grid, block, lds, s, ga, x, ldx, K, KC);
   } else {
-    auto kern = gemv_fused_kernel<M, R, true>;
+    auto kern = gemv_fused_kernel<M, R, true, CPW>;
     if (hipError_t e = raise_lds_limit(kern, lds, &raisedg); e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, grid, block, lds, s, ga, x, ldx, K, KC);
   }
@@ -436,49 +542,35 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
   if (kFused) {
     const int groups = K >> 3;
     float xv[M][8];
+    float2* s_mm2 = reinterpret_cast<float2*>(s_mm);
+    const int c = (int)threadIdx.x < groups ? threadIdx.x : groups - 1;  // duplicates: harmless for min/max
 #pragma unroll
     for (int m = 0; m < M; ++m) {
-      float lo = 3.402823466e+38f, hi = -3.402823466e+38f;
-      if ((int)threadIdx.x < groups) {
-        const float* src = x + (size_t)m * ldx + 8 * threadIdx.x;
-        const float4 v0 = *reinterpret_cast<const float4*>(src);
-        const float4 v1 = *reinterpret_cast<const float4*>(src + 4);
-        const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+      const float* src = x + (size_t)m * ldx + 8 * c;
+      const float4 v0 = *reinterpret_cast<const float4*>(src);
+      const float4 v1 = *reinterpret_cast<const float4*>(src + 4);
+      const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+      float lo = f[0], hi = f[0];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          xv[m][e] = f[e];
-          lo = fminf(lo, f[e]);
-          hi = fmaxf(hi, f[e]);
-        }
+      for (int e = 0; e < 8; ++e) {
+        xv[m][e] = f[e];
+        lo = fminf(lo, f[e]);
+        hi = fmaxf(hi, f[e]);
       }
-      lo = wave_minmax<false>(lo);
-      hi = wave_minmax<true>(hi);
-      if (lane == 0) {
-        s_mm[(wave * M + m) * 2 + 0] = lo;
-        s_mm[(wave * M + m) * 2 + 1] = hi;
-      }
+      wave_minmax_pair(lo, hi);
+      if (lane == 63) s_mm2[wave * M + m] = make_float2(lo, hi);
     }
     __syncthreads();
 #pragma unroll
     for (int m = 0; m < M; ++m) {
-      float lo = 3.402823466e+38f, hi = -3.402823466e+38f;
-#pragma unroll
-      for (int w = 0; w < kWideWaves; ++w) {
-        lo = fminf(lo, s_mm[(w * M + m) * 2 + 0]);
-        hi = fmaxf(hi, s_mm[(w * M + m) * 2 + 1]);
-      }
-      const RowQuant p = row_quant_params(lo, hi);
+      float2 v = s_mm2[(j < kWideWaves ? j : kWideWaves - 1) * M + m];
+      row16_minmax_pair(v.x, v.y);
+      const RowQuant p = row_quant_params(v.x, v.y);
       recip_m[m] = p.recip;
       negzp_m[m] = -p.zp;
       if ((int)threadIdx.x < (Kp >> 3)) {
-        uint2 out = make_uint2(0, 0);
-        if ((int)threadIdx.x < groups) {
-          int q[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) q[e] = quant_one(xv[m][e], p);
-          out.x = pack4(q);
-          out.y = pack4(q + 4);
-        }
+        uint2 out = quant_group8(xv[m], p);
+        if ((int)threadIdx.x >= groups) out = make_uint2(0, 0);
         *reinterpret_cast<uint2*>(s_a + (size_t)m * Kp + 8 * threadIdx.x) = out;
       }
     }
@@ -623,31 +715,45 @@ hipError_t launch_gemv(float* y, const uint8_t* ws, const uint8_t* packed, int M
 #undef W4_CALL
 }
 
-// Row groups (of 8 k) per thread the fused kernel needs: 1 if the padded row fits one pass of
-// the workgroup, else 2.
-static int fused_groups_per_thread(int K) {
-  const int KC = (K + kTileK - 1) / kTileK;
-  const long per_pass = (long)8 * 64 * pick_waves(KC);
-  return (int)(((long)KC * kTileK + per_pass - 1) / per_pass);
-}
-
 bool gemv_fused_applies(int M, int K, int N) {
   // Every workgroup re-reads and re-quantises the M rows. That is cheaper than a second kernel
   // launch while the rows are small next to the workgroup's weights and each thread can hold its
   // share of them in registers.
   if (M < 1 || M > kGemvMaxM || (long)M * K > 16384) return false;
   if (wide_applies(K, N)) return K <= 8 * 64 * kWideWaves;  // one group of 8 per thread and row
-  const int r = fused_groups_per_thread(K);
-  return r == 1 || (r == 2 && M == 1);
+  return fused_plan(M, K).W != 0;
+}
+
+template <int M, int R>
+static hipError_t launch_fused_cpw(const GroupArgs& ga, const float* x, int ldx, int K,
+                                   const FusedPlan& p, hipStream_t s) {
+#define W4_CASE(c)                                                  \
+  case c:                                                           \
+    if constexpr (fused_shape_ok(M, c)) {                           \
+      return launch_fused_m<M, R, c>(ga, x, ldx, K, p.W, s);        \
+    } else {                                                        \
+      return hipErrorInvalidValue;                                  \
+    }
+  switch (p.CPW) {
+    W4_CASE(1)
+    W4_CASE(2)
+    W4_CASE(3)
+    W4_CASE(4)
+    W4_CASE(5)
+    default: return hipErrorInvalidValue;
+  }
+#undef W4_CASE
 }
 
 static hipError_t launch_fused_group(const GroupArgs& ga, const float* x, int ldx, int M, int K,
                                      hipStream_t s) {
-  if (fused_groups_per_thread(K) == 2) {
+  const FusedPlan p = fused_plan(M, K);
+  if (p.W == 0) return hipErrorInvalidValue;
+  if (p.R == 2) {
     if (M != 1) return hipErrorInvalidValue;
-    return launch_fused_m<1, 2>(ga, x, ldx, K, s);
+    return launch_fused_cpw<1, 2>(ga, x, ldx, K, p, s);
   }
-#define W4_CALL(m) (launch_fused_m<m, 1>(ga, x, ldx, K, s))
+#define W4_CALL(m) (launch_fused_cpw<m, 1>(ga, x, ldx, K, p, s))
   W4_DISPATCH_M(W4_CALL)
 #undef W4_CALL
 }

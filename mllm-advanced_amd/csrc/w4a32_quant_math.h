@@ -32,9 +32,15 @@ __device__ __forceinline__ RowQuant row_quant_params(float lo, float hi) {
   return p;
 }
 
+// round_half_away(v) for |v| < 2^23 as trunc(v + copysign(0.5 - 2^-25, v)): below a tie the sum
+// stays under the next integer (it is exact or rounds down), at a tie it rounds up to it.
+__device__ __forceinline__ float round_half_away(float v) {
+  return __builtin_truncf(__fadd_rn(v, __builtin_copysignf(0.49999997f, v)));
+}
+
 // round_half_away(x * scale) + zp, clamped to int8. |x * scale| <= 255, so the cast is safe.
 __device__ __forceinline__ int quant_one(float x, const RowQuant& p) {
-  int r = (int)roundf(__fmul_rn(x, p.scale)) + p.zp;
+  int r = (int)round_half_away(__fmul_rn(x, p.scale)) + p.zp;
   r = r < -128 ? -128 : r;
   return r > 127 ? 127 : r;
 }
@@ -42,6 +48,20 @@ __device__ __forceinline__ int quant_one(float x, const RowQuant& p) {
 __device__ __forceinline__ uint32_t pack4(const int* q) {
   return (uint32_t)(q[0] & 0xFF) | ((uint32_t)(q[1] & 0xFF) << 8) | ((uint32_t)(q[2] & 0xFF) << 16) |
          ((uint32_t)(q[3] & 0xFF) << 24);
+}
+
+// Eight consecutive values of a row -> eight int8, packed in memory order. The rounded value plus
+// zp + 128 is an integer in f32; v_cvt_pk_u8_f32 saturates it to [0, 255] and drops it into its
+// byte, and flipping bit 7 of every byte subtracts the 128 again.
+__device__ __forceinline__ uint2 quant_group8(const float (&x)[8], const RowQuant& p) {
+  const float shift = (float)(p.zp + 128);
+  uint32_t w[2] = {0u, 0u};
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float r = round_half_away(__fmul_rn(x[e], p.scale));
+    w[e >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(__fadd_rn(r, shift), e & 3, w[e >> 2]);
+  }
+  return make_uint2(w[0] ^ 0x80808080u, w[1] ^ 0x80808080u);
 }
 
 // Wavefront-wide min / max with DPP lane permutations (no LDS traffic): after the four
@@ -63,6 +83,51 @@ __device__ __forceinline__ float wave_minmax(float v) {
   W4_DPP_STEP(0x143, 0xc)  // row_bcast:31 into rows 2 and 3
 #undef W4_DPP_STEP
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
+// min and max of two values per lane across the wavefront, both chains interleaved so that each
+// DPP read finds its register two issue slots after the write. The totals end up in lane 63.
+__device__ __forceinline__ void wave_minmax_pair(float& lo, float& hi) {
+  asm volatile(
+      "s_nop 1\n\t"
+      "v_min_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 0\n\t"
+      "v_min_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 0\n\t"
+      "v_min_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 0\n\t"
+      "v_min_f32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 row_mirror row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 0\n\t"
+      "v_min_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+      "s_nop 0\n\t"
+      "v_min_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+      "s_nop 1"
+      : "+v"(lo), "+v"(hi));
+}
+
+// The same within every row of 16 lanes; all 16 lanes of a row end up with the row's totals.
+__device__ __forceinline__ void row16_minmax_pair(float& lo, float& hi) {
+  asm volatile(
+      "s_nop 1\n\t"
+      "v_min_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 0\n\t"
+      "v_min_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 0\n\t"
+      "v_min_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 0\n\t"
+      "v_min_f32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 row_mirror row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 1"
+      : "+v"(lo), "+v"(hi));
 }
 
 }  // namespace w4
