@@ -1,0 +1,118 @@
+/*
+ * C ABI of the f32 operators that run between the W4A32 Linears of a Qwen2-style decoder, and of a
+ * decoder runner built from them (one call = prefill of a prompt, or one greedy decode step).
+ * Same conventions as w4a32_hip.h: d_* pointers are device memory, calls only enqueue on
+ * `stream`, nothing allocates, synchronises or exits; the return value is a W4A32_* code.
+ *
+ * Positions and lengths are read from device memory, so a decode step is one fixed launch
+ * sequence that a caller may capture into a HIP graph and replay per token.
+ */
+#ifndef W4A32_DECODER_H
+#define W4A32_DECODER_H
+
+#include "w4a32_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- operators ------------------------------------------------------------------------- */
+
+/* d_out[m][:] = d_table[d_ids[m]][:]  (f32 rows of D, int64 ids clamped to [0, vocab)).
+ * LLMEmbeddingTokenOp::forward, mllm/Backends/Arm/Ops/LLMEmbeddingTokenOp.cpp:24-50. */
+int w4a32_op_embedding(const int64_t* d_ids, const float* d_table, int M, int D, int vocab,
+                       float* d_out, void* stream);
+
+/* h_out = h + delta (skipped when d_delta is NULL); y = h_out * (w * 1/sqrt(mean(h_out^2) + eps)).
+ * d_h_out may alias d_h. D % 4 == 0.
+ * ArmRMSNormOp::forward, mllm/Backends/Arm/Ops/RMSNormOp.cpp:36-76, with the residual add of
+ * QWenDecoder::forward (mllm/Models/ds_qwen2/modeling_ds_qwen2.hpp:175-183) in front. */
+int w4a32_op_rmsnorm(const float* d_h, const float* d_delta, const float* d_weight, int M, int D,
+                     float eps, float* d_h_out, float* d_y, void* stream);
+
+/* out = a + b; out = silu(gate) * up (QWenMLP::forward, modeling_ds_qwen2.hpp:47-54). n % 4 == 0. */
+int w4a32_op_add(const float* d_a, const float* d_b, float* d_out, size_t n, void* stream);
+int w4a32_op_silu_mul(const float* d_gate, const float* d_up, float* d_out, size_t n, void* stream);
+
+/* sin/cos tables [max_pos][head_dim/2]: theta = pos / base^(2d/head_dim).
+ * precompute_normal_hf_sin_cos, mllm/Backends/Arm/Kernels/rope.cpp:20-37. */
+int w4a32_op_rope_table(float* d_sin, float* d_cos, int max_pos, int head_dim, float base,
+                        void* stream);
+
+/* Rotates q [M][n_heads*head_dim] in place, rotates k and copies v [M][n_kv_heads*head_dim] into the
+ * caches [n_kv_heads][max_seq][head_dim] at positions pos0 + m. pos0 = *d_pos0 when d_pos0 is not
+ * NULL, else the argument. normal_hf_rope (rope.cpp:39-80) + ArmKVCacheOp::forward
+ * (mllm/Backends/Arm/Ops/KVCacheOp.cpp:44-72; the reference's head-repeated copies are not stored). */
+int w4a32_op_rope_kv(float* d_q, const float* d_k, const float* d_v, const float* d_sin,
+                     const float* d_cos, float* d_kcache, float* d_vcache, int M, int n_heads,
+                     int n_kv_heads, int head_dim, int max_seq, const int* d_pos0, int pos0,
+                     void* stream);
+
+/* Scratch of the decode attention and of argmax: arrival counters + partial results. Must be cleared
+ * once with w4a32_op_scratch_init before its first use; the kernels leave it cleared. */
+size_t w4a32_op_scratch_bytes(int n_heads);
+int w4a32_op_scratch_init(void* d_scratch, int n_heads, void* stream);
+
+/* out[m][h][:] = softmax(q[m][h] . K[0..pos0+m] / sqrt(head_dim)) V, head h reading KV head
+ * h / (n_heads / n_kv_heads). head_dim must be 128. With M == 1 and d_scratch given, the keys are split
+ * over several wavefronts per head (decode); otherwise one wavefront per (head, query).
+ * QWenAttention::forward, modeling_ds_qwen2.hpp:133-151 (matmul, CausalMaskOp.cpp:22-71,
+ * SoftmaxOp.cpp:18-50, matmul). */
+int w4a32_op_attention(const float* d_q, const float* d_kcache, const float* d_vcache, float* d_out,
+                       int M, int n_heads, int n_kv_heads, int head_dim, int max_seq,
+                       const int* d_pos0, int pos0, void* d_scratch, void* stream);
+
+/* *d_token = index of the first maximum of d_logits[0..n) (AutoLLM.hpp:70-88); when d_pos_to_advance
+ * is not NULL, *d_pos_to_advance += 1 afterwards. */
+int w4a32_op_argmax(const float* d_logits, int n, void* d_scratch, int64_t* d_token,
+                    int* d_pos_to_advance, void* stream);
+
+/* ---- decoder runner -------------------------------------------------------------------- */
+
+typedef struct {
+  int hidden, n_heads, n_kv_heads, head_dim, intermediate, n_layers, vocab;
+  int max_seq;           /* KV cache capacity (the reference's max_cache_length) */
+  int max_batch_tokens;  /* longest prompt chunk a prefill call may take */
+  float rope_theta, rms_eps;
+} w4a32_decoder_config;
+
+/* Device pointers; W4 blobs as produced by w4a32_quant_pack_rhs ([N][K] = [out][in]). */
+typedef struct {
+  const void *q, *k, *v, *o, *gate, *up, *down;
+  const float *attn_norm, *ffn_norm;
+} w4a32_layer_weights;
+
+typedef struct {
+  const float* embedding;             /* [vocab][hidden] f32 */
+  const float* final_norm;            /* [hidden] */
+  const void* lm_head;                /* W4 blob [vocab][hidden] */
+  const w4a32_layer_weights* layers;  /* HOST array of n_layers entries */
+} w4a32_decoder_weights;
+
+/* Bytes of the decoder state (KV caches, activations, tables, counters), 256-byte aligned base. */
+size_t w4a32_decoder_state_bytes(const w4a32_decoder_config* cfg);
+/* Byte offsets inside the state, for inspection: 0 = position counter (int32), 1 = last logits
+ * (f32 [vocab]), 2 = residual stream rows (f32 [max_batch_tokens][hidden]). */
+size_t w4a32_decoder_state_offset(const w4a32_decoder_config* cfg, int which);
+
+/* Builds the RoPE tables, clears the counters, position = 0. */
+int w4a32_decoder_init(const w4a32_decoder_config* cfg, void* d_state, void* stream);
+
+/* Runs n_tokens prompt tokens at positions pos0.. through the model (QWenForCausalLM::forward,
+ * modeling_ds_qwen2.hpp:202-215), leaves the last row's logits in the state, the greedy next token in
+ * *d_next_token and the position counter at pos0 + n_tokens. */
+int w4a32_decoder_prefill(const w4a32_decoder_config* cfg, const w4a32_decoder_weights* w,
+                          void* d_state, const int64_t* d_tokens, int n_tokens, int pos0,
+                          int64_t* d_next_token, void* stream);
+
+/* One greedy decode step at the state's current position (AutoLLM generate loop, AutoLLM.hpp:40-66):
+ * reads *d_token_in, writes *d_token_out (may be the same address), advances the position. The launch
+ * sequence does not depend on the position: capture it once, replay it per token. The caller keeps
+ * the position below max_seq. */
+int w4a32_decoder_step(const w4a32_decoder_config* cfg, const w4a32_decoder_weights* w, void* d_state,
+                       const int64_t* d_token_in, int64_t* d_token_out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* W4A32_DECODER_H */

@@ -40,7 +40,42 @@ ABI = {
     "w4a32_matmul_quantized_ex": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp]),
     "w4a32_matmul": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a32_matmul_grouped": (_ci, [_vp, _vp, _vp, _vp, _ci, _vp, _ci, _ci, _vp]),
+    # include/w4a32_decoder.h
+    "w4a32_op_embedding": (_ci, [_vp, _vp, _ci, _ci, _ci, _vp, _vp]),
+    "w4a32_op_rmsnorm": (_ci, [_vp, _vp, _vp, _ci, _ci, ctypes.c_float, _vp, _vp, _vp]),
+    "w4a32_op_add": (_ci, [_vp, _vp, _vp, _sz, _vp]),
+    "w4a32_op_silu_mul": (_ci, [_vp, _vp, _vp, _sz, _vp]),
+    "w4a32_op_rope_table": (_ci, [_vp, _vp, _ci, _ci, ctypes.c_float, _vp]),
+    "w4a32_op_rope_kv": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _ci, _vp]),
+    "w4a32_op_scratch_bytes": (_sz, [_ci]),
+    "w4a32_op_scratch_init": (_ci, [_vp, _ci, _vp]),
+    "w4a32_op_attention": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _ci, _vp, _vp]),
+    "w4a32_op_argmax": (_ci, [_vp, _ci, _vp, _vp, _vp, _vp]),
+    "w4a32_decoder_state_bytes": (_sz, [_vp]),
+    "w4a32_decoder_state_offset": (_sz, [_vp, _ci]),
+    "w4a32_decoder_init": (_ci, [_vp, _vp, _vp]),
+    "w4a32_decoder_prefill": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _vp, _vp]),
+    "w4a32_decoder_step": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp]),
 }
+
+
+class DecoderConfig(ctypes.Structure):
+    """w4a32_decoder_config"""
+    _fields_ = [(n, ctypes.c_int) for n in ("hidden", "n_heads", "n_kv_heads", "head_dim", "intermediate",
+                                            "n_layers", "vocab", "max_seq", "max_batch_tokens")] + \
+               [("rope_theta", ctypes.c_float), ("rms_eps", ctypes.c_float)]
+
+
+class LayerWeights(ctypes.Structure):
+    """w4a32_layer_weights"""
+    _fields_ = [(n, ctypes.c_void_p) for n in ("q", "k", "v", "o", "gate", "up", "down", "attn_norm",
+                                               "ffn_norm")]
+
+
+class DecoderWeights(ctypes.Structure):
+    """w4a32_decoder_weights"""
+    _fields_ = [("embedding", ctypes.c_void_p), ("final_norm", ctypes.c_void_p),
+                ("lm_head", ctypes.c_void_p), ("layers", ctypes.POINTER(LayerWeights))]
 
 
 class W4A32Error(RuntimeError):
@@ -210,3 +245,146 @@ def matmul_grouped(x, packed_list, n_list, ws=None):
     _check(lib().w4a32_matmul_grouped(y_arr, _ptr(x), p_arr, n_arr, cnt, _ptr(ws), M, K, _stream()),
            "w4a32_matmul_grouped")
     return ys
+
+
+# ---- decoder operators and runner (include/w4a32_decoder.h) ---------------------------------
+
+def op_embedding(ids, table):
+    import torch
+
+    M, (V, D) = ids.numel(), table.shape
+    out = torch.empty((M, D), dtype=torch.float32, device="cuda")
+    _check(lib().w4a32_op_embedding(_ptr(ids), _ptr(table), M, D, V, _ptr(out), _stream()),
+           "w4a32_op_embedding")
+    return out
+
+
+def op_rmsnorm(h, weight, eps, delta=None):
+    """Returns y, or (h + delta, y) when delta is given."""
+    import torch
+
+    M, D = h.shape
+    y = torch.empty_like(h)
+    h_out = torch.empty_like(h) if delta is not None else None
+    _check(lib().w4a32_op_rmsnorm(_ptr(h), _ptr(delta), _ptr(weight), M, D, eps, _ptr(h_out), _ptr(y),
+                                  _stream()), "w4a32_op_rmsnorm")
+    return y if delta is None else (h_out, y)
+
+
+def op_add(a, b):
+    import torch
+
+    out = torch.empty_like(a)
+    _check(lib().w4a32_op_add(_ptr(a), _ptr(b), _ptr(out), a.numel(), _stream()), "w4a32_op_add")
+    return out
+
+
+def op_silu_mul(gate, up):
+    import torch
+
+    out = torch.empty_like(gate)
+    _check(lib().w4a32_op_silu_mul(_ptr(gate), _ptr(up), _ptr(out), gate.numel(), _stream()),
+           "w4a32_op_silu_mul")
+    return out
+
+
+def op_rope_table(max_pos, head_dim, base):
+    import torch
+
+    sin = torch.empty((max_pos, head_dim // 2), dtype=torch.float32, device="cuda")
+    cos = torch.empty_like(sin)
+    _check(lib().w4a32_op_rope_table(_ptr(sin), _ptr(cos), max_pos, head_dim, base, _stream()),
+           "w4a32_op_rope_table")
+    return sin, cos
+
+
+def op_rope_kv(q, k, v, sin, cos, kcache, vcache, n_heads, n_kv_heads, head_dim, pos0, d_pos0=None):
+    """q is rotated in place; kcache/vcache [n_kv_heads][max_seq][head_dim] receive rows pos0.."""
+    M = q.shape[0]
+    _check(lib().w4a32_op_rope_kv(_ptr(q), _ptr(k), _ptr(v), _ptr(sin), _ptr(cos), _ptr(kcache),
+                                  _ptr(vcache), M, n_heads, n_kv_heads, head_dim, kcache.shape[1],
+                                  _ptr(d_pos0), pos0, _stream()), "w4a32_op_rope_kv")
+
+
+def op_scratch(n_heads):
+    sc = _dev_empty(int(lib().w4a32_op_scratch_bytes(n_heads)))
+    _check(lib().w4a32_op_scratch_init(_ptr(sc), n_heads, _stream()), "w4a32_op_scratch_init")
+    return sc
+
+
+def op_attention(q, kcache, vcache, n_heads, n_kv_heads, head_dim, pos0, scratch=None, d_pos0=None):
+    import torch
+
+    M = q.shape[0]
+    out = torch.empty((M, n_heads * head_dim), dtype=torch.float32, device="cuda")
+    _check(lib().w4a32_op_attention(_ptr(q), _ptr(kcache), _ptr(vcache), _ptr(out), M, n_heads,
+                                    n_kv_heads, head_dim, kcache.shape[1], _ptr(d_pos0), pos0,
+                                    _ptr(scratch), _stream()), "w4a32_op_attention")
+    return out
+
+
+def op_argmax(logits, scratch, d_pos=None):
+    import torch
+
+    tok = torch.empty((1,), dtype=torch.int64, device="cuda")
+    _check(lib().w4a32_op_argmax(_ptr(logits), logits.numel(), _ptr(scratch), _ptr(tok), _ptr(d_pos),
+                                 _stream()), "w4a32_op_argmax")
+    return tok
+
+
+class Decoder:
+    """Plumbing around the decoder runner: owns the state buffer and the argument structs.
+
+    `layers` is a list of dicts with the packed blobs q,k,v,o,gate,up,down and the f32 norm weights
+    attn_norm, ffn_norm (cuda tensors); embedding f32 [vocab][hidden]; lm_head a packed blob."""
+
+    def __init__(self, hidden, n_heads, n_kv_heads, intermediate, vocab, layers, embedding, final_norm,
+                 lm_head, max_seq=1024, max_batch_tokens=512, rope_theta=1e6, rms_eps=1e-6, head_dim=128):
+        import torch
+
+        self.cfg = DecoderConfig(hidden, n_heads, n_kv_heads, head_dim, intermediate, len(layers), vocab,
+                                 max_seq, max_batch_tokens, rope_theta, rms_eps)
+        self._keep = (layers, embedding, final_norm, lm_head)
+        arr = (LayerWeights * len(layers))()
+        for i, lw in enumerate(layers):
+            for name, _ in LayerWeights._fields_:
+                setattr(arr[i], name, lw[name].data_ptr())
+        self._layers = arr
+        self.weights = DecoderWeights(embedding.data_ptr(), final_norm.data_ptr(), lm_head.data_ptr(), arr)
+        nbytes = int(lib().w4a32_decoder_state_bytes(ctypes.byref(self.cfg)))
+        if nbytes == 0:
+            raise W4A32Error("w4a32_decoder_state_bytes: invalid configuration")
+        self.state = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        self.token = torch.zeros((1,), dtype=torch.int64, device="cuda")
+        _check(lib().w4a32_decoder_init(ctypes.byref(self.cfg), _ptr(self.state), _stream()),
+               "w4a32_decoder_init")
+
+    def _view(self, which, count, dtype):
+        off = int(lib().w4a32_decoder_state_offset(ctypes.byref(self.cfg), which))
+        return self.state[off:off + count * dtype.itemsize].view(dtype)
+
+    @property
+    def position(self):
+        import torch
+
+        return int(self._view(0, 1, torch.int32).item())
+
+    @property
+    def logits(self):
+        import torch
+
+        return self._view(1, self.cfg.vocab, torch.float32)
+
+    def prefill(self, tokens, pos0=0):
+        """tokens: int64 cuda tensor [n]. Leaves the greedy next token in self.token."""
+        _check(lib().w4a32_decoder_prefill(ctypes.byref(self.cfg), ctypes.byref(self.weights),
+                                           _ptr(self.state), _ptr(tokens), tokens.numel(), pos0,
+                                           _ptr(self.token), _stream()), "w4a32_decoder_prefill")
+        return self.token
+
+    def step(self):
+        """One greedy step: consumes self.token, replaces it with the next token."""
+        _check(lib().w4a32_decoder_step(ctypes.byref(self.cfg), ctypes.byref(self.weights),
+                                        _ptr(self.state), _ptr(self.token), _ptr(self.token), _stream()),
+               "w4a32_decoder_step")
+        return self.token

@@ -1,0 +1,316 @@
+// extern "C" surface of include/w4a32_decoder.h: the decoder operators and the runner that strings
+// them together with the W4A32 Linears. Host code only: argument checks, state geometry, launch order.
+#include "w4a32_decoder.h"
+
+#include <algorithm>
+
+#include "w4a32_internal.h"
+
+namespace {
+
+constexpr int kAttnSplit = 16;    // wavefronts per head in the decode attention
+constexpr int kArgmaxBlocks = 64;
+
+inline int from_hip(hipError_t e) { return e == hipSuccess ? W4A32_OK : W4A32_ELAUNCH; }
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+inline hipStream_t S(void* stream) { return static_cast<hipStream_t>(stream); }
+
+// Scratch of the decode attention + argmax.
+struct ScratchGeom {
+  size_t counters_off;  // u32 [n_heads + 1]
+  size_t part_off;      // f32 [n_heads][kAttnSplit][130]
+  size_t amax_val_off;  // f32 [kArgmaxBlocks]
+  size_t amax_idx_off;  // i32 [kArgmaxBlocks]
+  size_t total;
+};
+
+ScratchGeom scratch_geom(int n_heads) {
+  ScratchGeom g;
+  size_t o = 0;
+  g.counters_off = o;
+  o = align_up(o + sizeof(unsigned int) * (n_heads + 1), 256);
+  g.part_off = o;
+  o = align_up(o + sizeof(float) * (size_t)n_heads * kAttnSplit * 130, 256);
+  g.amax_val_off = o;
+  o = align_up(o + sizeof(float) * kArgmaxBlocks, 256);
+  g.amax_idx_off = o;
+  o = align_up(o + sizeof(int) * kArgmaxBlocks, 256);
+  g.total = o;
+  return g;
+}
+
+// Everything a decoder instance keeps on the device, in one caller-owned allocation.
+struct StateGeom {
+  size_t pos_off, scratch_off, sin_off, cos_off, kcache_off, vcache_off;
+  size_t h_off, xn_off, q_off, k_off, v_off, attn_off, delta_off, gate_off, up_off, act_off;
+  size_t logits_off, ws_off, total;
+  size_t cache_layer;  // floats per layer in each cache
+};
+
+bool config_ok(const w4a32_decoder_config* c) {
+  if (!c) return false;
+  if (c->hidden <= 0 || c->n_heads <= 0 || c->n_kv_heads <= 0 || c->intermediate <= 0 ||
+      c->n_layers <= 0 || c->vocab <= 0 || c->max_seq <= 0 || c->max_batch_tokens <= 0)
+    return false;
+  if (c->head_dim != 128 || c->n_heads % c->n_kv_heads != 0) return false;
+  if (c->hidden % 32 != 0 || c->intermediate % 32 != 0 || (c->n_heads * c->head_dim) % 32 != 0)
+    return false;
+  return true;
+}
+
+StateGeom state_geom(const w4a32_decoder_config* c) {
+  StateGeom g;
+  const size_t Mb = c->max_batch_tokens;
+  const size_t qd = (size_t)c->n_heads * c->head_dim, kvd = (size_t)c->n_kv_heads * c->head_dim;
+  size_t o = 0;
+  auto take = [&](size_t bytes) {
+    const size_t at = o;
+    o = align_up(o + bytes, 256);
+    return at;
+  };
+  g.pos_off = take(sizeof(int));
+  g.scratch_off = take(scratch_geom(c->n_heads).total);
+  g.sin_off = take(sizeof(float) * c->max_seq * (c->head_dim / 2));
+  g.cos_off = take(sizeof(float) * c->max_seq * (c->head_dim / 2));
+  g.cache_layer = kvd * c->max_seq;
+  g.kcache_off = take(sizeof(float) * g.cache_layer * c->n_layers);
+  g.vcache_off = take(sizeof(float) * g.cache_layer * c->n_layers);
+  g.h_off = take(sizeof(float) * Mb * c->hidden);
+  g.xn_off = take(sizeof(float) * Mb * c->hidden);
+  g.q_off = take(sizeof(float) * Mb * qd);
+  g.k_off = take(sizeof(float) * Mb * kvd);
+  g.v_off = take(sizeof(float) * Mb * kvd);
+  g.attn_off = take(sizeof(float) * Mb * qd);
+  g.delta_off = take(sizeof(float) * Mb * c->hidden);
+  g.gate_off = take(sizeof(float) * Mb * c->intermediate);
+  g.up_off = take(sizeof(float) * Mb * c->intermediate);
+  g.act_off = take(sizeof(float) * Mb * c->intermediate);
+  g.logits_off = take(sizeof(float) * c->vocab);
+  const int kmax = std::max(std::max(c->hidden, c->intermediate), (int)qd);
+  g.ws_off = take(w4a32_workspace_bytes(c->max_batch_tokens, kmax));
+  g.total = o;
+  return g;
+}
+
+#define W4_TRY(expr)                 \
+  do {                               \
+    const int rc_ = (expr);          \
+    if (rc_ != W4A32_OK) return rc_; \
+  } while (0)
+
+// The model on M rows that are already embedded in the residual stream `h`. Leaves the last row's
+// logits in the state and the greedy token in *d_token_out. d_pos: device position of row 0.
+int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, uint8_t* st,
+               const StateGeom& g, int M, int64_t* d_token_out, bool advance_by_argmax, void* stream) {
+  hipStream_t s = S(stream);
+  const int H = c->hidden, I = c->intermediate, D = c->head_dim;
+  const int Hq = c->n_heads, Hkv = c->n_kv_heads, qd = Hq * D, kvd = Hkv * D;
+  int* d_pos = reinterpret_cast<int*>(st + g.pos_off);
+  uint8_t* scratch = st + g.scratch_off;
+  const ScratchGeom sg = scratch_geom(Hq);
+  float* h = reinterpret_cast<float*>(st + g.h_off);
+  float* xn = reinterpret_cast<float*>(st + g.xn_off);
+  float* q = reinterpret_cast<float*>(st + g.q_off);
+  float* k = reinterpret_cast<float*>(st + g.k_off);
+  float* v = reinterpret_cast<float*>(st + g.v_off);
+  float* attn = reinterpret_cast<float*>(st + g.attn_off);
+  float* delta = reinterpret_cast<float*>(st + g.delta_off);
+  float* gate = reinterpret_cast<float*>(st + g.gate_off);
+  float* up = reinterpret_cast<float*>(st + g.up_off);
+  float* act = reinterpret_cast<float*>(st + g.act_off);
+  float* logits = reinterpret_cast<float*>(st + g.logits_off);
+  const float* sin_t = reinterpret_cast<const float*>(st + g.sin_off);
+  const float* cos_t = reinterpret_cast<const float*>(st + g.cos_off);
+  void* ws = st + g.ws_off;
+
+  for (int l = 0; l < c->n_layers; ++l) {
+    const w4a32_layer_weights& lw = w->layers[l];
+    float* kc = reinterpret_cast<float*>(st + g.kcache_off) + (size_t)l * g.cache_layer;
+    float* vc = reinterpret_cast<float*>(st + g.vcache_off) + (size_t)l * g.cache_layer;
+    // h += mlp output of the previous layer; xn = norm(h)
+    W4_TRY(from_hip(w4::launch_rmsnorm(h, l == 0 ? nullptr : delta, lw.attn_norm, M, H, c->rms_eps, h,
+                                       xn, s)));
+    {
+      float* ys[3] = {q, k, v};
+      const void* ps[3] = {lw.q, lw.k, lw.v};
+      const int ns[3] = {qd, kvd, kvd};
+      W4_TRY(w4a32_matmul_grouped(ys, xn, ps, ns, 3, ws, M, H, stream));
+    }
+    W4_TRY(from_hip(w4::launch_rope_kv(q, k, v, sin_t, cos_t, kc, vc, M, Hq, Hkv, D, c->max_seq, d_pos,
+                                       0, s)));
+    if (M == 1) {
+      W4_TRY(from_hip(w4::launch_attention_decode(
+          q, kc, vc, attn, Hq, Hkv, c->max_seq, d_pos, 0, kAttnSplit,
+          reinterpret_cast<float*>(scratch + sg.part_off),
+          reinterpret_cast<unsigned int*>(scratch + sg.counters_off), s)));
+    } else {
+      W4_TRY(from_hip(w4::launch_attention_prefill(q, kc, vc, attn, M, Hq, Hkv, c->max_seq, d_pos, 0, s)));
+    }
+    W4_TRY(w4a32_matmul(delta, attn, lw.o, ws, M, qd, H, stream));
+    // h += attention output; xn = norm(h)
+    W4_TRY(from_hip(w4::launch_rmsnorm(h, delta, lw.ffn_norm, M, H, c->rms_eps, h, xn, s)));
+    {
+      float* ys[2] = {gate, up};
+      const void* ps[2] = {lw.gate, lw.up};
+      const int ns[2] = {I, I};
+      W4_TRY(w4a32_matmul_grouped(ys, xn, ps, ns, 2, ws, M, H, stream));
+    }
+    W4_TRY(from_hip(w4::launch_silu_mul(gate, up, act, (size_t)M * I, s)));
+    W4_TRY(w4a32_matmul(delta, act, lw.down, ws, M, I, H, stream));
+  }
+  // Only the last row feeds the head: h_last += delta_last; xn_last = norm(h_last)
+  const size_t last = (size_t)(M - 1) * H;
+  W4_TRY(from_hip(w4::launch_rmsnorm(h + last, delta + last, w->final_norm, 1, H, c->rms_eps, h + last,
+                                     xn + last, s)));
+  W4_TRY(w4a32_matmul(logits, xn + last, w->lm_head, ws, 1, H, c->vocab, stream));
+  W4_TRY(from_hip(w4::launch_argmax(logits, c->vocab, reinterpret_cast<float*>(scratch + sg.amax_val_off),
+                                    reinterpret_cast<int*>(scratch + sg.amax_idx_off),
+                                    reinterpret_cast<unsigned int*>(scratch + sg.counters_off) + Hq,
+                                    d_token_out, advance_by_argmax ? d_pos : nullptr, kArgmaxBlocks, s)));
+  return W4A32_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int w4a32_op_embedding(const int64_t* d_ids, const float* d_table, int M, int D, int vocab,
+                       float* d_out, void* stream) {
+  if (!d_ids || !d_table || !d_out || M <= 0 || D <= 0 || vocab <= 0) return W4A32_EINVAL;
+  if (D % 4 != 0) return W4A32_ESHAPE;
+  return from_hip(w4::launch_embedding(d_ids, d_table, M, D, vocab, d_out, S(stream)));
+}
+
+int w4a32_op_rmsnorm(const float* d_h, const float* d_delta, const float* d_weight, int M, int D,
+                     float eps, float* d_h_out, float* d_y, void* stream) {
+  if (!d_h || !d_weight || !d_y || M <= 0 || D <= 0) return W4A32_EINVAL;
+  if (d_delta && !d_h_out) return W4A32_EINVAL;
+  if (D % 4 != 0) return W4A32_ESHAPE;
+  return from_hip(w4::launch_rmsnorm(d_h, d_delta, d_weight, M, D, eps, d_h_out, d_y, S(stream)));
+}
+
+int w4a32_op_add(const float* d_a, const float* d_b, float* d_out, size_t n, void* stream) {
+  if (!d_a || !d_b || !d_out || n == 0) return W4A32_EINVAL;
+  if (n % 4 != 0) return W4A32_ESHAPE;
+  return from_hip(w4::launch_add(d_a, d_b, d_out, n, S(stream)));
+}
+
+int w4a32_op_silu_mul(const float* d_gate, const float* d_up, float* d_out, size_t n, void* stream) {
+  if (!d_gate || !d_up || !d_out || n == 0) return W4A32_EINVAL;
+  if (n % 4 != 0) return W4A32_ESHAPE;
+  return from_hip(w4::launch_silu_mul(d_gate, d_up, d_out, n, S(stream)));
+}
+
+int w4a32_op_rope_table(float* d_sin, float* d_cos, int max_pos, int head_dim, float base, void* stream) {
+  if (!d_sin || !d_cos || max_pos <= 0 || head_dim <= 0 || !(base > 0.0f)) return W4A32_EINVAL;
+  if (head_dim % 2 != 0) return W4A32_ESHAPE;
+  return from_hip(w4::launch_rope_table(d_sin, d_cos, max_pos, head_dim, base, S(stream)));
+}
+
+int w4a32_op_rope_kv(float* d_q, const float* d_k, const float* d_v, const float* d_sin,
+                     const float* d_cos, float* d_kcache, float* d_vcache, int M, int n_heads,
+                     int n_kv_heads, int head_dim, int max_seq, const int* d_pos0, int pos0,
+                     void* stream) {
+  if (!d_q || !d_k || !d_v || !d_sin || !d_cos || !d_kcache || !d_vcache) return W4A32_EINVAL;
+  if (M <= 0 || n_heads <= 0 || n_kv_heads <= 0 || head_dim <= 0 || max_seq <= 0) return W4A32_EINVAL;
+  if (head_dim % 2 != 0) return W4A32_ESHAPE;
+  if (!d_pos0 && (pos0 < 0 || pos0 + M > max_seq)) return W4A32_ESHAPE;
+  return from_hip(w4::launch_rope_kv(d_q, d_k, d_v, d_sin, d_cos, d_kcache, d_vcache, M, n_heads,
+                                     n_kv_heads, head_dim, max_seq, d_pos0, pos0, S(stream)));
+}
+
+size_t w4a32_op_scratch_bytes(int n_heads) { return n_heads > 0 ? scratch_geom(n_heads).total : 0; }
+
+int w4a32_op_scratch_init(void* d_scratch, int n_heads, void* stream) {
+  if (!d_scratch || n_heads <= 0) return W4A32_EINVAL;
+  return from_hip(w4::launch_zero_u32(static_cast<unsigned int*>(d_scratch), n_heads + 1, S(stream)));
+}
+
+int w4a32_op_attention(const float* d_q, const float* d_kcache, const float* d_vcache, float* d_out,
+                       int M, int n_heads, int n_kv_heads, int head_dim, int max_seq,
+                       const int* d_pos0, int pos0, void* d_scratch, void* stream) {
+  if (!d_q || !d_kcache || !d_vcache || !d_out) return W4A32_EINVAL;
+  if (M <= 0 || n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0) return W4A32_EINVAL;
+  if (head_dim != 128 || n_heads % n_kv_heads != 0) return W4A32_ESHAPE;
+  if (!d_pos0 && (pos0 < 0 || pos0 + M > max_seq)) return W4A32_ESHAPE;
+  if (M == 1 && d_scratch) {
+    const ScratchGeom sg = scratch_geom(n_heads);
+    uint8_t* sc = static_cast<uint8_t*>(d_scratch);
+    return from_hip(w4::launch_attention_decode(
+        d_q, d_kcache, d_vcache, d_out, n_heads, n_kv_heads, max_seq, d_pos0, pos0, kAttnSplit,
+        reinterpret_cast<float*>(sc + sg.part_off), reinterpret_cast<unsigned int*>(sc + sg.counters_off),
+        S(stream)));
+  }
+  return from_hip(w4::launch_attention_prefill(d_q, d_kcache, d_vcache, d_out, M, n_heads, n_kv_heads,
+                                               max_seq, d_pos0, pos0, S(stream)));
+}
+
+int w4a32_op_argmax(const float* d_logits, int n, void* d_scratch, int64_t* d_token,
+                    int* d_pos_to_advance, void* stream) {
+  if (!d_logits || !d_scratch || !d_token || n <= 0) return W4A32_EINVAL;
+  // the counter slot after the per-head ones is argmax's; geometry for 1 head keeps it at index 1
+  const ScratchGeom sg = scratch_geom(1);
+  uint8_t* sc = static_cast<uint8_t*>(d_scratch);
+  return from_hip(w4::launch_argmax(d_logits, n, reinterpret_cast<float*>(sc + sg.amax_val_off),
+                                    reinterpret_cast<int*>(sc + sg.amax_idx_off),
+                                    reinterpret_cast<unsigned int*>(sc + sg.counters_off) + 1, d_token,
+                                    d_pos_to_advance, kArgmaxBlocks, S(stream)));
+}
+
+size_t w4a32_decoder_state_bytes(const w4a32_decoder_config* cfg) {
+  return config_ok(cfg) ? state_geom(cfg).total : 0;
+}
+
+size_t w4a32_decoder_state_offset(const w4a32_decoder_config* cfg, int which) {
+  if (!config_ok(cfg)) return 0;
+  const StateGeom g = state_geom(cfg);
+  switch (which) {
+    case 0: return g.pos_off;
+    case 1: return g.logits_off;
+    case 2: return g.h_off;
+    default: return 0;
+  }
+}
+
+int w4a32_decoder_init(const w4a32_decoder_config* cfg, void* d_state, void* stream) {
+  if (!config_ok(cfg) || !d_state) return W4A32_EINVAL;
+  if (reinterpret_cast<uintptr_t>(d_state) % 256 != 0) return W4A32_EINVAL;
+  const StateGeom g = state_geom(cfg);
+  uint8_t* st = static_cast<uint8_t*>(d_state);
+  hipStream_t s = S(stream);
+  W4_TRY(from_hip(w4::launch_set_int(reinterpret_cast<int*>(st + g.pos_off), 0, s)));
+  W4_TRY(from_hip(w4::launch_zero_u32(reinterpret_cast<unsigned int*>(st + g.scratch_off),
+                                      cfg->n_heads + 1, s)));
+  return from_hip(w4::launch_rope_table(reinterpret_cast<float*>(st + g.sin_off),
+                                        reinterpret_cast<float*>(st + g.cos_off), cfg->max_seq,
+                                        cfg->head_dim, cfg->rope_theta, s));
+}
+
+int w4a32_decoder_prefill(const w4a32_decoder_config* cfg, const w4a32_decoder_weights* w,
+                          void* d_state, const int64_t* d_tokens, int n_tokens, int pos0,
+                          int64_t* d_next_token, void* stream) {
+  if (!config_ok(cfg) || !w || !w->layers || !d_state || !d_tokens || !d_next_token) return W4A32_EINVAL;
+  if (n_tokens <= 0 || n_tokens > cfg->max_batch_tokens) return W4A32_ESHAPE;
+  if (pos0 < 0 || pos0 + n_tokens > cfg->max_seq) return W4A32_ESHAPE;
+  const StateGeom g = state_geom(cfg);
+  uint8_t* st = static_cast<uint8_t*>(d_state);
+  hipStream_t s = S(stream);
+  int* d_pos = reinterpret_cast<int*>(st + g.pos_off);
+  W4_TRY(from_hip(w4::launch_set_int(d_pos, pos0, s)));
+  W4_TRY(from_hip(w4::launch_embedding(d_tokens, w->embedding, n_tokens, cfg->hidden, cfg->vocab,
+                                       reinterpret_cast<float*>(st + g.h_off), s)));
+  W4_TRY(run_layers(cfg, w, st, g, n_tokens, d_next_token, false, stream));
+  return from_hip(w4::launch_add_to_int(d_pos, n_tokens, s));
+}
+
+int w4a32_decoder_step(const w4a32_decoder_config* cfg, const w4a32_decoder_weights* w, void* d_state,
+                       const int64_t* d_token_in, int64_t* d_token_out, void* stream) {
+  if (!config_ok(cfg) || !w || !w->layers || !d_state || !d_token_in || !d_token_out) return W4A32_EINVAL;
+  const StateGeom g = state_geom(cfg);
+  uint8_t* st = static_cast<uint8_t*>(d_state);
+  W4_TRY(from_hip(w4::launch_embedding(d_token_in, w->embedding, 1, cfg->hidden, cfg->vocab,
+                                       reinterpret_cast<float*>(st + g.h_off), S(stream))));
+  return run_layers(cfg, w, st, g, 1, d_token_out, true, stream);
+}
+
+}  // extern "C"

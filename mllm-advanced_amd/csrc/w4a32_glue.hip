@@ -1,0 +1,474 @@
+// The f32 operators a Qwen2-style decoder runs between its quantized Linears: embedding gather,
+// RMSNorm (optionally with the residual add in front), RoPE + KV-cache append, attention over the
+// cache, SiLU*mul, residual add, greedy argmax. All of them are small, latency-bound kernels at
+// decode sizes; the point of having them here is that a whole token runs on the device without a
+// host round trip and can be replayed from a HIP graph (positions and lengths are read from
+// device memory, never baked into the launch).
+//
+// Reference behaviour followed (file:line in the reference tree):
+//   RMSNorm     mllm/Backends/Arm/Ops/RMSNormOp.cpp:36-76     y = x * (w * 1/sqrt(mean(x^2) + eps))
+//   RoPE        mllm/Backends/Arm/Kernels/rope.cpp:20-80      half-split pairs (d, d + D/2),
+//               theta_d = pos / base^(2d/D), y0 = x0 c - x1 s, y1 = x0 s + x1 c
+//   KV cache    mllm/Backends/Arm/Ops/KVCacheOp.cpp:44-72     append at the current length; the
+//               reference stores every KV head `repeat` times, here a query head indexes its KV head
+//   attention   mllm/Models/ds_qwen2/modeling_ds_qwen2.hpp:133-151  softmax(q k^T / sqrt(D)) v,
+//               query at position p sees keys 0..p (CausalMaskOp.cpp:22-71, SoftmaxOp.cpp:18-50)
+//   SiLU * mul  modeling_ds_qwen2.hpp:47-54
+//   embedding   mllm/Backends/Arm/Ops/LLMEmbeddingTokenOp.cpp:24-50 (int64 ids, f32 rows)
+//   argmax      mllm/Models/AutoLLM.hpp:70-88 (strict '>': the first maximum wins)
+#include "w4a32_internal.h"
+
+namespace w4 {
+
+namespace {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+// Sum over the workgroup (blockDim.x a multiple of 64, at most 1024); every thread gets the total.
+__device__ __forceinline__ float block_sum(float v, float* s_part) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  if ((threadIdx.x & 63) == 0) s_part[wave] = v;
+  __syncthreads();
+  float t = 0.0f;
+  for (int w = 0; w < nw; ++w) t += s_part[w];
+  __syncthreads();
+  return t;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------
+// Embedding gather: out[m][:] = table[ids[m]][:]
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void embedding_kernel(const int64_t* __restrict__ ids,
+                                                        const float* __restrict__ table, int D,
+                                                        int vocab, float* __restrict__ out) {
+  const int m = blockIdx.x;
+  long id = ids[m];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);  // out-of-range ids are clamped, never read past the table
+  const float4* src = reinterpret_cast<const float4*>(table + (size_t)id * D);
+  float4* dst = reinterpret_cast<float4*>(out + (size_t)m * D);
+  for (int i = threadIdx.x; i < D / 4; i += blockDim.x) dst[i] = src[i];
+}
+
+// ---------------------------------------------------------------------------------------------
+// RMSNorm, optionally preceded by a residual add:
+//   h_out = h (+ delta);  y = h_out * (w * 1/sqrt(mean(h_out^2) + eps))
+// One workgroup per row. h_out may alias h; it is not written when delta is null.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ h,
+                                                      const float* __restrict__ delta,
+                                                      const float* __restrict__ w, int D, float eps,
+                                                      float* h_out, float* __restrict__ y) {
+  __shared__ float s_part[4];
+  const size_t row = (size_t)blockIdx.x * D;
+  float ss = 0.0f;
+  for (int i = 4 * threadIdx.x; i < D; i += 4 * blockDim.x) {
+    float4 v = *reinterpret_cast<const float4*>(h + row + i);
+    if (delta) {
+      const float4 d = *reinterpret_cast<const float4*>(delta + row + i);
+      v.x += d.x;
+      v.y += d.y;
+      v.z += d.z;
+      v.w += d.w;
+      *reinterpret_cast<float4*>(h_out + row + i) = v;
+    }
+    ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+  }
+  const float mean = block_sum(ss, s_part) / (float)D;
+  const float rstd = 1.0f / sqrtf(mean + eps);
+  const float* src = delta ? h_out : h;  // this thread re-reads exactly what it wrote above
+  for (int i = 4 * threadIdx.x; i < D; i += 4 * blockDim.x) {
+    const float4 v = *reinterpret_cast<const float4*>(src + row + i);
+    const float4 g = *reinterpret_cast<const float4*>(w + i);
+    float4 o;
+    o.x = v.x * (g.x * rstd);
+    o.y = v.y * (g.y * rstd);
+    o.z = v.z * (g.z * rstd);
+    o.w = v.w * (g.w * rstd);
+    *reinterpret_cast<float4*>(y + row + i) = o;
+  }
+}
+
+// out = a + b, elementwise (n a multiple of 4)
+__global__ __launch_bounds__(256) void add_kernel(const float* __restrict__ a,
+                                                  const float* __restrict__ b, float* out, size_t n4) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n4) {
+    const float4 x = reinterpret_cast<const float4*>(a)[i];
+    const float4 y = reinterpret_cast<const float4*>(b)[i];
+    reinterpret_cast<float4*>(out)[i] = make_float4(x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w);
+  }
+}
+
+// out = silu(g) * u = g / (1 + exp(-g)) * u
+__global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ g,
+                                                       const float* __restrict__ u,
+                                                       float* __restrict__ out, size_t n4) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n4) {
+    const float4 a = reinterpret_cast<const float4*>(g)[i];
+    const float4 b = reinterpret_cast<const float4*>(u)[i];
+    float4 o;
+    o.x = a.x / (1.0f + expf(-a.x)) * b.x;
+    o.y = a.y / (1.0f + expf(-a.y)) * b.y;
+    o.z = a.z / (1.0f + expf(-a.z)) * b.z;
+    o.w = a.w / (1.0f + expf(-a.w)) * b.w;
+    reinterpret_cast<float4*>(out)[i] = o;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// RoPE tables: sin/cos [max_pos][D/2] (the reference stores each value twice, at d and d + D/2).
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void rope_table_kernel(float* __restrict__ sin_t,
+                                                        float* __restrict__ cos_t, int D, float base) {
+  const int pos = blockIdx.x;
+  const int half = D / 2;
+  for (int d = threadIdx.x; d < half; d += blockDim.x) {
+    float theta = 1.0f / powf(base, 2.0f * (float)d / (float)D);
+    theta *= (float)pos;
+    sin_t[(size_t)pos * half + d] = sinf(theta);
+    cos_t[(size_t)pos * half + d] = cosf(theta);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// RoPE on q and k, then k and v into the cache at positions pos0 + m.
+//   q [M][Hq*D] rotated in place; k, v [M][Hkv*D]; caches [Hkv][max_seq][D].
+// grid (M, Hq + 2*Hkv), one wavefront per head vector. pos0 comes from device memory when
+// d_pos0 is given (graph replay), else from the argument.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void rope_kv_kernel(float* __restrict__ q,
+                                                     const float* __restrict__ k,
+                                                     const float* __restrict__ v,
+                                                     const float* __restrict__ sin_t,
+                                                     const float* __restrict__ cos_t,
+                                                     float* __restrict__ kc, float* __restrict__ vc,
+                                                     int Hq, int Hkv, int D, int max_seq,
+                                                     const int* __restrict__ d_pos0, int pos0) {
+  const int m = blockIdx.x, head = blockIdx.y;
+  const int half = D / 2;
+  if (d_pos0) pos0 = *d_pos0;
+  const int pos = pos0 + m;
+  if (pos >= max_seq) return;  // the host checks capacity; a replayed graph past the end does nothing
+  const float* st = sin_t + (size_t)pos * half;
+  const float* ct = cos_t + (size_t)pos * half;
+  if (head < Hq) {
+    float* x = q + ((size_t)m * Hq + head) * D;
+    for (int d = threadIdx.x; d < half; d += 64) {
+      const float x0 = x[d], x1 = x[d + half], s = st[d], c = ct[d];
+      x[d] = x0 * c - x1 * s;
+      x[d + half] = x0 * s + x1 * c;
+    }
+  } else if (head < Hq + Hkv) {
+    const int hk = head - Hq;
+    const float* x = k + ((size_t)m * Hkv + hk) * D;
+    float* dst = kc + ((size_t)hk * max_seq + pos) * D;
+    for (int d = threadIdx.x; d < half; d += 64) {
+      const float x0 = x[d], x1 = x[d + half], s = st[d], c = ct[d];
+      dst[d] = x0 * c - x1 * s;
+      dst[d + half] = x0 * s + x1 * c;
+    }
+  } else {
+    const int hk = head - Hq - Hkv;
+    const float* x = v + ((size_t)m * Hkv + hk) * D;
+    float* dst = vc + ((size_t)hk * max_seq + pos) * D;
+    for (int d = threadIdx.x; d < D; d += 64) dst[d] = x[d];
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Attention of one query vector per wavefront over the cached keys 0..pos (head_dim 128).
+//
+// A wavefront takes 64 keys at a time: lane = key for the scores (each lane walks its key's row,
+// q comes from LDS as a broadcast read), online softmax across chunks, then lane = 2 output
+// dims for P*V (one coalesced 512-byte row per key, the weight broadcast with v_readlane).
+//
+// kSplit = false (prefill): grid (Hq, M); query m sits at position pos0 + m; output written normalised.
+// kSplit = true  (decode, M = 1): grid (Hq, nsplit); every wavefront takes a contiguous share of
+//   the keys and leaves (max, sum, unnormalised acc[128]) in `part`; the last one to finish for a
+//   head (arrival counter, reset for the next launch) merges the shares and writes the output.
+// ---------------------------------------------------------------------------------------------
+constexpr int kHeadDim = 128;
+constexpr int kPartStride = kHeadDim + 2;
+
+template <bool kSplit>
+__global__ __launch_bounds__(64) void attention_kernel(const float* __restrict__ q,
+                                                       const float* __restrict__ kc,
+                                                       const float* __restrict__ vc,
+                                                       float* __restrict__ out, int Hq, int Hkv,
+                                                       int max_seq, const int* __restrict__ d_pos0,
+                                                       int pos0, float scale, float* part,
+                                                       unsigned int* counters) {
+  __shared__ __align__(16) float s_q[kHeadDim];
+  const int h = blockIdx.x, lane = threadIdx.x;
+  const int hk = h / (Hq / Hkv);
+  if (d_pos0) pos0 = *d_pos0;
+  int m, begin, end;
+  if (kSplit) {
+    m = 0;
+    const int len = min(pos0 + 1, max_seq);
+    const int per = (len + (int)gridDim.y - 1) / (int)gridDim.y;
+    begin = min((int)blockIdx.y * per, len);
+    end = min(begin + per, len);
+  } else {
+    m = blockIdx.y;
+    begin = 0;
+    end = min(pos0 + m + 1, max_seq);
+  }
+  const float* qv = q + ((size_t)m * Hq + h) * kHeadDim;
+  s_q[lane] = qv[lane];
+  s_q[lane + 64] = qv[lane + 64];
+  __syncthreads();
+
+  const float* kbase = kc + (size_t)hk * max_seq * kHeadDim;
+  const float* vbase = vc + (size_t)hk * max_seq * kHeadDim;
+  float run_max = -INFINITY, run_sum = 0.0f;
+  float acc0 = 0.0f, acc1 = 0.0f;  // output dims 2*lane, 2*lane + 1
+
+  for (int base = begin; base < end; base += 64) {
+    const int key = base + lane;
+    const bool valid = key < end;
+    const float4* krow = reinterpret_cast<const float4*>(kbase + (size_t)(valid ? key : end - 1) * kHeadDim);
+    float dot = 0.0f;
+#pragma unroll 8
+    for (int i = 0; i < kHeadDim / 4; ++i) {
+      const float4 kv = krow[i];
+      const float4 qq = *reinterpret_cast<const float4*>(s_q + 4 * i);
+      dot += qq.x * kv.x;
+      dot += qq.y * kv.y;
+      dot += qq.z * kv.z;
+      dot += qq.w * kv.w;
+    }
+    const float score = valid ? dot * scale : -INFINITY;
+    const float new_max = fmaxf(run_max, wave_max(score));
+    const float p = valid ? expf(score - new_max) : 0.0f;
+    const float corr = expf(run_max - new_max);  // 0 on the first chunk (run_max = -inf)
+    run_sum = run_sum * corr + wave_sum(p);
+    acc0 *= corr;
+    acc1 *= corr;
+    run_max = new_max;
+    const int cnt = min(64, end - base);
+    for (int i = 0; i < cnt; ++i) {
+      const float pi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), i));
+      const float2 vv = *reinterpret_cast<const float2*>(vbase + (size_t)(base + i) * kHeadDim + 2 * lane);
+      acc0 += pi * vv.x;
+      acc1 += pi * vv.y;
+    }
+  }
+
+  if (!kSplit) {
+    const float inv = 1.0f / run_sum;  // every query sees at least its own key
+    float* o = out + ((size_t)m * Hq + h) * kHeadDim;
+    *reinterpret_cast<float2*>(o + 2 * lane) = make_float2(acc0 * inv, acc1 * inv);
+    return;
+  }
+
+  // share of this wavefront
+  float* mine = part + ((size_t)h * gridDim.y + blockIdx.y) * kPartStride;
+  *reinterpret_cast<float2*>(mine + 2 + 2 * lane) = make_float2(acc0, acc1);
+  if (lane == 0) {
+    mine[0] = run_max;
+    mine[1] = run_sum;
+  }
+  __threadfence();
+  __shared__ unsigned int s_prev;
+  if (lane == 0) {
+    s_prev = __hip_atomic_fetch_add(counters + h, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (s_prev != gridDim.y - 1) return;
+  __threadfence();
+  // last arrival for this head: merge
+  const int ns = gridDim.y;
+  const float* all = part + (size_t)h * ns * kPartStride;
+  float gmax = -INFINITY;
+  for (int s = 0; s < ns; ++s) gmax = fmaxf(gmax, __builtin_nontemporal_load(all + (size_t)s * kPartStride));
+  float total = 0.0f, o0 = 0.0f, o1 = 0.0f;
+  for (int s = 0; s < ns; ++s) {
+    const float* ps = all + (size_t)s * kPartStride;
+    const float ms = __builtin_nontemporal_load(ps);
+    const float wgt = ms == -INFINITY ? 0.0f : expf(ms - gmax);  // an empty share has max = -inf
+    total += __builtin_nontemporal_load(ps + 1) * wgt;
+    o0 += __builtin_nontemporal_load(ps + 2 + 2 * lane) * wgt;
+    o1 += __builtin_nontemporal_load(ps + 3 + 2 * lane) * wgt;
+  }
+  const float inv = 1.0f / total;
+  float* o = out + (size_t)h * kHeadDim;
+  *reinterpret_cast<float2*>(o + 2 * lane) = make_float2(o0 * inv, o1 * inv);
+  if (lane == 0) counters[h] = 0;  // ready for the next launch
+}
+
+// ---------------------------------------------------------------------------------------------
+// Greedy argmax over one row of logits: the first maximum wins. Workgroups reduce slices, the
+// last one to finish (arrival counter) reduces the per-workgroup results, writes the token and,
+// when given, advances the position counter of the decoder state.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ void argmax_merge(float& bv, int& bi, float v, int i) {
+  if (v > bv || (v == bv && i < bi)) {
+    bv = v;
+    bi = i;
+  }
+}
+
+__global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ logits, int n,
+                                                     float* part_val, int* part_idx,
+                                                     unsigned int* counter, int64_t* __restrict__ token_out,
+                                                     int* pos_to_advance) {
+  __shared__ float s_val[256];
+  __shared__ int s_idx[256];
+  __shared__ unsigned int s_prev;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+    argmax_merge(bv, bi, logits[i], i);
+  }
+  s_val[threadIdx.x] = bv;
+  s_idx[threadIdx.x] = bi;
+  __syncthreads();
+  for (int off = 128; off >= 1; off >>= 1) {
+    if ((int)threadIdx.x < off) {
+      float v = s_val[threadIdx.x];
+      int i = s_idx[threadIdx.x];
+      argmax_merge(v, i, s_val[threadIdx.x + off], s_idx[threadIdx.x + off]);
+      s_val[threadIdx.x] = v;
+      s_idx[threadIdx.x] = i;
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    part_val[blockIdx.x] = s_val[0];
+    part_idx[blockIdx.x] = s_idx[0];
+    __threadfence();
+    s_prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (s_prev != gridDim.x - 1) return;
+  __threadfence();
+  bv = -INFINITY;
+  bi = 0x7fffffff;
+  for (int b = threadIdx.x; b < (int)gridDim.x; b += blockDim.x) {
+    argmax_merge(bv, bi, __builtin_nontemporal_load(part_val + b), __builtin_nontemporal_load(part_idx + b));
+  }
+  s_val[threadIdx.x] = bv;
+  s_idx[threadIdx.x] = bi;
+  __syncthreads();
+  for (int off = 128; off >= 1; off >>= 1) {
+    if ((int)threadIdx.x < off) {
+      float v = s_val[threadIdx.x];
+      int i = s_idx[threadIdx.x];
+      argmax_merge(v, i, s_val[threadIdx.x + off], s_idx[threadIdx.x + off]);
+      s_val[threadIdx.x] = v;
+      s_idx[threadIdx.x] = i;
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    const int best = s_idx[0] == 0x7fffffff ? 0 : s_idx[0];  // all -inf / NaN: token 0, as the reference's scan
+    *token_out = best;
+    *counter = 0;
+    if (pos_to_advance) *pos_to_advance += 1;
+  }
+}
+
+__global__ void add_to_int_kernel(int* p, int delta) { *p += delta; }
+__global__ void set_int_kernel(int* p, int value) { *p = value; }
+__global__ void zero_u32_kernel(unsigned int* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// launchers
+// ---------------------------------------------------------------------------------------------
+hipError_t launch_embedding(const int64_t* ids, const float* table, int M, int D, int vocab,
+                            float* out, hipStream_t s) {
+  hipLaunchKernelGGL(embedding_kernel, dim3(M), dim3(256), 0, s, ids, table, D, vocab, out);
+  return hipGetLastError();
+}
+
+hipError_t launch_rmsnorm(const float* h, const float* delta, const float* w, int M, int D, float eps,
+                          float* h_out, float* y, hipStream_t s) {
+  hipLaunchKernelGGL(rmsnorm_kernel, dim3(M), dim3(256), 0, s, h, delta, w, D, eps, h_out, y);
+  return hipGetLastError();
+}
+
+hipError_t launch_add(const float* a, const float* b, float* out, size_t n, hipStream_t s) {
+  const size_t n4 = n / 4;
+  hipLaunchKernelGGL(add_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, a, b, out, n4);
+  return hipGetLastError();
+}
+
+hipError_t launch_silu_mul(const float* g, const float* u, float* out, size_t n, hipStream_t s) {
+  const size_t n4 = n / 4;
+  hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, g, u, out, n4);
+  return hipGetLastError();
+}
+
+hipError_t launch_rope_table(float* sin_t, float* cos_t, int max_pos, int D, float base, hipStream_t s) {
+  hipLaunchKernelGGL(rope_table_kernel, dim3(max_pos), dim3(64), 0, s, sin_t, cos_t, D, base);
+  return hipGetLastError();
+}
+
+hipError_t launch_rope_kv(float* q, const float* k, const float* v, const float* sin_t,
+                          const float* cos_t, float* kc, float* vc, int M, int Hq, int Hkv, int D,
+                          int max_seq, const int* d_pos0, int pos0, hipStream_t s) {
+  hipLaunchKernelGGL(rope_kv_kernel, dim3(M, Hq + 2 * Hkv), dim3(64), 0, s, q, k, v, sin_t, cos_t, kc,
+                     vc, Hq, Hkv, D, max_seq, d_pos0, pos0);
+  return hipGetLastError();
+}
+
+hipError_t launch_attention_prefill(const float* q, const float* kc, const float* vc, float* out,
+                                    int M, int Hq, int Hkv, int max_seq, const int* d_pos0, int pos0,
+                                    hipStream_t s) {
+  const float scale = 1.0f / sqrtf((float)kHeadDim);
+  hipLaunchKernelGGL(attention_kernel<false>, dim3(Hq, M), dim3(64), 0, s, q, kc, vc, out, Hq, Hkv,
+                     max_seq, d_pos0, pos0, scale, nullptr, nullptr);
+  return hipGetLastError();
+}
+
+hipError_t launch_attention_decode(const float* q, const float* kc, const float* vc, float* out,
+                                   int Hq, int Hkv, int max_seq, const int* d_pos0, int pos0,
+                                   int nsplit, float* part, unsigned int* counters, hipStream_t s) {
+  const float scale = 1.0f / sqrtf((float)kHeadDim);
+  hipLaunchKernelGGL(attention_kernel<true>, dim3(Hq, nsplit), dim3(64), 0, s, q, kc, vc, out, Hq, Hkv,
+                     max_seq, d_pos0, pos0, scale, part, counters);
+  return hipGetLastError();
+}
+
+hipError_t launch_argmax(const float* logits, int n, float* part_val, int* part_idx,
+                         unsigned int* counter, int64_t* token_out, int* pos_to_advance, int blocks,
+                         hipStream_t s) {
+  hipLaunchKernelGGL(argmax_kernel, dim3(blocks), dim3(256), 0, s, logits, n, part_val, part_idx,
+                     counter, token_out, pos_to_advance);
+  return hipGetLastError();
+}
+
+hipError_t launch_set_int(int* p, int value, hipStream_t s) {
+  hipLaunchKernelGGL(set_int_kernel, dim3(1), dim3(1), 0, s, p, value);
+  return hipGetLastError();
+}
+
+hipError_t launch_add_to_int(int* p, int delta, hipStream_t s) {
+  hipLaunchKernelGGL(add_to_int_kernel, dim3(1), dim3(1), 0, s, p, delta);
+  return hipGetLastError();
+}
+
+hipError_t launch_zero_u32(unsigned int* p, int n, hipStream_t s) {
+  hipLaunchKernelGGL(zero_u32_kernel, dim3((n + 255) / 256), dim3(256), 0, s, p, n);
+  return hipGetLastError();
+}
+
+}  // namespace w4

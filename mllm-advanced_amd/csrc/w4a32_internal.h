@@ -34,6 +34,30 @@ hipError_t launch_gemv_group(float* const* y, const float* x, int ldx, const uin
 hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                        int kernel, hipStream_t s);
 
+// decoder operators (f32), w4a32_glue.hip
+hipError_t launch_embedding(const int64_t* ids, const float* table, int M, int D, int vocab,
+                            float* out, hipStream_t s);
+hipError_t launch_rmsnorm(const float* h, const float* delta, const float* w, int M, int D, float eps,
+                          float* h_out, float* y, hipStream_t s);
+hipError_t launch_add(const float* a, const float* b, float* out, size_t n, hipStream_t s);
+hipError_t launch_silu_mul(const float* g, const float* u, float* out, size_t n, hipStream_t s);
+hipError_t launch_rope_table(float* sin_t, float* cos_t, int max_pos, int D, float base, hipStream_t s);
+hipError_t launch_rope_kv(float* q, const float* k, const float* v, const float* sin_t,
+                          const float* cos_t, float* kc, float* vc, int M, int Hq, int Hkv, int D,
+                          int max_seq, const int* d_pos0, int pos0, hipStream_t s);
+hipError_t launch_attention_prefill(const float* q, const float* kc, const float* vc, float* out,
+                                    int M, int Hq, int Hkv, int max_seq, const int* d_pos0, int pos0,
+                                    hipStream_t s);
+hipError_t launch_attention_decode(const float* q, const float* kc, const float* vc, float* out,
+                                   int Hq, int Hkv, int max_seq, const int* d_pos0, int pos0,
+                                   int nsplit, float* part, unsigned int* counters, hipStream_t s);
+hipError_t launch_argmax(const float* logits, int n, float* part_val, int* part_idx,
+                         unsigned int* counter, int64_t* token_out, int* pos_to_advance, int blocks,
+                         hipStream_t s);
+hipError_t launch_set_int(int* p, int value, hipStream_t s);
+hipError_t launch_add_to_int(int* p, int delta, hipStream_t s);
+hipError_t launch_zero_u32(unsigned int* p, int n, hipStream_t s);
+
 // kernel selectors of w4a32_matmul_quantized_ex (0 = the library's own choice)
 constexpr int kKernelAuto = 0;
 constexpr int kKernelGemv = 1;

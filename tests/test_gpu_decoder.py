@@ -1,0 +1,228 @@
+"""GPU: the decoder operators against torch's float32 operators, and the decoder runner against the
+CPU oracle (teacher-forced with the runner's own tokens so both see the same history).
+
+Tolerances (f32 operators, different summation order only): 1e-5 relative for the elementwise and
+normalisation operators, 2e-5 for attention; whole-model logits 2e-3 max-abs-rel (every Linear
+re-quantises its input rows to int8, so a last-bit difference upstream can flip a quantised value)."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import max_abs_rel
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def test_embedding_rmsnorm_add_silu(pkg):
+    g = torch.Generator(device="cuda").manual_seed(0)
+    table = torch.randn((300, 256), generator=g, device="cuda")
+    ids = torch.tensor([5, 299, 0, 17, 1000, -4], dtype=torch.int64, device="cuda")   # the last two are clamped
+    out = pkg.op_embedding(ids, table)
+    assert torch.equal(out, table[ids.clamp(0, 299)])
+
+    for M, D in [(1, 1536), (7, 1536), (3, 8960), (2, 96)]:
+        h = torch.randn((M, D), generator=g, device="cuda") * 3
+        d = torch.randn((M, D), generator=g, device="cuda")
+        w = 1 + 0.1 * torch.randn((D,), generator=g, device="cuda")
+        y = pkg.op_rmsnorm(h, w, 1e-6)
+        ref = torch.nn.functional.rms_norm(h, (D,), w, eps=1e-6)
+        assert max_abs_rel(y.cpu().numpy(), ref.cpu().numpy()) < 1e-5
+        h2, y2 = pkg.op_rmsnorm(h, w, 1e-6, delta=d)
+        assert torch.equal(h2, h + d)
+        assert max_abs_rel(y2.cpu().numpy(), torch.nn.functional.rms_norm(h + d, (D,), w, eps=1e-6).cpu().numpy()) < 1e-5
+
+    a = torch.randn((4, 8960), generator=g, device="cuda") * 4
+    b = torch.randn((4, 8960), generator=g, device="cuda")
+    assert torch.equal(pkg.op_add(a, b), a + b)
+    ref = torch.nn.functional.silu(a) * b
+    assert max_abs_rel(pkg.op_silu_mul(a, b).cpu().numpy(), ref.cpu().numpy()) < 1e-5
+
+
+def test_rope_table_and_kv_append(pkg):
+    import decoder_oracle as do
+
+    sin, cos = pkg.op_rope_table(1024, 128, 1e6)
+    rs, rc = do.rope_tables(1024, 128, 1e6)
+    # The angle itself is a float32 product pos * base^(-2d/D): one ulp of difference in powf is a
+    # relative 6e-8 of an angle of up to 1023 rad, i.e. up to ~6e-5 in the sine. Small angles agree closely.
+    err_s = float(np.abs(sin.cpu().numpy() - rs).max())
+    err_c = float(np.abs(cos.cpu().numpy() - rc).max())
+    assert err_s < 1.5e-4 and err_c < 1.5e-4
+    assert float(np.abs(sin.cpu().numpy() - rs)[:16].max()) < 2e-6
+
+    rng = np.random.default_rng(1)
+    M, Hq, Hkv, D, S, pos0 = 5, 4, 2, 128, 32, 9
+    q = rng.standard_normal((M, Hq * D)).astype(np.float32)
+    k = rng.standard_normal((M, Hkv * D)).astype(np.float32)
+    v = rng.standard_normal((M, Hkv * D)).astype(np.float32)
+    kc = torch.zeros((Hkv, S, D), device="cuda")
+    vc = torch.zeros((Hkv, S, D), device="cuda")
+    dq = dev(q)
+    pkg.op_rope_kv(dq, dev(k), dev(v), sin, cos, kc, vc, Hq, Hkv, D, pos0)
+    s_np, c_np = sin.cpu().numpy(), cos.cpu().numpy()
+    assert np.allclose(dq.cpu().numpy().reshape(M, Hq, D), do.rope(q.reshape(M, Hq, D), s_np, c_np, pos0),
+                       rtol=1e-6, atol=1e-6)
+    want_k = do.rope(k.reshape(M, Hkv, D), s_np, c_np, pos0).transpose(1, 0, 2)
+    assert np.allclose(kc[:, pos0:pos0 + M].cpu().numpy(), want_k, rtol=1e-6, atol=1e-6)
+    assert np.array_equal(vc[:, pos0:pos0 + M].cpu().numpy(), v.reshape(M, Hkv, D).transpose(1, 0, 2))
+    assert float(kc[:, :pos0].abs().max()) == 0 and float(kc[:, pos0 + M:].abs().max()) == 0
+    # position from device memory (what a replayed graph uses)
+    d_pos = torch.tensor([pos0], dtype=torch.int32, device="cuda")
+    kc2, vc2, dq2 = torch.zeros_like(kc), torch.zeros_like(vc), dev(q)
+    pkg.op_rope_kv(dq2, dev(k), dev(v), sin, cos, kc2, vc2, Hq, Hkv, D, 0, d_pos0=d_pos)
+    assert torch.equal(kc2, kc) and torch.equal(vc2, vc) and torch.equal(dq2, dq)
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(12, 2), (4, 4), (2, 1)])
+def test_attention_prefill_and_decode(pkg, Hq, Hkv):
+    g = torch.Generator(device="cuda").manual_seed(2)
+    D, S = 128, 1024
+    kc = torch.randn((Hkv, S, D), generator=g, device="cuda")
+    vc = torch.randn((Hkv, S, D), generator=g, device="cuda")
+
+    def ref(q, pos0):
+        M = q.shape[0]
+        tq = q.view(M, Hq, D).permute(1, 0, 2)[None]
+        n = pos0 + M
+        tk = kc[:, :n].repeat_interleave(Hq // Hkv, dim=0)[None]
+        tv = vc[:, :n].repeat_interleave(Hq // Hkv, dim=0)[None]
+        mask = torch.ones(M, n, dtype=torch.bool, device="cuda").tril(diagonal=pos0)
+        with torch.nn.attention.sdpa_kernel(torch.nn.attention.SDPBackend.MATH):
+            o = torch.nn.functional.scaled_dot_product_attention(tq, tk, tv, attn_mask=mask)
+        return o[0].permute(1, 0, 2).reshape(M, Hq * D)
+
+    for M, pos0 in [(1, 0), (5, 0), (70, 0), (33, 100), (130, 0)]:
+        q = torch.randn((M, Hq * D), generator=g, device="cuda")
+        out = pkg.op_attention(q, kc, vc, Hq, Hkv, D, pos0)
+        assert max_abs_rel(out.cpu().numpy(), ref(q, pos0).cpu().numpy()) < 2e-5, (M, pos0)
+
+    scratch = pkg.op_scratch(Hq)
+    for pos in [0, 1, 15, 16, 63, 64, 200, 767, 1023]:     # lengths around the split and chunk sizes
+        q = torch.randn((1, Hq * D), generator=g, device="cuda")
+        out = pkg.op_attention(q, kc, vc, Hq, Hkv, D, pos, scratch=scratch)
+        assert max_abs_rel(out.cpu().numpy(), ref(q, pos).cpu().numpy()) < 2e-5, pos
+        d_pos = torch.tensor([pos], dtype=torch.int32, device="cuda")
+        out2 = pkg.op_attention(q, kc, vc, Hq, Hkv, D, 0, scratch=scratch, d_pos0=d_pos)
+        assert torch.equal(out, out2)
+    # the kernels leave the arrival counters cleared
+    assert int(scratch[:4 * (Hq + 1)].view(torch.int32).abs().sum()) == 0
+
+
+def test_argmax_first_maximum(pkg):
+    g = torch.Generator(device="cuda").manual_seed(3)
+    scratch = pkg.op_scratch(12)
+    for n in [151936, 1000, 7, 1]:
+        x = torch.randn((n,), generator=g, device="cuda")
+        assert int(pkg.op_argmax(x, scratch)) == int(torch.argmax(x))
+    x = torch.zeros((151936,), device="cuda")
+    x[[70000, 140000, 300]] = 5.0
+    assert int(pkg.op_argmax(x, scratch)) == 300
+    pos = torch.tensor([41], dtype=torch.int32, device="cuda")
+    pkg.op_argmax(x, scratch, d_pos=pos)
+    assert int(pos) == 42
+    assert int(pkg.op_argmax(torch.full((100,), float("-inf"), device="cuda"), scratch)) == 0
+
+
+def tiny_model(rng, H, Hq, Hkv, I, V, layers):
+    def w(n, k):
+        return (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+
+    weights = {"embedding": rng.standard_normal((V, H)).astype(np.float32), "lm_head": w(V, H),
+               "final_norm": (1 + 0.1 * rng.standard_normal(H)).astype(np.float32), "layers": []}
+    for _ in range(layers):
+        weights["layers"].append({
+            "q": w(Hq * 128, H), "k": w(Hkv * 128, H), "v": w(Hkv * 128, H), "o": w(H, Hq * 128),
+            "gate": w(I, H), "up": w(I, H), "down": w(H, I),
+            "q_bias": (0.1 * rng.standard_normal(Hq * 128)).astype(np.float32),
+            "k_bias": (0.1 * rng.standard_normal(Hkv * 128)).astype(np.float32),
+            "v_bias": (0.1 * rng.standard_normal(Hkv * 128)).astype(np.float32),
+            "attn_norm": (1 + 0.1 * rng.standard_normal(H)).astype(np.float32),
+            "ffn_norm": (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)})
+    return weights
+
+
+def to_device_model(pkg, weights, Hq, Hkv, **kw):
+    layers = []
+    for lw in weights["layers"]:
+        d = {}
+        for name in ("q", "k", "v", "o", "gate", "up", "down"):
+            b = lw.get(name + "_bias")
+            d[name] = pkg.quant_pack_rhs(dev(lw[name]), None if b is None else dev(b))
+        d["attn_norm"], d["ffn_norm"] = dev(lw["attn_norm"]), dev(lw["ffn_norm"])
+        layers.append(d)
+    V, H = weights["embedding"].shape
+    return pkg.Decoder(H, Hq, Hkv, weights["layers"][0]["gate"].shape[0], V, layers, dev(weights["embedding"]),
+                       dev(weights["final_norm"]), pkg.quant_pack_rhs(dev(weights["lm_head"])), **kw)
+
+
+def test_decoder_runner_matches_oracle(pkg):
+    import decoder_oracle as do
+
+    rng = np.random.default_rng(4)
+    H, Hq, Hkv, I, V, L = 256, 2, 1, 384, 640, 2
+    weights = tiny_model(rng, H, Hq, Hkv, I, V, L)
+    dec = to_device_model(pkg, weights, Hq, Hkv, max_seq=64, max_batch_tokens=16, rope_theta=1e6)
+    ref = do.Decoder(weights, Hq, Hkv, rope_theta=1e6, max_seq=64)
+
+    prompt = rng.integers(0, V, size=11)
+    tok = dec.prefill(dev(prompt.astype(np.int64)))
+    torch.cuda.synchronize()
+    want = ref.forward(prompt)
+    got = dec.logits.cpu().numpy()
+    assert max_abs_rel(got, want) < 2e-3
+    assert int(tok) == do.greedy(got) and dec.position == 11
+    for step in range(12):
+        fed = int(dec.token)                      # teacher forcing: the oracle consumes the runner's token
+        dec.step()
+        torch.cuda.synchronize()
+        want = ref.forward([fed])
+        got = dec.logits.cpu().numpy()
+        assert max_abs_rel(got, want) < 2e-3, step
+        assert int(dec.token) == do.greedy(got)
+        assert dec.position == 12 + step
+
+
+def test_decoder_step_replays_from_a_graph(pkg):
+    """The decode step's launch sequence does not depend on the position: captured once, replayed
+    per token (with eager work and synchronisations in between), it produces the tokens and logits
+    of eager steps."""
+    rng = np.random.default_rng(5)
+    H, Hq, Hkv, I, V, L = 256, 2, 1, 384, 640, 2
+    weights = tiny_model(rng, H, Hq, Hkv, I, V, L)
+    prompt = dev(rng.integers(0, V, size=9).astype(np.int64))
+
+    eager = to_device_model(pkg, weights, Hq, Hkv, max_seq=64, max_batch_tokens=16)
+    eager.prefill(prompt)
+    toks_e, logits_e = [], []
+    for _ in range(10):
+        eager.step()
+        toks_e.append(int(eager.token))
+        logits_e.append(eager.logits.clone())
+
+    dec = to_device_model(pkg, weights, Hq, Hkv, max_seq=64, max_batch_tokens=16)
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        dec.prefill(prompt)
+        first = dec.token.clone()
+        dec.step()                                # warm-up outside the capture
+        s.synchronize()
+        # rewind: prefill again so the captured step starts from the same state as the eager run
+        dec.prefill(prompt)
+        assert torch.equal(dec.token, first)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            dec.step()
+        # capture does not execute: position is still 9
+        s.synchronize()
+        assert dec.position == 9
+        for i in range(10):
+            graph.replay()
+            s.synchronize()
+            assert int(dec.token) == toks_e[i], i
+            assert torch.equal(dec.logits, logits_e[i]), i
+            _ = (dec.logits * 2).sum().item()     # unrelated eager work between replays
+        assert dec.position == 19
