@@ -57,6 +57,7 @@ def parse():
     ap.add_argument("--eager", action="store_true", help="launch from Python instead of a HIP graph")
     ap.add_argument("--roofline-only", action="store_true",
                     help="only the decode passes (the run profiled under rocprofv3 --kernel-trace)")
+    ap.add_argument("--no-decoder", action="store_true", help="skip the whole-decoder tokens/s leg")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="a 256 MiB copy, then the decode kernel on gate_proj and lm_head and the "
                          "prefill kernel on gate_proj (the run profiled under rocprofv3 --pmc)")
@@ -317,6 +318,60 @@ def main():
                                      "frac": round(best / 2500.0, 4),
                                      "M512_gate_proj_kernel_TFLOPs":
                                          prefill["M512"]["per_shape"]["gate_proj"]["kernel_TFLOPs"]}
+
+    # ---- config 4: the whole decoder (same Linears plus the f32 operators between them), batch 1,
+    # 512-token random-id prompt, then 256 greedy steps replayed from one captured HIP graph
+    if not args.no_decoder:
+        H, V, I = 1536, 151936, 8960
+        dgen = torch.Generator(device="cuda")
+        dgen.manual_seed(2)
+        emb = torch.randn((V, H), generator=dgen, device="cuda")
+        norm = lambda: 1 + 0.1 * torch.randn((H,), generator=dgen, device="cuda")
+        dl = []
+        for layer in layers:
+            d = {n: lin.packed for n, lin in zip(("q", "k", "v", "o", "gate", "up", "down"), layer)}
+            d["attn_norm"], d["ffn_norm"] = norm(), norm()
+            dl.append(d)
+        with torch.cuda.stream(stream):
+            dec = pkg.Decoder(H, 12, 2, I, V, dl, emb, norm(), lm_head.packed, max_seq=1024,
+                              max_batch_tokens=512, rope_theta=1e6, rms_eps=1e-6)
+            prompt = torch.randint(0, V, (512,), generator=dgen, device="cuda", dtype=torch.int64)
+            dec.prefill(prompt)                      # warm-up (allocations, code objects)
+            stream.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            dec.prefill(prompt)
+            e1.record(stream)
+            stream.synchronize()
+            prefill_ms = e0.elapsed_time(e1)
+            first = int(dec.token)
+            dec.step()                               # warm-up of the step, then rewind by prefilling again
+            dec.prefill(prompt)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                dec.step()
+            stream.synchronize()
+            n_new = 256
+            e0.record(stream)
+            for _ in range(n_new):
+                graph.replay()
+            e1.record(stream)
+            stream.synchronize()
+            decode_ms = e0.elapsed_time(e1)
+            assert dec.position == 512 + n_new and first == int(first)
+        extra["decoder_config4"] = {
+            "workload": "28 layers, hidden 1536, 12 q / 2 kv heads x 128, MLP 8960, vocab 151936, rope theta 1e6, "
+                        "f32 KV cache; batch 1, 512 random prompt ids, 256 greedy steps; all Linears W4A32 "
+                        "(lm_head included), random-init weights",
+            "prefill_ms_512_tokens": round(prefill_ms, 2),
+            "prefill_tokens_per_s": round(512 / (prefill_ms * 1e-3), 1),
+            "decode_ms_per_token": round(decode_ms / n_new, 4),
+            "decode_tokens_per_s": round(n_new / (decode_ms * 1e-3), 1),
+            "decode_weight_GBps": round(step_bytes / (decode_ms / n_new * 1e-3) / 1e9, 1),
+            "note": "one decode step = 1 embedding + 28 x 8 + 3 launches, captured once and replayed; "
+                    "positions and cache lengths are read from device memory",
+        }
+        del dec, emb
 
     # ---- CPU baseline: scalar restatement of the reference path, bounded sample
     cpu = None

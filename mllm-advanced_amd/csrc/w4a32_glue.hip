@@ -46,6 +46,25 @@ __device__ __forceinline__ float block_sum(float v, float* s_part) {
   return t;
 }
 
+// Partial results that another workgroup of the same launch will read. The L2s of the XCDs are not
+// coherent with each other for plain accesses, and an agent-scope fence pays for that with a
+// write-back / invalidate of the whole cache; a device-scope store or load of just these words
+// goes to the coherence point directly.
+__device__ __forceinline__ void store_shared_across_wgs(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_shared_across_wgs(int* p, int v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_shared_across_wgs(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ int load_shared_across_wgs(const int* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// All of this wavefront's stores above have reached the coherence point.
+__device__ __forceinline__ void stores_done() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); }
+
 }  // namespace
 
 // ---------------------------------------------------------------------------------------------
@@ -312,6 +331,230 @@ __global__ __launch_bounds__(64) void attention_kernel(const float* __restrict__
 }
 
 // ---------------------------------------------------------------------------------------------
+// Decode attention (one query row): workgroup (x = group of kGW query heads that share a KV head,
+// y = slice of the cached keys), 4 wavefronts per workgroup, each taking a quarter of the slice
+// in blocks of 16 keys.
+//
+// Inside a wavefront 16 lanes share one key: lane (kq, dl) holds dims 8*dl..8*dl+7 of key slot kq,
+// so a block's K and V rows are read as whole 512-byte rows, four rows per load instruction, and
+// all of a block's loads are requested before the first is used. Scores are summed over the 16
+// lanes with DPP adds, the softmax runs online per key slot, and the four slots, the four
+// wavefronts (through LDS) and finally the workgroups of a head group (through `part`, by the last
+// one to arrive) are merged with the usual max / rescale rule.
+// ---------------------------------------------------------------------------------------------
+constexpr int kDecWaves = 4;
+constexpr int kMaxAttnSplit = 32;  // key slices per head group, at most
+
+// v += the same register of the other 15 lanes of the row (all lanes get the row's sum). Callers
+// interleave several independent values per step so that no DPP read follows its write directly.
+#define W4_ROW_ADD(v, ctrl) asm volatile("v_add_f32_dpp %0, %0, %0 " ctrl " row_mask:0xf bank_mask:0xf" : "+v"(v))
+
+template <int kGW>
+__device__ __forceinline__ void row16_sum(float (&d)[kGW]) {
+  asm volatile("s_nop 1");
+#pragma unroll
+  for (int g = 0; g < kGW; ++g) W4_ROW_ADD(d[g], "quad_perm:[1,0,3,2]");
+  if (kGW < 3) asm volatile("s_nop 1");
+#pragma unroll
+  for (int g = 0; g < kGW; ++g) W4_ROW_ADD(d[g], "quad_perm:[2,3,0,1]");
+  if (kGW < 3) asm volatile("s_nop 1");
+#pragma unroll
+  for (int g = 0; g < kGW; ++g) W4_ROW_ADD(d[g], "row_half_mirror");
+  if (kGW < 3) asm volatile("s_nop 1");
+#pragma unroll
+  for (int g = 0; g < kGW; ++g) W4_ROW_ADD(d[g], "row_mirror");
+  asm volatile("s_nop 1");
+}
+
+// (m, l, acc) <- merge with (m2, l2, acc2): softmax partial results over disjoint key sets.
+__device__ __forceinline__ void softmax_merge_weights(float m, float m2, float& w1, float& w2, float& mn) {
+  mn = fmaxf(m, m2);
+  w1 = m == -INFINITY ? 0.0f : __expf(m - mn);
+  w2 = m2 == -INFINITY ? 0.0f : __expf(m2 - mn);
+}
+
+template <int kGW>
+__global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
+    const float* __restrict__ q, const float* __restrict__ kc, const float* __restrict__ vc,
+    float* __restrict__ out, int Hq, int Hkv, int max_seq, const int* __restrict__ d_pos0, int pos0,
+    float scale, float* part, unsigned int* counters) {
+  __shared__ float s_part[kDecWaves][kGW][kPartStride];
+  __shared__ unsigned int s_prev;
+  const int h0 = blockIdx.x * kGW;             // first query head of this group
+  const int hk = h0 / (Hq / Hkv);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int kq = lane >> 4, dl = lane & 15;
+  if (d_pos0) pos0 = *d_pos0;
+  const int len = min(pos0 + 1, max_seq);
+  // keys of this workgroup, then of this wavefront (multiples of 4 so that slots stay aligned)
+  const int per_wg = ((len + (int)gridDim.y - 1) / (int)gridDim.y + 15) / 16 * 16;
+  const int per_wave = per_wg / kDecWaves;
+  const int begin = min((int)blockIdx.y * per_wg + wave * per_wave, len);
+  const int end = min(begin + per_wave, len);
+
+  float qr[kGW][8];
+#pragma unroll
+  for (int g = 0; g < kGW; ++g) {
+    const float4* src = reinterpret_cast<const float4*>(q + (size_t)(h0 + g) * kHeadDim + 8 * dl);
+    const float4 a = src[0], b = src[1];
+    qr[g][0] = a.x; qr[g][1] = a.y; qr[g][2] = a.z; qr[g][3] = a.w;
+    qr[g][4] = b.x; qr[g][5] = b.y; qr[g][6] = b.z; qr[g][7] = b.w;
+  }
+  const float* kbase = kc + (size_t)hk * max_seq * kHeadDim + 8 * dl;
+  const float* vbase = vc + (size_t)hk * max_seq * kHeadDim + 8 * dl;
+
+  float m[kGW], l[kGW], acc[kGW][8];
+#pragma unroll
+  for (int g = 0; g < kGW; ++g) {
+    m[g] = -INFINITY;
+    l[g] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[g][i] = 0.0f;
+  }
+
+  for (int blk = begin; blk < end; blk += 16) {
+    float kk[4][8], vv[4][8];
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int key = blk + 4 * it + kq;
+      const size_t row = (size_t)(key < end ? key : end - 1) * kHeadDim;
+      const float4 a = *reinterpret_cast<const float4*>(kbase + row);
+      const float4 b = *reinterpret_cast<const float4*>(kbase + row + 4);
+      kk[it][0] = a.x; kk[it][1] = a.y; kk[it][2] = a.z; kk[it][3] = a.w;
+      kk[it][4] = b.x; kk[it][5] = b.y; kk[it][6] = b.z; kk[it][7] = b.w;
+    }
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int key = blk + 4 * it + kq;
+      const size_t row = (size_t)(key < end ? key : end - 1) * kHeadDim;
+      const float4 a = *reinterpret_cast<const float4*>(vbase + row);
+      const float4 b = *reinterpret_cast<const float4*>(vbase + row + 4);
+      vv[it][0] = a.x; vv[it][1] = a.y; vv[it][2] = a.z; vv[it][3] = a.w;
+      vv[it][4] = b.x; vv[it][5] = b.y; vv[it][6] = b.z; vv[it][7] = b.w;
+    }
+    float sc[4][kGW];
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      float d[kGW];
+#pragma unroll
+      for (int g = 0; g < kGW; ++g) {
+        float t = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) t += qr[g][i] * kk[it][i];
+        d[g] = t;
+      }
+      row16_sum<kGW>(d);
+      const bool valid = blk + 4 * it + kq < end;
+#pragma unroll
+      for (int g = 0; g < kGW; ++g) sc[it][g] = valid ? d[g] * scale : -INFINITY;
+    }
+#pragma unroll
+    for (int g = 0; g < kGW; ++g) {
+      const float bm = fmaxf(fmaxf(sc[0][g], sc[1][g]), fmaxf(sc[2][g], sc[3][g]));
+      const float mn = fmaxf(m[g], bm);
+      // mn stays -inf only while this slot has seen no valid key: everything it holds is 0
+      const float corr = m[g] == -INFINITY ? 0.0f : __expf(m[g] - mn);
+      l[g] *= corr;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[g][i] *= corr;
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const float p = sc[it][g] == -INFINITY ? 0.0f : __expf(sc[it][g] - mn);
+        l[g] += p;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[g][i] += p * vv[it][i];
+      }
+      m[g] = mn;
+    }
+  }
+
+  // the four key slots of the wavefront -> lanes 0..15
+#pragma unroll
+  for (int g = 0; g < kGW; ++g) {
+#pragma unroll
+    for (int off = 16; off <= 32; off <<= 1) {
+      const float m2 = __shfl_xor(m[g], off, 64);
+      const float l2 = __shfl_xor(l[g], off, 64);
+      float w1, w2, mn;
+      softmax_merge_weights(m[g], m2, w1, w2, mn);
+      l[g] = l[g] * w1 + l2 * w2;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[g][i] = acc[g][i] * w1 + __shfl_xor(acc[g][i], off, 64) * w2;
+      m[g] = mn;
+    }
+    if (kq == 0) {
+      float* dst = &s_part[wave][g][0];
+      if (dl == 0) {
+        dst[0] = m[g];
+        dst[1] = l[g];
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) dst[2 + 8 * dl + i] = acc[g][i];
+    }
+  }
+  __syncthreads();
+
+  // the four wavefronts -> one share per head, thread t: head t / 128, dim t % 128
+  const int ns = gridDim.y;
+  for (int t = threadIdx.x; t < kGW * kHeadDim; t += blockDim.x) {
+    const int g = t / kHeadDim, d = t % kHeadDim;
+    float mm = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kDecWaves; ++w) mm = fmaxf(mm, s_part[w][g][0]);
+    float ll = 0.0f, a = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kDecWaves; ++w) {
+      const float mw = s_part[w][g][0];
+      const float wt = mw == -INFINITY ? 0.0f : __expf(mw - mm);
+      ll += s_part[w][g][1] * wt;
+      a += s_part[w][g][2 + d] * wt;
+    }
+    float* mine = part + ((size_t)(h0 + g) * ns + blockIdx.y) * kPartStride;
+    store_shared_across_wgs(mine + 2 + d, a);
+    if (d == 0) {
+      store_shared_across_wgs(mine, mm);
+      store_shared_across_wgs(mine + 1, ll);
+    }
+  }
+  stores_done();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    s_prev = __hip_atomic_fetch_add(counters + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (s_prev != gridDim.y - 1) return;
+  // Last workgroup of this head group: merge the shares of all key slices. Their (max, sum)
+  // headers go through LDS first so that every thread can weigh its own dim's loads, which are
+  // then independent of each other.
+  __shared__ float s_hdr[kGW][kMaxAttnSplit][2];
+  for (int i = threadIdx.x; i < kGW * ns; i += blockDim.x) {
+    const int g = i / ns, sidx = i % ns;
+    const float* ps = part + ((size_t)(h0 + g) * ns + sidx) * kPartStride;
+    s_hdr[g][sidx][0] = load_shared_across_wgs(ps);
+    s_hdr[g][sidx][1] = load_shared_across_wgs(ps + 1);
+  }
+  __syncthreads();
+  for (int t = threadIdx.x; t < kGW * kHeadDim; t += blockDim.x) {
+    const int g = t / kHeadDim, d = t % kHeadDim;
+    const float* all = part + (size_t)(h0 + g) * ns * kPartStride + 2 + d;
+    float mm = -INFINITY;
+    for (int sidx = 0; sidx < ns; ++sidx) mm = fmaxf(mm, s_hdr[g][sidx][0]);
+    float ll = 0.0f, a = 0.0f;
+#pragma unroll 8
+    for (int sidx = 0; sidx < ns; ++sidx) {
+      const float ms = s_hdr[g][sidx][0];
+      const float wt = ms == -INFINITY ? 0.0f : __expf(ms - mm);
+      ll += s_hdr[g][sidx][1] * wt;
+      a += load_shared_across_wgs(all + (size_t)sidx * kPartStride) * wt;
+    }
+    out[(size_t)(h0 + g) * kHeadDim + d] = a / ll;  // key 0 is always there: ll > 0
+  }
+  if (threadIdx.x == 0) {  // ready for the next launch
+    __hip_atomic_store(counters + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // Greedy argmax over one row of logits: the first maximum wins. Workgroups reduce slices, the
 // last one to finish (arrival counter) reduces the per-workgroup results, writes the token and,
 // when given, advances the position counter of the decoder state.
@@ -349,18 +592,17 @@ __global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ l
     __syncthreads();
   }
   if (threadIdx.x == 0) {
-    part_val[blockIdx.x] = s_val[0];
-    part_idx[blockIdx.x] = s_idx[0];
-    __threadfence();
-    s_prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    store_shared_across_wgs(part_val + blockIdx.x, s_val[0]);
+    store_shared_across_wgs(part_idx + blockIdx.x, s_idx[0]);
+    stores_done();
+    s_prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __syncthreads();
   if (s_prev != gridDim.x - 1) return;
-  __threadfence();
   bv = -INFINITY;
   bi = 0x7fffffff;
   for (int b = threadIdx.x; b < (int)gridDim.x; b += blockDim.x) {
-    argmax_merge(bv, bi, __builtin_nontemporal_load(part_val + b), __builtin_nontemporal_load(part_idx + b));
+    argmax_merge(bv, bi, load_shared_across_wgs(part_val + b), load_shared_across_wgs(part_idx + b));
   }
   s_val[threadIdx.x] = bv;
   s_idx[threadIdx.x] = bi;
@@ -378,7 +620,7 @@ __global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ l
   if (threadIdx.x == 0) {
     const int best = s_idx[0] == 0x7fffffff ? 0 : s_idx[0];  // all -inf / NaN: token 0, as the reference's scan
     *token_out = best;
-    *counter = 0;
+    __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (pos_to_advance) *pos_to_advance += 1;
   }
 }
@@ -443,8 +685,17 @@ hipError_t launch_attention_decode(const float* q, const float* kc, const float*
                                    int Hq, int Hkv, int max_seq, const int* d_pos0, int pos0,
                                    int nsplit, float* part, unsigned int* counters, hipStream_t s) {
   const float scale = 1.0f / sqrtf((float)kHeadDim);
-  hipLaunchKernelGGL(attention_kernel<true>, dim3(Hq, nsplit), dim3(64), 0, s, q, kc, vc, out, Hq, Hkv,
-                     max_seq, d_pos0, pos0, scale, part, counters);
+  const int G = Hq / Hkv;  // query heads per KV head; a workgroup takes 2 or 3 of them when it divides
+  if (G % 2 == 0) {
+    hipLaunchKernelGGL(attention_decode_kernel<2>, dim3(Hq / 2, nsplit), dim3(64 * kDecWaves), 0, s, q, kc,
+                       vc, out, Hq, Hkv, max_seq, d_pos0, pos0, scale, part, counters);
+  } else if (G % 3 == 0) {
+    hipLaunchKernelGGL(attention_decode_kernel<3>, dim3(Hq / 3, nsplit), dim3(64 * kDecWaves), 0, s, q, kc,
+                       vc, out, Hq, Hkv, max_seq, d_pos0, pos0, scale, part, counters);
+  } else {
+    hipLaunchKernelGGL(attention_decode_kernel<1>, dim3(Hq, nsplit), dim3(64 * kDecWaves), 0, s, q, kc, vc,
+                       out, Hq, Hkv, max_seq, d_pos0, pos0, scale, part, counters);
+  }
   return hipGetLastError();
 }
 

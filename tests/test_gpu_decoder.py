@@ -77,7 +77,7 @@ def test_rope_table_and_kv_append(pkg):
     assert torch.equal(kc2, kc) and torch.equal(vc2, vc) and torch.equal(dq2, dq)
 
 
-@pytest.mark.parametrize("Hq,Hkv", [(12, 2), (4, 4), (2, 1)])
+@pytest.mark.parametrize("Hq,Hkv", [(12, 2), (4, 4), (2, 1), (3, 1)])
 def test_attention_prefill_and_decode(pkg, Hq, Hkv):
     g = torch.Generator(device="cuda").manual_seed(2)
     D, S = 128, 1024
