@@ -67,6 +67,29 @@ int w4a32_op_attention(const float* d_q, const float* d_kcache, const float* d_v
 int w4a32_op_argmax(const float* d_logits, int n, void* d_scratch, int64_t* d_token,
                     int* d_pos_to_advance, void* stream);
 
+/* One decode row (M = 1) through 1..4 W4A32 Linears that share it, with the operators around them
+ * folded into the same launch:
+ *   in front  (d_norm_weight != NULL): row = d_x + d_delta (d_delta may be NULL; the sum is also stored
+ *             to d_sum_out when that is not NULL - it must not alias d_x), then RMSNorm with d_norm_weight;
+ *   behind    (silu_pair != 0, count == 2, N[0] == N[1]): d_y[0] = silu(linear0) * linear1, d_y[1] unused.
+ * The fusions of QWenDecoder::forward / QWenMLP::forward (modeling_ds_qwen2.hpp:47-54,175-183) that cost a
+ * launch each when run as separate operators. Returns W4A32_ENOTSUP when the shape does not fit the
+ * single-launch kernel (the caller then runs the operators one by one). */
+typedef struct {
+  const float* d_x;
+  const float* d_delta;
+  float* d_sum_out;
+  const float* d_norm_weight;
+  float norm_eps;
+  int K;
+  int count;
+  const void* d_packed[4];
+  int N[4];
+  float* d_y[4];
+  int silu_pair;
+} w4a32_decode_linear_args;
+int w4a32_decode_linear(const w4a32_decode_linear_args* args, void* stream);
+
 /* ---- decoder runner -------------------------------------------------------------------- */
 
 typedef struct {

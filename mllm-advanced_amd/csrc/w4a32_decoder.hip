@@ -170,6 +170,88 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
   return W4A32_OK;
 }
 
+// One decode row with the operators between the Linears folded into them: 6 launches per layer
+// ([add+norm+q,k,v] [rope+cache] [attention] [o] [add+norm+gate,up+silu*mul] [down]) instead of 9.
+// The residual stream alternates between two buffers because the launch that completes a row
+// (x + delta) is read by every workgroup while one of them stores the sum.
+bool decode_fusable(const w4a32_decoder_config* c) {
+  const int qd = c->n_heads * c->head_dim, kvd = c->n_kv_heads * c->head_dim;
+  const int qkv[3] = {qd, kvd, kvd}, gu[2] = {c->intermediate, c->intermediate};
+  const int o[1] = {c->hidden}, head[1] = {c->vocab};
+  return w4::gemv_decode_applies(c->hidden, qkv, 3, false) && w4::gemv_decode_applies(c->hidden, gu, 2, true) &&
+         w4::gemv_decode_applies(qd, o, 1, false) && w4::gemv_decode_applies(c->intermediate, o, 1, false) &&
+         w4::gemv_decode_applies(c->hidden, head, 1, false);
+}
+
+int run_decode_fused(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, uint8_t* st,
+                     const StateGeom& g, int64_t* d_token_out, void* stream) {
+  hipStream_t s = S(stream);
+  const int H = c->hidden, I = c->intermediate, D = c->head_dim;
+  const int Hq = c->n_heads, Hkv = c->n_kv_heads, qd = Hq * D, kvd = Hkv * D;
+  int* d_pos = reinterpret_cast<int*>(st + g.pos_off);
+  uint8_t* scratch = st + g.scratch_off;
+  const ScratchGeom sg = scratch_geom(Hq);
+  float* hcur = reinterpret_cast<float*>(st + g.h_off);    // the embedding was written here
+  float* hnext = reinterpret_cast<float*>(st + g.xn_off);
+  float* q = reinterpret_cast<float*>(st + g.q_off);
+  float* k = reinterpret_cast<float*>(st + g.k_off);
+  float* v = reinterpret_cast<float*>(st + g.v_off);
+  float* attn = reinterpret_cast<float*>(st + g.attn_off);
+  float* delta = reinterpret_cast<float*>(st + g.delta_off);
+  float* act = reinterpret_cast<float*>(st + g.act_off);
+  float* logits = reinterpret_cast<float*>(st + g.logits_off);
+  const float* sin_t = reinterpret_cast<const float*>(st + g.sin_off);
+  const float* cos_t = reinterpret_cast<const float*>(st + g.cos_off);
+
+  auto one = [&](const float* x, const void* packed, int K, int N, float* y) {
+    const uint8_t* pk[1] = {static_cast<const uint8_t*>(packed)};
+    float* ys[1] = {y};
+    const int ns[1] = {N};
+    return from_hip(w4::launch_gemv_decode(ys, x, pk, ns, 1, K, nullptr, nullptr, nullptr, 0.0f, false, s));
+  };
+
+  for (int l = 0; l < c->n_layers; ++l) {
+    const w4a32_layer_weights& lw = w->layers[l];
+    float* kc = reinterpret_cast<float*>(st + g.kcache_off) + (size_t)l * g.cache_layer;
+    float* vc = reinterpret_cast<float*>(st + g.vcache_off) + (size_t)l * g.cache_layer;
+    {
+      const uint8_t* pk[3] = {static_cast<const uint8_t*>(lw.q), static_cast<const uint8_t*>(lw.k),
+                              static_cast<const uint8_t*>(lw.v)};
+      float* ys[3] = {q, k, v};
+      const int ns[3] = {qd, kvd, kvd};
+      W4_TRY(from_hip(w4::launch_gemv_decode(ys, hcur, pk, ns, 3, H, l == 0 ? nullptr : delta,
+                                             l == 0 ? nullptr : hnext, lw.attn_norm, c->rms_eps, false, s)));
+      if (l != 0) std::swap(hcur, hnext);
+    }
+    W4_TRY(from_hip(w4::launch_rope_kv(q, k, v, sin_t, cos_t, kc, vc, 1, Hq, Hkv, D, c->max_seq, d_pos, 0, s)));
+    W4_TRY(from_hip(w4::launch_attention_decode(
+        q, kc, vc, attn, Hq, Hkv, c->max_seq, d_pos, 0, kAttnSplit,
+        reinterpret_cast<float*>(scratch + sg.part_off),
+        reinterpret_cast<unsigned int*>(scratch + sg.counters_off), s)));
+    W4_TRY(one(attn, lw.o, qd, H, delta));
+    {
+      const uint8_t* pk[2] = {static_cast<const uint8_t*>(lw.gate), static_cast<const uint8_t*>(lw.up)};
+      float* ys[2] = {act, nullptr};
+      const int ns[2] = {I, I};
+      W4_TRY(from_hip(w4::launch_gemv_decode(ys, hcur, pk, ns, 2, H, delta, hnext, lw.ffn_norm, c->rms_eps,
+                                             true, s)));
+      std::swap(hcur, hnext);
+    }
+    W4_TRY(one(act, lw.down, I, H, delta));
+  }
+  {
+    const uint8_t* pk[1] = {static_cast<const uint8_t*>(w->lm_head)};
+    float* ys[1] = {logits};
+    const int ns[1] = {c->vocab};
+    W4_TRY(from_hip(w4::launch_gemv_decode(ys, hcur, pk, ns, 1, H, delta, nullptr, w->final_norm, c->rms_eps,
+                                           false, s)));
+  }
+  return from_hip(w4::launch_argmax(logits, c->vocab, reinterpret_cast<float*>(scratch + sg.amax_val_off),
+                                    reinterpret_cast<int*>(scratch + sg.amax_idx_off),
+                                    reinterpret_cast<unsigned int*>(scratch + sg.counters_off) + Hq,
+                                    d_token_out, d_pos, kArgmaxBlocks, s));
+}
+
 }  // namespace
 
 extern "C" {
@@ -257,6 +339,24 @@ int w4a32_op_argmax(const float* d_logits, int n, void* d_scratch, int64_t* d_to
                                     d_pos_to_advance, kArgmaxBlocks, S(stream)));
 }
 
+int w4a32_decode_linear(const w4a32_decode_linear_args* a, void* stream) {
+  if (!a || !a->d_x || a->count < 1 || a->count > 4 || a->K <= 0) return W4A32_EINVAL;
+  if (a->K % 32 != 0) return W4A32_ESHAPE;
+  if (a->d_sum_out && (!a->d_delta || !a->d_norm_weight || a->d_sum_out == a->d_x)) return W4A32_EINVAL;
+  if (a->d_delta && !a->d_norm_weight) return W4A32_EINVAL;
+  const bool pair = a->silu_pair != 0;
+  const uint8_t* pk[4];
+  for (int i = 0; i < a->count; ++i) {
+    if (!a->d_packed[i] || a->N[i] <= 0) return W4A32_EINVAL;
+    if (!a->d_y[i] && !(pair && i == 1)) return W4A32_EINVAL;
+    pk[i] = static_cast<const uint8_t*>(a->d_packed[i]);
+  }
+  if (reinterpret_cast<uintptr_t>(a->d_x) % 16 != 0) return W4A32_EINVAL;
+  if (!w4::gemv_decode_applies(a->K, a->N, a->count, pair)) return W4A32_ENOTSUP;
+  return from_hip(w4::launch_gemv_decode(a->d_y, a->d_x, pk, a->N, a->count, a->K, a->d_delta,
+                                         a->d_sum_out, a->d_norm_weight, a->norm_eps, pair, S(stream)));
+}
+
 size_t w4a32_decoder_state_bytes(const w4a32_decoder_config* cfg) {
   return config_ok(cfg) ? state_geom(cfg).total : 0;
 }
@@ -310,6 +410,7 @@ int w4a32_decoder_step(const w4a32_decoder_config* cfg, const w4a32_decoder_weig
   uint8_t* st = static_cast<uint8_t*>(d_state);
   W4_TRY(from_hip(w4::launch_embedding(d_token_in, w->embedding, 1, cfg->hidden, cfg->vocab,
                                        reinterpret_cast<float*>(st + g.h_off), S(stream))));
+  if (decode_fusable(cfg)) return run_decode_fused(cfg, w, st, g, d_token_out, stream);
   return run_layers(cfg, w, st, g, 1, d_token_out, true, stream);
 }
 

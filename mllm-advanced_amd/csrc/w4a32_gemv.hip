@@ -203,6 +203,12 @@ __device__ __forceinline__ T load_global(const void* p) {
 // Up to kMaxGroup Linears that share their activation rows (and therefore K), run by one launch:
 // workgroup b serves tile row b - first[i] of Linear i, where first[] are running sums of tile rows.
 constexpr int kMaxGroup = 4;
+struct RowPrologue {
+  const float* delta;   // optional: added to x before anything else
+  float* sum_out;       // optional: receives x + delta (must not alias x)
+  const float* norm_w;  // RMSNorm weight [K]
+  float eps;
+};
 struct GroupArgs {
   const uint8_t* packed[kMaxGroup];
   float* y[kMaxGroup];
@@ -221,11 +227,18 @@ struct GroupArgs {
 // Nearly every instruction here is executed once per wavefront and depends on the one before, so
 // the kernel's duration at decode sizes is its instruction count times the issue latency: the
 // reductions use one DPP instruction per step and the quantiser four VALU instructions per value.
-template <int M, int kFusedR, bool kGrouped, int kCPW>
+//
+// kNorm: the row is first completed and normalised, as the decoder does between its blocks:
+//   x <- x + delta (when delta is given; workgroup 0 also stores the sum to sum_out),
+//   x <- x * (norm_w * 1/sqrt(mean(x^2) + eps))       (the RMSNorm kernel's arithmetic)
+// kPair: exactly two Linears of the same N (gate, up): a workgroup multiplies tile row nt of both
+//   and stores silu(y0) * y1 to y[0].
+template <int M, int kFusedR, bool kGrouped, int kCPW, bool kNorm, bool kPair>
 __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(const GroupArgs ga,
                                                           const float* __restrict__ x, int ldx,
-                                                          int K, int KC) {
+                                                          int K, int KC, const RowPrologue pro) {
   extern __shared__ __align__(16) uint8_t smem[];
+  constexpr int kSets = kPair ? 2 : 1;  // weight matrices a workgroup multiplies
   const uint8_t* packed = ga.packed[0];
   float* y = ga.y[0];
   int N = ga.N[0], nt_first = 0;
@@ -256,12 +269,12 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(const G
   }
   const int NT = (N + kTileRows - 1) / kTileRows;
   const float* rsum = reinterpret_cast<const float*>(packed + (size_t)NT * KC * kTileBytes);
-  const float* bias = rsum + NT * kTileRows;
   const int Kp = KC * kTileK;
   const int W = blockDim.x >> 6;
   int8_t* s_a = reinterpret_cast<int8_t*>(smem);                          // [M][Kp]
-  float* s_red = reinterpret_cast<float*>(smem + (size_t)M * Kp);         // [W][M][16]
-  float2* s_mm = reinterpret_cast<float2*>(s_red + W * M * 16);     // [W][M] (min, max)
+  float* s_red = reinterpret_cast<float*>(smem + (size_t)M * Kp);         // [W][kSets][M][16]
+  float2* s_mm = reinterpret_cast<float2*>(s_red + W * kSets * M * 16);   // [W][M] (min, max)
+  float* s_ss = reinterpret_cast<float*>(s_mm + W * M);                   // [W][M] sums of squares
 
   const int nt = (int)blockIdx.x - nt_first;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -285,24 +298,98 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(const G
       for (int e = 0; e < 8; ++e) xv[m][r][e] = f[e];
     }
   }
-  u32x4 wq[kCPW];
-  u32x2 sc[kCPW];
-  const uint8_t* tiles = packed + (size_t)nt * KC * kTileBytes;
+  float dv[kNorm ? M : 1][kNorm ? kFusedR : 1][8];  // delta, then the norm weight
+  if (kNorm && pro.delta) {
 #pragma unroll
-  for (int i = 0; i < kCPW; ++i) {
-    const int kc = wave + i * W < KC ? wave + i * W : KC - 1;  // masked where used
-    wq[i] = load_global<u32x4>(tiles + (size_t)kc * kTileBytes + 16 * lane);
-    sc[i] = load_global<u32x2>(tiles + (size_t)kc * kTileBytes + kTileQBytes + 8 * j);
+    for (int m = 0; m < M; ++m) {
+      const float* row = pro.delta + (size_t)m * ldx;
+#pragma unroll
+      for (int r = 0; r < kFusedR; ++r) {
+        const int c = threadIdx.x + r * blockDim.x;
+        const int cc = c < groups ? c : groups - 1;
+        const float4 v0 = *reinterpret_cast<const float4*>(row + 8 * cc);
+        const float4 v1 = *reinterpret_cast<const float4*>(row + 8 * cc + 4);
+        const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dv[m][r][e] = f[e];
+      }
+    }
+  }
+  u32x4 wq[kSets][kCPW];
+  u32x2 sc[kSets][kCPW];
+#pragma unroll
+  for (int st = 0; st < kSets; ++st) {
+    const uint8_t* tiles = (st == 0 ? packed : ga.packed[1]) + (size_t)nt * KC * kTileBytes;
+#pragma unroll
+    for (int i = 0; i < kCPW; ++i) {
+      const int kc = wave + i * W < KC ? wave + i * W : KC - 1;  // masked where used
+      wq[st][i] = load_global<u32x4>(tiles + (size_t)kc * kTileBytes + 16 * lane);
+      sc[st][i] = load_global<u32x2>(tiles + (size_t)kc * kTileBytes + kTileQBytes + 8 * j);
+    }
   }
   // Output o = m * 16 + jj belongs to thread o when the workgroup has that many threads; its
   // rsum / bias are requested now so the epilogue does not wait on memory.
   constexpr int kOutputs = M * 16;
-  float rs = 0.0f, bs = 0.0f;
-  {
+  float rs[kSets], bs[kSets];
+#pragma unroll
+  for (int st = 0; st < kSets; ++st) {
+    rs[st] = 0.0f;
+    bs[st] = 0.0f;
     const int n = kTileRows * nt + j;
     if (threadIdx.x < kOutputs && n < N) {
-      rs = load_global<float>(rsum + n);
-      bs = load_global<float>(bias + n);
+      const float* rsp = st == 0 ? rsum : reinterpret_cast<const float*>(ga.packed[1] + (size_t)NT * KC * kTileBytes);
+      rs[st] = load_global<float>(rsp + n);
+      bs[st] = load_global<float>(rsp + NT * kTileRows + n);
+    }
+  }
+
+  if (kNorm) {
+    // complete the row, sum its squares, normalise: all before the quantiser sees it
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      float ss = 0.0f;
+#pragma unroll
+      for (int r = 0; r < kFusedR; ++r) {
+        const int c = threadIdx.x + r * blockDim.x;
+        if (pro.delta) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) xv[m][r][e] += dv[m][r][e];
+          if (pro.sum_out && blockIdx.x == 0 && c < groups) {
+            float* dst = pro.sum_out + (size_t)m * ldx + 8 * c;
+            *reinterpret_cast<float4*>(dst) = make_float4(xv[m][r][0], xv[m][r][1], xv[m][r][2], xv[m][r][3]);
+            *reinterpret_cast<float4*>(dst + 4) = make_float4(xv[m][r][4], xv[m][r][5], xv[m][r][6], xv[m][r][7]);
+          }
+        }
+        if (c < groups) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) ss += xv[m][r][e] * xv[m][r][e];
+        }
+      }
+      ss = wave_sum_to_lane63(ss);
+      if (lane == 63) s_ss[wave * M + m] = ss;
+    }
+    // the norm weight travels while the partial sums meet
+#pragma unroll
+    for (int r = 0; r < kFusedR; ++r) {
+      const int c = threadIdx.x + r * blockDim.x;
+      const int cc = c < groups ? c : groups - 1;
+      const float4 v0 = *reinterpret_cast<const float4*>(pro.norm_w + 8 * cc);
+      const float4 v1 = *reinterpret_cast<const float4*>(pro.norm_w + 8 * cc + 4);
+      const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dv[0][r][e] = f[e];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      const float part = j < W ? s_ss[j * M + m] : 0.0f;
+      const float total = row16_sum_all(part);
+      const float rstd = 1.0f / sqrtf(total / (float)K + pro.eps);
+#pragma unroll
+      for (int r = 0; r < kFusedR; ++r) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xv[m][r][e] = xv[m][r][e] * (dv[0][r][e] * rstd);
+      }
     }
   }
 
@@ -347,9 +434,11 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(const G
   }
   __syncthreads();
 
-  float acc[M];
+  float acc[kSets][M];
 #pragma unroll
-  for (int m = 0; m < M; ++m) acc[m] = 0.0f;
+  for (int st = 0; st < kSets; ++st)
+#pragma unroll
+    for (int m = 0; m < M; ++m) acc[st][m] = 0.0f;
 #pragma unroll
   for (int i = 0; i < kCPW; ++i) {
     const bool valid = wave + i * W < KC;
@@ -360,27 +449,33 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(const G
       int2 a[M];
 #pragma unroll
       for (int m = 0; m < M; ++m) a[m] = *reinterpret_cast<const int2*>(a_base + (size_t)m * Kp);
-      const uint32_t wv = wq[i][d];
-      const uint32_t sw = sc[i][d >> 1];
-      const uint32_t sbits = valid ? ((d & 1) ? (sw & 0xFFFF0000u) : (sw << 16)) : 0u;
-      const float sv = __uint_as_float(sbits);
-      const int lo = (int)((wv << 4) & 0xF0F0F0F0u);  // 16*q at k offsets 0..3
-      const int hi = (int)(wv & 0xF0F0F0F0u);         // 16*q at k offsets 4..7
 #pragma unroll
-      for (int m = 0; m < M; ++m) {
-        int dot = __builtin_amdgcn_sdot4(a[m].x, lo, 0, false);
-        dot = __builtin_amdgcn_sdot4(a[m].y, hi, dot, false);
-        acc[m] = __fmaf_rn((float)dot, sv, acc[m]);
+      for (int st = 0; st < kSets; ++st) {
+        const uint32_t wv = wq[st][i][d];
+        const uint32_t sw = sc[st][i][d >> 1];
+        const uint32_t sbits = valid ? ((d & 1) ? (sw & 0xFFFF0000u) : (sw << 16)) : 0u;
+        const float sv = __uint_as_float(sbits);
+        const int lo = (int)((wv << 4) & 0xF0F0F0F0u);  // 16*q at k offsets 0..3
+        const int hi = (int)(wv & 0xF0F0F0F0u);         // 16*q at k offsets 4..7
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+          int dot = __builtin_amdgcn_sdot4(a[m].x, lo, 0, false);
+          dot = __builtin_amdgcn_sdot4(a[m].y, hi, dot, false);
+          acc[st][m] = __fmaf_rn((float)dot, sv, acc[st][m]);
+        }
       }
     }
   }
   // Sum the four k-groups of a row (lanes j, j+16, j+32, j+48), then across wavefronts via LDS.
 #pragma unroll
-  for (int m = 0; m < M; ++m) {
-    float v = acc[m];
-    v += __shfl_xor(v, 16, 64);
-    v += __shfl_xor(v, 32, 64);
-    if (lane < 16) s_red[(wave * M + m) * 16 + lane] = v;
+  for (int st = 0; st < kSets; ++st) {
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      float v = acc[st][m];
+      v += __shfl_xor(v, 16, 64);
+      v += __shfl_xor(v, 32, 64);
+      if (lane < 16) s_red[((wave * kSets + st) * M + m) * 16 + lane] = v;
+    }
   }
   __syncthreads();
 
@@ -390,9 +485,6 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(const G
     const int m = o >> 4;
     const int n = kTileRows * nt + (o & 15);
     if (n < N) {
-      float s = 0.0f;
-#pragma unroll 4
-      for (int w = 0; w < W; ++w) s += s_red[w * kOutputs + o];
       float rcp = 0.0f;
       int off = 0;
 #pragma unroll
@@ -402,11 +494,21 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(const G
           off = -par[mm].zp;
         }
       }
-      const float rsn = prefetched ? rs : load_global<float>(rsum + n);
-      const float bsn = prefetched ? bs : load_global<float>(bias + n);
-      float v = __fmaf_rn((float)off, rsn, s * 0.0625f);
-      v = __fmaf_rn(v, rcp, bsn);
-      v = fminf(fmaxf(v, -3.402823466e+38f), 3.402823466e+38f);
+      float res[kSets];
+#pragma unroll
+      for (int st = 0; st < kSets; ++st) {
+        float s = 0.0f;
+#pragma unroll 4
+        for (int w = 0; w < W; ++w) s += s_red[(w * kSets + st) * kOutputs + o];
+        const float* rsp = st == 0 ? rsum : reinterpret_cast<const float*>(ga.packed[1] + (size_t)NT * KC * kTileBytes);
+        const float rsn = prefetched ? rs[st] : load_global<float>(rsp + n);
+        const float bsn = prefetched ? bs[st] : load_global<float>(rsp + NT * kTileRows + n);
+        float v = __fmaf_rn((float)off, rsn, s * 0.0625f);
+        v = __fmaf_rn(v, rcp, bsn);
+        res[st] = fminf(fmaxf(v, -3.402823466e+38f), 3.402823466e+38f);
+      }
+      float v = res[0];
+      if (kPair) v = res[0] / (1.0f + expf(-res[0])) * res[kSets - 1];  // silu(gate) * up
       *(W4_GLOBAL float*)(y + (size_t)m * N + n) = v;
     }
   }
@@ -474,23 +576,24 @@ static FusedPlan fused_plan(int M, int K) {
   return FusedPlan{0, 0, 0};
 }
 
-template <int M, int R, int CPW>
+template <int M, int R, int CPW, bool kNorm, bool kPair>
 static hipError_t launch_fused_m(const GroupArgs& ga, const float* x, int ldx, int K, int W,
-                                 hipStream_t s) {
+                                 const RowPrologue& pro, hipStream_t s) {
   const int KC = (K + kTileK - 1) / kTileK;
   const int Kp = KC * kTileK;
-  const size_t lds = (size_t)M * Kp + (size_t)W * M * 16 * sizeof(float) +
-                     (size_t)W * M * 2 * sizeof(float);
-  const dim3 grid(ga.first[ga.count]), block(64 * W);
+  const int sets = kPair ? 2 : 1;
+  const size_t lds = (size_t)M * Kp + (size_t)W * sets * M * 16 * sizeof(float) +
+                     (size_t)W * M * 3 * sizeof(float);
+  const dim3 grid(kPair ? ga.first[1] : ga.first[ga.count]), block(64 * W);
   static bool raised1 = false, raisedg = false;
-  if (ga.count == 1) {
-    auto kern = gemv_fused_kernel<M, R, false, CPW>;
+  if (ga.count == 1 || kPair) {
+    auto kern = gemv_fused_kernel<M, R, false, CPW, kNorm, kPair>;
     if (hipError_t e = raise_lds_limit(kern, lds, &raised1); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, grid, block, lds, s, ga, x, ldx, K, KC);
+    hipLaunchKernelGGL(kern, grid, block, lds, s, ga, x, ldx, K, KC, pro);
   } else {
-    auto kern = gemv_fused_kernel<M, R, true, CPW>;
+    auto kern = gemv_fused_kernel<M, R, true, CPW, kNorm, false>;
     if (hipError_t e = raise_lds_limit(kern, lds, &raisedg); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, grid, block, lds, s, ga, x, ldx, K, KC);
+    hipLaunchKernelGGL(kern, grid, block, lds, s, ga, x, ldx, K, KC, pro);
   }
   return hipGetLastError();
 }
@@ -504,12 +607,13 @@ constexpr int kWideDepth = 4;        // chunk loads a wavefront keeps in flight
 
 // kFused: quantise x (f32, K <= 8 * 64 * kWideWaves so one group of 8 per thread and row
 // suffices) into LDS first; otherwise copy the already quantised rows from the workspace.
-template <int M, bool kFused>
+// kNorm (with kFused): residual add + RMSNorm of the row first, as in gemv_fused_kernel.
+template <int M, bool kFused, bool kNorm>
 __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
     float* __restrict__ y, const float* __restrict__ x, int ldx, const int8_t* __restrict__ aq,
     const float* __restrict__ recip, const int32_t* __restrict__ negzp,
     const uint8_t* __restrict__ packed, int N, int K, int NT, int KC, const float* __restrict__ rsum,
-    const float* __restrict__ bias) {
+    const float* __restrict__ bias, const RowPrologue pro) {
   extern __shared__ __align__(16) uint8_t smem[];
   const int Kp = KC * kTileK;
   int8_t* s_a = reinterpret_cast<int8_t*>(smem);                   // [M][Kp]
@@ -549,7 +653,38 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
       const float* src = x + (size_t)m * ldx + 8 * c;
       const float4 v0 = *reinterpret_cast<const float4*>(src);
       const float4 v1 = *reinterpret_cast<const float4*>(src + 4);
-      const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+      float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+      if (kNorm) {
+        if (pro.delta) {
+          const float* dsrc = pro.delta + (size_t)m * ldx + 8 * c;
+          const float4 d0 = *reinterpret_cast<const float4*>(dsrc);
+          const float4 d1 = *reinterpret_cast<const float4*>(dsrc + 4);
+          const float dd[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
+#pragma unroll
+          for (int e = 0; e < 8; ++e) f[e] += dd[e];
+          if (pro.sum_out && blockIdx.x == 0 && (int)threadIdx.x < groups) {
+            float* dst = pro.sum_out + (size_t)m * ldx + 8 * c;
+            *reinterpret_cast<float4*>(dst) = make_float4(f[0], f[1], f[2], f[3]);
+            *reinterpret_cast<float4*>(dst + 4) = make_float4(f[4], f[5], f[6], f[7]);
+          }
+        }
+        const float4 w0 = *reinterpret_cast<const float4*>(pro.norm_w + 8 * c);
+        const float4 w1 = *reinterpret_cast<const float4*>(pro.norm_w + 8 * c + 4);
+        const float ww[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+        float ss = 0.0f;
+        if ((int)threadIdx.x < groups) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
+        }
+        ss = wave_sum_to_lane63(ss);
+        float* s_ss = s_mm + 2 * kWideWaves * M;
+        if (lane == 63) s_ss[wave * M + m] = ss;
+        __syncthreads();
+        const float total = row16_sum_all(j < kWideWaves ? s_ss[j * M + m] : 0.0f);
+        const float rstd = 1.0f / sqrtf(total / (float)K + pro.eps);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = f[e] * (ww[e] * rstd);
+      }
       float lo = f[0], hi = f[0];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
@@ -665,13 +800,13 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
   }
 }
 
-template <int M, bool kFused>
+template <int M, bool kFused, bool kNorm>
 static hipError_t launch_wide(float* y, const float* x, int ldx, const uint8_t* ws,
-                              const uint8_t* packed, int K, int N, hipStream_t s) {
+                              const uint8_t* packed, int K, int N, const RowPrologue& pro, hipStream_t s) {
   const WeightGeom g = weight_geom(N, K);
   const WsGeom w = ws_geom(M, K);
-  const size_t lds = (size_t)M * g.Kp + (size_t)kWideWaves * M * 2 * sizeof(float);
-  auto kern = gemv_wide_kernel<M, kFused>;
+  const size_t lds = (size_t)M * g.Kp + (size_t)kWideWaves * M * 3 * sizeof(float);
+  auto kern = gemv_wide_kernel<M, kFused, kNorm>;
   static bool raised = false;
   if (hipError_t e = raise_lds_limit(kern, lds, &raised); e != hipSuccess) return e;
   // 4 workgroups of 4 wavefronts per CU; every wavefront then walks NT / 4096 tile rows
@@ -681,7 +816,7 @@ static hipError_t launch_wide(float* y, const float* x, int ldx, const uint8_t* 
                      ws ? reinterpret_cast<const float*>(ws + w.scale_off) : nullptr,
                      ws ? reinterpret_cast<const int32_t*>(ws + w.off_off) : nullptr, packed, N, K,
                      g.NT, g.KC, reinterpret_cast<const float*>(packed + g.rsum_off),
-                     reinterpret_cast<const float*>(packed + g.bias_off));
+                     reinterpret_cast<const float*>(packed + g.bias_off), pro);
   return hipGetLastError();
 }
 
@@ -706,7 +841,7 @@ static bool wide_applies(int K, int N) {
 hipError_t launch_gemv(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                        hipStream_t s) {
   if (wide_applies(K, N)) {
-#define W4_CALL(m) (launch_wide<m, false>(y, nullptr, 0, ws, packed, K, N, s))
+#define W4_CALL(m) (launch_wide<m, false, false>(y, nullptr, 0, ws, packed, K, N, RowPrologue{nullptr, nullptr, nullptr, 0.0f}, s))
     W4_DISPATCH_M(W4_CALL)
 #undef W4_CALL
   }
@@ -724,15 +859,15 @@ bool gemv_fused_applies(int M, int K, int N) {
   return fused_plan(M, K).W != 0;
 }
 
-template <int M, int R>
+template <int M, int R, bool kNorm, bool kPair>
 static hipError_t launch_fused_cpw(const GroupArgs& ga, const float* x, int ldx, int K,
-                                   const FusedPlan& p, hipStream_t s) {
-#define W4_CASE(c)                                                  \
-  case c:                                                           \
-    if constexpr (fused_shape_ok(M, c)) {                           \
-      return launch_fused_m<M, R, c>(ga, x, ldx, K, p.W, s);        \
-    } else {                                                        \
-      return hipErrorInvalidValue;                                  \
+                                   const FusedPlan& p, const RowPrologue& pro, hipStream_t s) {
+#define W4_CASE(c)                                                                  \
+  case c:                                                                           \
+    if constexpr (fused_shape_ok(M, c) && (!kPair || c <= 3)) {                     \
+      return launch_fused_m<M, R, c, kNorm, kPair>(ga, x, ldx, K, p.W, pro, s);     \
+    } else {                                                                        \
+      return hipErrorInvalidValue;                                                  \
     }
   switch (p.CPW) {
     W4_CASE(1)
@@ -745,15 +880,29 @@ static hipError_t launch_fused_cpw(const GroupArgs& ga, const float* x, int ldx,
 #undef W4_CASE
 }
 
+// norm / pair: decode extras, M = 1 only (see gemv_decode_applies)
 static hipError_t launch_fused_group(const GroupArgs& ga, const float* x, int ldx, int M, int K,
-                                     hipStream_t s) {
+                                     const RowPrologue* pro, bool pair, hipStream_t s) {
   const FusedPlan p = fused_plan(M, K);
   if (p.W == 0) return hipErrorInvalidValue;
+  const RowPrologue none{nullptr, nullptr, nullptr, 0.0f};
+  if (pro || pair) {
+    if (M != 1) return hipErrorInvalidValue;
+    const RowPrologue& pr = pro ? *pro : none;
+    if (p.R == 2) {
+      if (pro && pair) return launch_fused_cpw<1, 2, true, true>(ga, x, ldx, K, p, pr, s);
+      if (pro) return launch_fused_cpw<1, 2, true, false>(ga, x, ldx, K, p, pr, s);
+      return launch_fused_cpw<1, 2, false, true>(ga, x, ldx, K, p, pr, s);
+    }
+    if (pro && pair) return launch_fused_cpw<1, 1, true, true>(ga, x, ldx, K, p, pr, s);
+    if (pro) return launch_fused_cpw<1, 1, true, false>(ga, x, ldx, K, p, pr, s);
+    return launch_fused_cpw<1, 1, false, true>(ga, x, ldx, K, p, pr, s);
+  }
   if (p.R == 2) {
     if (M != 1) return hipErrorInvalidValue;
-    return launch_fused_cpw<1, 2>(ga, x, ldx, K, p, s);
+    return launch_fused_cpw<1, 2, false, false>(ga, x, ldx, K, p, none, s);
   }
-#define W4_CALL(m) (launch_fused_cpw<m, 1>(ga, x, ldx, K, p, s))
+#define W4_CALL(m) (launch_fused_cpw<m, 1, false, false>(ga, x, ldx, K, p, none, s))
   W4_DISPATCH_M(W4_CALL)
 #undef W4_CALL
 }
@@ -761,7 +910,7 @@ static hipError_t launch_fused_group(const GroupArgs& ga, const float* x, int ld
 hipError_t launch_gemv_fused(float* y, const float* x, int ldx, const uint8_t* packed, int M, int K,
                              int N, hipStream_t s) {
   if (wide_applies(K, N)) {
-#define W4_CALL(m) (launch_wide<m, true>(y, x, ldx, nullptr, packed, K, N, s))
+#define W4_CALL(m) (launch_wide<m, true, false>(y, x, ldx, nullptr, packed, K, N, RowPrologue{nullptr, nullptr, nullptr, 0.0f}, s))
     W4_DISPATCH_M(W4_CALL)
 #undef W4_CALL
   }
@@ -772,7 +921,7 @@ hipError_t launch_gemv_fused(float* y, const float* x, int ldx, const uint8_t* p
   ga.first[0] = 0;
   ga.first[1] = (N + kTileRows - 1) / kTileRows;
   ga.count = 1;
-  return launch_fused_group(ga, x, ldx, M, K, s);
+  return launch_fused_group(ga, x, ldx, M, K, nullptr, false, s);
 }
 
 bool gemv_group_applies(int M, int K, const int* N, int count) {
@@ -794,7 +943,41 @@ hipError_t launch_gemv_group(float* const* y, const float* x, int ldx, const uin
     ga.first[i + 1] = ga.first[i] + (N[i] + kTileRows - 1) / kTileRows;
   }
   ga.count = count;
-  return launch_fused_group(ga, x, ldx, M, K, s);
+  return launch_fused_group(ga, x, ldx, M, K, nullptr, false, s);
+}
+
+// One decode row (M = 1) through 1..4 Linears with the decoder's extras: residual add + RMSNorm in
+// front (norm_w != null), silu(y0) * y1 behind (pair: two Linears of equal N, result in y[0]).
+bool gemv_decode_applies(int K, const int* N, int count, bool pair) {
+  if (count < 1 || count > kMaxGroup || (pair && (count != 2 || N[0] != N[1]))) return false;
+  const FusedPlan p = fused_plan(1, K);
+  if (p.W == 0 || (pair && p.CPW > 3)) return false;
+  bool wide = false;
+  for (int i = 0; i < count; ++i) {
+    if (!gemv_fused_applies(1, K, N[i])) return false;
+    wide = wide || wide_applies(K, N[i]);
+  }
+  return !wide || (count == 1 && !pair);  // a wide layer goes alone
+}
+
+hipError_t launch_gemv_decode(float* const* y, const float* x, const uint8_t* const* packed,
+                              const int* N, int count, int K, const float* delta, float* sum_out,
+                              const float* norm_w, float eps, bool pair, hipStream_t s) {
+  const RowPrologue pro{delta, sum_out, norm_w, eps};
+  if (count == 1 && wide_applies(K, N[0])) {
+    if (norm_w) return launch_wide<1, true, true>(y[0], x, K, nullptr, packed[0], K, N[0], pro, s);
+    return launch_wide<1, true, false>(y[0], x, K, nullptr, packed[0], K, N[0], pro, s);
+  }
+  GroupArgs ga{};
+  ga.first[0] = 0;
+  for (int i = 0; i < count; ++i) {
+    ga.packed[i] = packed[i];
+    ga.y[i] = y[i];
+    ga.N[i] = N[i];
+    ga.first[i + 1] = ga.first[i] + (N[i] + kTileRows - 1) / kTileRows;
+  }
+  ga.count = count;
+  return launch_fused_group(ga, x, K, 1, K, norm_w ? &pro : nullptr, pair, s);
 }
 
 }  // namespace w4

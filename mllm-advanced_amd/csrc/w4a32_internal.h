@@ -31,6 +31,12 @@ hipError_t launch_gemv_fused(float* y, const float* x, int ldx, const uint8_t* p
 bool gemv_group_applies(int M, int K, const int* N, int count);
 hipError_t launch_gemv_group(float* const* y, const float* x, int ldx, const uint8_t* const* packed,
                              const int* N, int count, int M, int K, hipStream_t s);
+// one decode row through 1..4 Linears, optionally with (residual add +) RMSNorm in front and
+// silu(y0) * y1 behind
+bool gemv_decode_applies(int K, const int* N, int count, bool pair);
+hipError_t launch_gemv_decode(float* const* y, const float* x, const uint8_t* const* packed,
+                              const int* N, int count, int K, const float* delta, float* sum_out,
+                              const float* norm_w, float eps, bool pair, hipStream_t s);
 hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                        int kernel, hipStream_t s);
 

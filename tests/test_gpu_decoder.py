@@ -226,3 +226,44 @@ def test_decoder_step_replays_from_a_graph(pkg):
             assert torch.equal(dec.logits, logits_e[i]), i
             _ = (dec.logits * 2).sum().item()     # unrelated eager work between replays
         assert dec.position == 19
+
+
+@pytest.mark.parametrize("K,Ns,pair", [(1536, [1536, 256, 256], False), (1536, [8960, 8960], True),
+                                         (1536, [151936], False), (8960, [1536], False), (256, [640], False)])
+def test_decode_linear_fusions_match_separate_operators(pkg, orc, K, Ns, pair):
+    """Residual add + RMSNorm in front of the Linears and silu*mul behind them, in one launch, against
+    the same operators run one by one and against the CPU oracle fed with the fused row."""
+    import decoder_oracle as do
+
+    rng = np.random.default_rng(K + len(Ns))
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    d = rng.standard_normal((1, K)).astype(np.float32)
+    nw = (1 + 0.1 * rng.standard_normal(K)).astype(np.float32)
+    ws = [(rng.standard_normal((n, K)) * 0.02).astype(np.float32) for n in Ns]
+    packed = [pkg.quant_pack_rhs(dev(w)) for w in ws]
+
+    ys, total = pkg.decode_linear(dev(x), packed, Ns, norm_weight=dev(nw), eps=1e-6, delta=dev(d),
+                                  want_sum=True, silu_pair=pair)
+    torch.cuda.synchronize()
+    assert torch.equal(total, dev(x) + dev(d))
+    # the separate operators
+    h2, xn = pkg.op_rmsnorm(dev(x), dev(nw), 1e-6, delta=dev(d))
+    sep = pkg.matmul_grouped(xn, packed, Ns) if len(Ns) > 1 else [pkg.matmul(xn, packed[0], Ns[0])]
+    if pair:
+        sep = [pkg.op_silu_mul(sep[0], sep[1])]
+    # the oracle on the normalised row
+    xn_ref = do.rmsnorm((x + d).astype(np.float32), nw, 1e-6)
+    want = []
+    for w in ws if len(Ns) < 4 or Ns[0] < 100000 else ws:
+        u4, sc = orc.quant_rhs(w)
+        want.append(orc.linear(xn_ref, u4, sc))
+    if pair:
+        want = [do.silu_mul(want[0], want[1])]
+    for got, s, ref in zip(ys, sep, want):
+        assert max_abs_rel(got.cpu().numpy(), s.cpu().numpy()) < 2e-3
+        assert max_abs_rel(got.cpu().numpy(), ref) < 2e-3
+    # without the extras the call is the plain grouped product
+    plain, _ = pkg.decode_linear(dev(x), packed, Ns)
+    base = pkg.matmul_grouped(dev(x), packed, Ns) if len(Ns) > 1 else [pkg.matmul(dev(x), packed[0], Ns[0])]
+    for a, b in zip(plain, base):
+        assert torch.equal(a, b)
