@@ -62,6 +62,16 @@ int w4a32_op_attention(const float* d_q, const float* d_kcache, const float* d_v
                        int M, int n_heads, int n_kv_heads, int head_dim, int max_seq,
                        const int* d_pos0, int pos0, void* d_scratch, void* stream);
 
+/* Decode step (one token at position pos0) with w4a32_op_rope_kv folded into the attention launch:
+ * d_q, d_k, d_v are the un-rotated outputs of the q/k/v Linears; the kernel rotates q and k, appends k
+ * and v to the caches at pos0 and attends over keys 0..pos0. Same results as the two operators in
+ * sequence (d_q itself is left un-rotated). */
+int w4a32_op_rope_attention_decode(const float* d_q, const float* d_k, const float* d_v,
+                                   const float* d_sin, const float* d_cos, float* d_kcache,
+                                   float* d_vcache, float* d_out, int n_heads, int n_kv_heads,
+                                   int head_dim, int max_seq, const int* d_pos0, int pos0,
+                                   void* d_scratch, void* stream);
+
 /* *d_token = index of the first maximum of d_logits[0..n) (AutoLLM.hpp:70-88); when d_pos_to_advance
  * is not NULL, *d_pos_to_advance += 1 afterwards. */
 int w4a32_op_argmax(const float* d_logits, int n, void* d_scratch, int64_t* d_token,

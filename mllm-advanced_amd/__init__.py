@@ -50,6 +50,8 @@ ABI = {
     "w4a32_op_scratch_bytes": (_sz, [_ci]),
     "w4a32_op_scratch_init": (_ci, [_vp, _ci, _vp]),
     "w4a32_op_attention": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _ci, _vp, _vp]),
+    "w4a32_op_rope_attention_decode": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci,
+                                             _vp, _ci, _vp, _vp]),
     "w4a32_op_argmax": (_ci, [_vp, _ci, _vp, _vp, _vp, _vp]),
     "w4a32_decode_linear": (_ci, [_vp, _vp]),
     "w4a32_decoder_state_bytes": (_sz, [_vp]),
@@ -329,6 +331,20 @@ def op_attention(q, kcache, vcache, n_heads, n_kv_heads, head_dim, pos0, scratch
     _check(lib().w4a32_op_attention(_ptr(q), _ptr(kcache), _ptr(vcache), _ptr(out), M, n_heads,
                                     n_kv_heads, head_dim, kcache.shape[1], _ptr(d_pos0), pos0,
                                     _ptr(scratch), _stream()), "w4a32_op_attention")
+    return out
+
+
+def op_rope_attention_decode(q, k, v, sin, cos, kcache, vcache, n_heads, n_kv_heads, head_dim, pos0,
+                             scratch, d_pos0=None):
+    """RoPE + cache append + attention of one token in one launch (q, k, v un-rotated)."""
+    import torch
+
+    out = torch.empty((1, n_heads * head_dim), dtype=torch.float32, device="cuda")
+    _check(lib().w4a32_op_rope_attention_decode(_ptr(q), _ptr(k), _ptr(v), _ptr(sin), _ptr(cos),
+                                                _ptr(kcache), _ptr(vcache), _ptr(out), n_heads,
+                                                n_kv_heads, head_dim, kcache.shape[1], _ptr(d_pos0), pos0,
+                                                _ptr(scratch), _stream()),
+           "w4a32_op_rope_attention_decode")
     return out
 
 

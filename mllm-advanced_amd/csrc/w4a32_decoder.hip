@@ -142,7 +142,7 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
       W4_TRY(from_hip(w4::launch_attention_decode(
           q, kc, vc, attn, Hq, Hkv, c->max_seq, d_pos, 0, kAttnSplit,
           reinterpret_cast<float*>(scratch + sg.part_off),
-          reinterpret_cast<unsigned int*>(scratch + sg.counters_off), s)));
+          reinterpret_cast<unsigned int*>(scratch + sg.counters_off), nullptr, nullptr, nullptr, nullptr, s)));
     } else {
       W4_TRY(from_hip(w4::launch_attention_prefill(q, kc, vc, attn, M, Hq, Hkv, c->max_seq, d_pos, 0, s)));
     }
@@ -170,8 +170,8 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
   return W4A32_OK;
 }
 
-// One decode row with the operators between the Linears folded into them: 6 launches per layer
-// ([add+norm+q,k,v] [rope+cache] [attention] [o] [add+norm+gate,up+silu*mul] [down]) instead of 9.
+// One decode row with the operators between the Linears folded into them: 5 launches per layer
+// ([add+norm+q,k,v] [rope+cache+attention] [o] [add+norm+gate,up+silu*mul] [down]) instead of 9.
 // The residual stream alternates between two buffers because the launch that completes a row
 // (x + delta) is read by every workgroup while one of them stores the sum.
 bool decode_fusable(const w4a32_decoder_config* c) {
@@ -223,11 +223,10 @@ int run_decode_fused(const w4a32_decoder_config* c, const w4a32_decoder_weights*
                                              l == 0 ? nullptr : hnext, lw.attn_norm, c->rms_eps, false, s)));
       if (l != 0) std::swap(hcur, hnext);
     }
-    W4_TRY(from_hip(w4::launch_rope_kv(q, k, v, sin_t, cos_t, kc, vc, 1, Hq, Hkv, D, c->max_seq, d_pos, 0, s)));
     W4_TRY(from_hip(w4::launch_attention_decode(
         q, kc, vc, attn, Hq, Hkv, c->max_seq, d_pos, 0, kAttnSplit,
         reinterpret_cast<float*>(scratch + sg.part_off),
-        reinterpret_cast<unsigned int*>(scratch + sg.counters_off), s)));
+        reinterpret_cast<unsigned int*>(scratch + sg.counters_off), k, v, sin_t, cos_t, s)));
     W4_TRY(one(attn, lw.o, qd, H, delta));
     {
       const uint8_t* pk[2] = {static_cast<const uint8_t*>(lw.gate), static_cast<const uint8_t*>(lw.up)};
@@ -319,12 +318,30 @@ int w4a32_op_attention(const float* d_q, const float* d_kcache, const float* d_v
     const ScratchGeom sg = scratch_geom(n_heads);
     uint8_t* sc = static_cast<uint8_t*>(d_scratch);
     return from_hip(w4::launch_attention_decode(
-        d_q, d_kcache, d_vcache, d_out, n_heads, n_kv_heads, max_seq, d_pos0, pos0, kAttnSplit,
-        reinterpret_cast<float*>(sc + sg.part_off), reinterpret_cast<unsigned int*>(sc + sg.counters_off),
-        S(stream)));
+        d_q, const_cast<float*>(d_kcache), const_cast<float*>(d_vcache), d_out, n_heads, n_kv_heads,
+        max_seq, d_pos0, pos0, kAttnSplit, reinterpret_cast<float*>(sc + sg.part_off),
+        reinterpret_cast<unsigned int*>(sc + sg.counters_off), nullptr, nullptr, nullptr, nullptr, S(stream)));
   }
   return from_hip(w4::launch_attention_prefill(d_q, d_kcache, d_vcache, d_out, M, n_heads, n_kv_heads,
                                                max_seq, d_pos0, pos0, S(stream)));
+}
+
+int w4a32_op_rope_attention_decode(const float* d_q, const float* d_k, const float* d_v,
+                                   const float* d_sin, const float* d_cos, float* d_kcache,
+                                   float* d_vcache, float* d_out, int n_heads, int n_kv_heads,
+                                   int head_dim, int max_seq, const int* d_pos0, int pos0,
+                                   void* d_scratch, void* stream) {
+  if (!d_q || !d_k || !d_v || !d_sin || !d_cos || !d_kcache || !d_vcache || !d_out || !d_scratch)
+    return W4A32_EINVAL;
+  if (n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0) return W4A32_EINVAL;
+  if (head_dim != 128 || n_heads % n_kv_heads != 0) return W4A32_ESHAPE;
+  if (!d_pos0 && (pos0 < 0 || pos0 >= max_seq)) return W4A32_ESHAPE;
+  const ScratchGeom sg = scratch_geom(n_heads);
+  uint8_t* sc = static_cast<uint8_t*>(d_scratch);
+  return from_hip(w4::launch_attention_decode(
+      d_q, d_kcache, d_vcache, d_out, n_heads, n_kv_heads, max_seq, d_pos0, pos0, kAttnSplit,
+      reinterpret_cast<float*>(sc + sg.part_off), reinterpret_cast<unsigned int*>(sc + sg.counters_off),
+      d_k, d_v, d_sin, d_cos, S(stream)));
 }
 
 int w4a32_op_argmax(const float* d_logits, int n, void* d_scratch, int64_t* d_token,

@@ -343,7 +343,7 @@ __global__ __launch_bounds__(64) void attention_kernel(const float* __restrict__
 // one to arrive) are merged with the usual max / rescale rule.
 // ---------------------------------------------------------------------------------------------
 constexpr int kDecWaves = 4;
-constexpr int kMaxAttnSplit = 32;  // key slices per head group, at most
+constexpr int kMaxAttnSplit = 16;  // key slices per head group, at most
 
 // v += the same register of the other 15 lanes of the row (all lanes get the row's sum). Callers
 // interleave several independent values per step so that no DPP read follows its write directly.
@@ -373,32 +373,79 @@ __device__ __forceinline__ void softmax_merge_weights(float m, float m2, float& 
   w2 = m2 == -INFINITY ? 0.0f : __expf(m2 - mn);
 }
 
-template <int kGW>
+// kRope: q, k_new, v_new are the raw outputs of the q/k/v Linears for the token at position pos0.
+// The kernel rotates q itself, and the wavefront whose share contains key pos0 rotates k_new, uses
+// it and v_new in place of the (not yet written) cache row and - in the first head group of each KV
+// head - appends both to the cache. That is the RoPE + cache-append operator folded in.
+// A lane holds dims 8*dl..8*dl+7; its RoPE partner dims (d +- 64) are read with a second load.
+template <int kGW, bool kRope>
 __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
-    const float* __restrict__ q, const float* __restrict__ kc, const float* __restrict__ vc,
+    const float* __restrict__ q, float* __restrict__ kc, float* __restrict__ vc,
     float* __restrict__ out, int Hq, int Hkv, int max_seq, const int* __restrict__ d_pos0, int pos0,
-    float scale, float* part, unsigned int* counters) {
+    float scale, float* part, unsigned int* counters, const float* __restrict__ k_new,
+    const float* __restrict__ v_new, const float* __restrict__ sin_t, const float* __restrict__ cos_t) {
   __shared__ float s_part[kDecWaves][kGW][kPartStride];
   __shared__ unsigned int s_prev;
   const int h0 = blockIdx.x * kGW;             // first query head of this group
-  const int hk = h0 / (Hq / Hkv);
+  const int G = Hq / Hkv;
+  const int hk = h0 / G;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int kq = lane >> 4, dl = lane & 15;
   if (d_pos0) pos0 = *d_pos0;
-  const int len = min(pos0 + 1, max_seq);
+  if (pos0 >= max_seq) pos0 = max_seq - 1;     // the caller keeps the position inside the cache
+  const int len = pos0 + 1;
   // keys of this workgroup, then of this wavefront (multiples of 4 so that slots stay aligned)
   const int per_wg = ((len + (int)gridDim.y - 1) / (int)gridDim.y + 15) / 16 * 16;
   const int per_wave = per_wg / kDecWaves;
   const int begin = min((int)blockIdx.y * per_wg + wave * per_wave, len);
   const int end = min(begin + per_wave, len);
 
+  auto load8 = [](const float* src, float (&dst)[8]) {
+    const float4 a = *reinterpret_cast<const float4*>(src);
+    const float4 b = *reinterpret_cast<const float4*>(src + 4);
+    dst[0] = a.x; dst[1] = a.y; dst[2] = a.z; dst[3] = a.w;
+    dst[4] = b.x; dst[5] = b.y; dst[6] = b.z; dst[7] = b.w;
+  };
+  // y0 = x0 c - x1 s (first half of the head), y1 = x0 s + x1 c (second half)
+  const int pdl = dl ^ 8;                      // the lane position that holds the partner dims
+  float sn[8], cs[8];
+  if (kRope) {
+    load8(sin_t + (size_t)pos0 * (kHeadDim / 2) + 8 * (dl & 7), sn);
+    load8(cos_t + (size_t)pos0 * (kHeadDim / 2) + 8 * (dl & 7), cs);
+  }
+  auto rotate = [&](const float* vec, float (&dst)[8]) {
+    float own[8], oth[8];
+    load8(vec + 8 * dl, own);
+    load8(vec + 8 * pdl, oth);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      dst[i] = dl < 8 ? own[i] * cs[i] - oth[i] * sn[i] : oth[i] * sn[i] + own[i] * cs[i];
+    }
+  };
+
   float qr[kGW][8];
 #pragma unroll
   for (int g = 0; g < kGW; ++g) {
-    const float4* src = reinterpret_cast<const float4*>(q + (size_t)(h0 + g) * kHeadDim + 8 * dl);
-    const float4 a = src[0], b = src[1];
-    qr[g][0] = a.x; qr[g][1] = a.y; qr[g][2] = a.z; qr[g][3] = a.w;
-    qr[g][4] = b.x; qr[g][5] = b.y; qr[g][6] = b.z; qr[g][7] = b.w;
+    const float* src = q + (size_t)(h0 + g) * kHeadDim;
+    if (kRope) {
+      rotate(src, qr[g]);
+    } else {
+      load8(src + 8 * dl, qr[g]);
+    }
+  }
+  float knew[8], vnew[8];
+  const bool has_new = kRope && begin <= pos0 && pos0 < end;   // wavefront-uniform
+  if (has_new) {
+    rotate(k_new + (size_t)hk * kHeadDim, knew);
+    load8(v_new + (size_t)hk * kHeadDim + 8 * dl, vnew);
+    if (h0 % G == 0 && blockIdx.x * kGW == (unsigned)h0 && kq == 0) {
+      float* kd = kc + ((size_t)hk * max_seq + pos0) * kHeadDim + 8 * dl;
+      float* vd = vc + ((size_t)hk * max_seq + pos0) * kHeadDim + 8 * dl;
+      *reinterpret_cast<float4*>(kd) = make_float4(knew[0], knew[1], knew[2], knew[3]);
+      *reinterpret_cast<float4*>(kd + 4) = make_float4(knew[4], knew[5], knew[6], knew[7]);
+      *reinterpret_cast<float4*>(vd) = make_float4(vnew[0], vnew[1], vnew[2], vnew[3]);
+      *reinterpret_cast<float4*>(vd + 4) = make_float4(vnew[4], vnew[5], vnew[6], vnew[7]);
+    }
   }
   const float* kbase = kc + (size_t)hk * max_seq * kHeadDim + 8 * dl;
   const float* vbase = vc + (size_t)hk * max_seq * kHeadDim + 8 * dl;
@@ -431,6 +478,17 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
       const float4 b = *reinterpret_cast<const float4*>(vbase + row + 4);
       vv[it][0] = a.x; vv[it][1] = a.y; vv[it][2] = a.z; vv[it][3] = a.w;
       vv[it][4] = b.x; vv[it][5] = b.y; vv[it][6] = b.z; vv[it][7] = b.w;
+    }
+    if (has_new) {
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const bool is_new = blk + 4 * it + kq == pos0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          kk[it][i] = is_new ? knew[i] : kk[it][i];
+          vv[it][i] = is_new ? vnew[i] : vv[it][i];
+        }
+      }
     }
     float sc[4][kGW];
 #pragma unroll
@@ -523,29 +581,28 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
   }
   __syncthreads();
   if (s_prev != gridDim.y - 1) return;
-  // Last workgroup of this head group: merge the shares of all key slices. Their (max, sum)
-  // headers go through LDS first so that every thread can weigh its own dim's loads, which are
-  // then independent of each other.
-  __shared__ float s_hdr[kGW][kMaxAttnSplit][2];
-  for (int i = threadIdx.x; i < kGW * ns; i += blockDim.x) {
-    const int g = i / ns, sidx = i % ns;
-    const float* ps = part + ((size_t)(h0 + g) * ns + sidx) * kPartStride;
-    s_hdr[g][sidx][0] = load_shared_across_wgs(ps);
-    s_hdr[g][sidx][1] = load_shared_across_wgs(ps + 1);
-  }
-  __syncthreads();
+  // Last workgroup of this head group: merge the shares of all key slices. Every thread requests
+  // all headers and its own dim of all shares at once (ns <= kMaxAttnSplit, loads independent).
   for (int t = threadIdx.x; t < kGW * kHeadDim; t += blockDim.x) {
     const int g = t / kHeadDim, d = t % kHeadDim;
-    const float* all = part + (size_t)(h0 + g) * ns * kPartStride + 2 + d;
+    const float* all = part + (size_t)(h0 + g) * ns * kPartStride;
+    float ms[kMaxAttnSplit], ls[kMaxAttnSplit], as[kMaxAttnSplit];
+#pragma unroll
+    for (int sidx = 0; sidx < kMaxAttnSplit; ++sidx) {
+      const float* ps = all + (size_t)(sidx < ns ? sidx : ns - 1) * kPartStride;
+      ms[sidx] = load_shared_across_wgs(ps);
+      ls[sidx] = load_shared_across_wgs(ps + 1);
+      as[sidx] = load_shared_across_wgs(ps + 2 + d);
+    }
     float mm = -INFINITY;
-    for (int sidx = 0; sidx < ns; ++sidx) mm = fmaxf(mm, s_hdr[g][sidx][0]);
+#pragma unroll
+    for (int sidx = 0; sidx < kMaxAttnSplit; ++sidx) mm = fmaxf(mm, sidx < ns ? ms[sidx] : -INFINITY);
     float ll = 0.0f, a = 0.0f;
-#pragma unroll 8
-    for (int sidx = 0; sidx < ns; ++sidx) {
-      const float ms = s_hdr[g][sidx][0];
-      const float wt = ms == -INFINITY ? 0.0f : __expf(ms - mm);
-      ll += s_hdr[g][sidx][1] * wt;
-      a += load_shared_across_wgs(all + (size_t)sidx * kPartStride) * wt;
+#pragma unroll
+    for (int sidx = 0; sidx < kMaxAttnSplit; ++sidx) {
+      const float wt = (sidx < ns && ms[sidx] != -INFINITY) ? __expf(ms[sidx] - mm) : 0.0f;
+      ll += ls[sidx] * wt;
+      a += as[sidx] * wt;
     }
     out[(size_t)(h0 + g) * kHeadDim + d] = a / ll;  // key 0 is always there: ll > 0
   }
@@ -681,21 +738,27 @@ hipError_t launch_attention_prefill(const float* q, const float* kc, const float
   return hipGetLastError();
 }
 
-hipError_t launch_attention_decode(const float* q, const float* kc, const float* vc, float* out,
-                                   int Hq, int Hkv, int max_seq, const int* d_pos0, int pos0,
-                                   int nsplit, float* part, unsigned int* counters, hipStream_t s) {
+// k_new != null: q, k_new, v_new are un-rotated Linear outputs of the token at pos0 and the kernel
+// performs RoPE and the cache append itself (then sin_t / cos_t are the RoPE tables).
+hipError_t launch_attention_decode(const float* q, float* kc, float* vc, float* out, int Hq, int Hkv,
+                                   int max_seq, const int* d_pos0, int pos0, int nsplit, float* part,
+                                   unsigned int* counters, const float* k_new, const float* v_new,
+                                   const float* sin_t, const float* cos_t, hipStream_t s) {
   const float scale = 1.0f / sqrtf((float)kHeadDim);
   const int G = Hq / Hkv;  // query heads per KV head; a workgroup takes 2 or 3 of them when it divides
+  if (nsplit > kMaxAttnSplit) return hipErrorInvalidValue;
+#define W4_ATTN(gw, rope)                                                                              \
+  hipLaunchKernelGGL((attention_decode_kernel<gw, rope>), dim3(Hq / gw, nsplit), dim3(64 * kDecWaves), \
+                     0, s, q, kc, vc, out, Hq, Hkv, max_seq, d_pos0, pos0, scale, part, counters,      \
+                     k_new, v_new, sin_t, cos_t)
   if (G % 2 == 0) {
-    hipLaunchKernelGGL(attention_decode_kernel<2>, dim3(Hq / 2, nsplit), dim3(64 * kDecWaves), 0, s, q, kc,
-                       vc, out, Hq, Hkv, max_seq, d_pos0, pos0, scale, part, counters);
+    if (k_new) W4_ATTN(2, true); else W4_ATTN(2, false);
   } else if (G % 3 == 0) {
-    hipLaunchKernelGGL(attention_decode_kernel<3>, dim3(Hq / 3, nsplit), dim3(64 * kDecWaves), 0, s, q, kc,
-                       vc, out, Hq, Hkv, max_seq, d_pos0, pos0, scale, part, counters);
+    if (k_new) W4_ATTN(3, true); else W4_ATTN(3, false);
   } else {
-    hipLaunchKernelGGL(attention_decode_kernel<1>, dim3(Hq, nsplit), dim3(64 * kDecWaves), 0, s, q, kc, vc,
-                       out, Hq, Hkv, max_seq, d_pos0, pos0, scale, part, counters);
+    if (k_new) W4_ATTN(1, true); else W4_ATTN(1, false);
   }
+#undef W4_ATTN
   return hipGetLastError();
 }
 

@@ -54,9 +54,10 @@ hipError_t launch_rope_kv(float* q, const float* k, const float* v, const float*
 hipError_t launch_attention_prefill(const float* q, const float* kc, const float* vc, float* out,
                                     int M, int Hq, int Hkv, int max_seq, const int* d_pos0, int pos0,
                                     hipStream_t s);
-hipError_t launch_attention_decode(const float* q, const float* kc, const float* vc, float* out,
-                                   int Hq, int Hkv, int max_seq, const int* d_pos0, int pos0,
-                                   int nsplit, float* part, unsigned int* counters, hipStream_t s);
+hipError_t launch_attention_decode(const float* q, float* kc, float* vc, float* out, int Hq, int Hkv,
+                                   int max_seq, const int* d_pos0, int pos0, int nsplit, float* part,
+                                   unsigned int* counters, const float* k_new, const float* v_new,
+                                   const float* sin_t, const float* cos_t, hipStream_t s);
 hipError_t launch_argmax(const float* logits, int n, float* part_val, int* part_idx,
                          unsigned int* counter, int64_t* token_out, int* pos_to_advance, int blocks,
                          hipStream_t s);

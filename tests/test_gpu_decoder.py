@@ -112,6 +112,27 @@ def test_attention_prefill_and_decode(pkg, Hq, Hkv):
     assert int(scratch[:4 * (Hq + 1)].view(torch.int32).abs().sum()) == 0
 
 
+@pytest.mark.parametrize("Hq,Hkv", [(12, 2), (4, 4), (3, 1)])
+def test_rope_attention_decode_equals_the_two_operators(pkg, Hq, Hkv):
+    g = torch.Generator(device="cuda").manual_seed(6)
+    D, S = 128, 256
+    sin, cos = pkg.op_rope_table(S, D, 1e6)
+    scratch = pkg.op_scratch(Hq)
+    for pos in [0, 3, 15, 16, 17, 100, 255]:
+        kc = torch.randn((Hkv, S, D), generator=g, device="cuda")
+        vc = torch.randn((Hkv, S, D), generator=g, device="cuda")
+        q = torch.randn((1, Hq * D), generator=g, device="cuda")
+        k = torch.randn((1, Hkv * D), generator=g, device="cuda")
+        v = torch.randn((1, Hkv * D), generator=g, device="cuda")
+        kc1, vc1, q1 = kc.clone(), vc.clone(), q.clone()
+        pkg.op_rope_kv(q1, k, v, sin, cos, kc1, vc1, Hq, Hkv, D, pos)
+        want = pkg.op_attention(q1, kc1, vc1, Hq, Hkv, D, pos, scratch=scratch)
+        kc2, vc2 = kc.clone(), vc.clone()
+        got = pkg.op_rope_attention_decode(q, k, v, sin, cos, kc2, vc2, Hq, Hkv, D, pos, scratch)
+        assert torch.equal(got, want), pos
+        assert torch.equal(kc2, kc1) and torch.equal(vc2, vc1), pos
+
+
 def test_argmax_first_maximum(pkg):
     g = torch.Generator(device="cuda").manual_seed(3)
     scratch = pkg.op_scratch(12)
