@@ -48,6 +48,15 @@ int w4a32_op_rope_kv(float* d_q, const float* d_k, const float* d_v, const float
                      int n_kv_heads, int head_dim, int max_seq, const int* d_pos0, int pos0,
                      void* stream);
 
+/* im2col of a Conv3D without padding or dilation: d_in [B][C][T][H][W] -> d_out [B*OT*OH*OW][ld_out] with
+ * column (c, kt, kh, kw) at c*kt*kh*kw + ..., O* = (size - kernel) / stride + 1; columns from C*kt*kh*kw up
+ * to ld_out are written as zeros (pad K to a multiple of 32 and zero-pad the weight rows alike: the
+ * convolution is then w4a32_matmul on d_out, as ArmConv3DOp::forward does it,
+ * mllm/Backends/Arm/Ops/Conv3DOp.cpp:48-188 with mllm/Backends/Arm/Kernels/conv3d.cpp:15-78). The result
+ * rows are [b][ot][oh][ow] x out_channels, i.e. channels-last. */
+int w4a32_op_im2col_conv3d(const float* d_in, float* d_out, int B, int C, int T, int H, int W, int kt,
+                           int kh, int kw, int st, int sh, int sw, int ld_out, void* stream);
+
 /* Scratch of the decode attention and of argmax: arrival counters + partial results. Must be cleared
  * once with w4a32_op_scratch_init before its first use; the kernels leave it cleared. */
 size_t w4a32_op_scratch_bytes(int n_heads);

@@ -47,6 +47,7 @@ ABI = {
     "w4a32_op_silu_mul": (_ci, [_vp, _vp, _vp, _sz, _vp]),
     "w4a32_op_rope_table": (_ci, [_vp, _vp, _ci, _ci, ctypes.c_float, _vp]),
     "w4a32_op_rope_kv": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _ci, _vp]),
+    "w4a32_op_im2col_conv3d": (_ci, [_vp, _vp] + [_ci] * 12 + [_vp]),
     "w4a32_op_scratch_bytes": (_sz, [_ci]),
     "w4a32_op_scratch_init": (_ci, [_vp, _ci, _vp]),
     "w4a32_op_attention": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _ci, _vp, _vp]),
@@ -315,6 +316,21 @@ def op_rope_kv(q, k, v, sin, cos, kcache, vcache, n_heads, n_kv_heads, head_dim,
     _check(lib().w4a32_op_rope_kv(_ptr(q), _ptr(k), _ptr(v), _ptr(sin), _ptr(cos), _ptr(kcache),
                                   _ptr(vcache), M, n_heads, n_kv_heads, head_dim, kcache.shape[1],
                                   _ptr(d_pos0), pos0, _stream()), "w4a32_op_rope_kv")
+
+
+def op_im2col_conv3d(x, kernel, stride, ld_out=None):
+    """x [B][C][T][H][W] f32 -> [B*OT*OH*OW][ld_out] (columns beyond C*kt*kh*kw are zero)."""
+    import torch
+
+    B, C, T, H, W = x.shape
+    (kt, kh, kw), (st, sh, sw) = kernel, stride
+    rows = B * ((T - kt) // st + 1) * ((H - kh) // sh + 1) * ((W - kw) // sw + 1)
+    cols = C * kt * kh * kw
+    ld = ld_out or (cols + 31) // 32 * 32
+    out = torch.empty((rows, ld), dtype=torch.float32, device="cuda")
+    _check(lib().w4a32_op_im2col_conv3d(_ptr(x), _ptr(out), B, C, T, H, W, kt, kh, kw, st, sh, sw, ld,
+                                        _stream()), "w4a32_op_im2col_conv3d")
+    return out
 
 
 def op_scratch(n_heads):

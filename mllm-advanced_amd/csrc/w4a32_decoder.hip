@@ -300,6 +300,16 @@ int w4a32_op_rope_kv(float* d_q, const float* d_k, const float* d_v, const float
                                      n_kv_heads, head_dim, max_seq, d_pos0, pos0, S(stream)));
 }
 
+int w4a32_op_im2col_conv3d(const float* d_in, float* d_out, int B, int C, int T, int H, int W, int kt,
+                           int kh, int kw, int st, int sh, int sw, int ld_out, void* stream) {
+  if (!d_in || !d_out || B <= 0 || C <= 0 || kt <= 0 || kh <= 0 || kw <= 0 || st <= 0 || sh <= 0 || sw <= 0)
+    return W4A32_EINVAL;
+  if (T < kt || H < kh || W < kw) return W4A32_ESHAPE;
+  if (ld_out < C * kt * kh * kw) return W4A32_ESHAPE;
+  return from_hip(w4::launch_im2col_conv3d(d_in, d_out, B, C, T, H, W, kt, kh, kw, st, sh, sw, ld_out,
+                                           S(stream)));
+}
+
 size_t w4a32_op_scratch_bytes(int n_heads) { return n_heads > 0 ? scratch_geom(n_heads).total : 0; }
 
 int w4a32_op_scratch_init(void* d_scratch, int n_heads, void* stream) {

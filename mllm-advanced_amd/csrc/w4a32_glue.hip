@@ -682,6 +682,33 @@ __global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ l
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// im2col for a Conv3D without padding and dilation (the vision patch embedding), so that the
+// convolution becomes the same quantized Linear: row = (b, ot, oh, ow), column = (c, kt, kh, kw),
+// as im2col_conv3d_p0_d1_activation_fp32 (mllm/Backends/Arm/Kernels/conv3d.cpp:15-78) lays it out.
+// Columns from the true width up to ld are written as 0 (K is padded to a multiple of 32 for the
+// block-32 weights; a zero column changes neither the row's quantisation range nor any sum).
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void im2col_conv3d_kernel(const float* __restrict__ a,
+                                                            float* __restrict__ z, int C, int T, int H,
+                                                            int W, int kt, int kh, int kw, int st, int sh,
+                                                            int sw, int OT, int OH, int OW, int ld) {
+  const int row = blockIdx.x;  // (b, ot, oh, ow)
+  const int ow = row % OW, oh = (row / OW) % OH, ot = (row / (OW * OH)) % OT, b = row / (OW * OH * OT);
+  const int kvol = kt * kh * kw, cols = C * kvol;
+  const float* ab = a + (size_t)b * C * T * H * W;
+  float* zr = z + (size_t)row * ld;
+  for (int col = threadIdx.x; col < ld; col += blockDim.x) {
+    float v = 0.0f;
+    if (col < cols) {
+      const int c = col / kvol, r = col % kvol;
+      const int dt = r / (kh * kw), dh = (r / kw) % kh, dw = r % kw;
+      v = ab[(((size_t)c * T + (ot * st + dt)) * H + (oh * sh + dh)) * W + (ow * sw + dw)];
+    }
+    zr[col] = v;
+  }
+}
+
 __global__ void add_to_int_kernel(int* p, int delta) { *p += delta; }
 __global__ void set_int_kernel(int* p, int value) { *p = value; }
 __global__ void zero_u32_kernel(unsigned int* p, int n) {
@@ -767,6 +794,14 @@ hipError_t launch_argmax(const float* logits, int n, float* part_val, int* part_
                          hipStream_t s) {
   hipLaunchKernelGGL(argmax_kernel, dim3(blocks), dim3(256), 0, s, logits, n, part_val, part_idx,
                      counter, token_out, pos_to_advance);
+  return hipGetLastError();
+}
+
+hipError_t launch_im2col_conv3d(const float* a, float* z, int B, int C, int T, int H, int W, int kt,
+                                int kh, int kw, int st, int sh, int sw, int ld, hipStream_t s) {
+  const int OT = (T - kt) / st + 1, OH = (H - kh) / sh + 1, OW = (W - kw) / sw + 1;
+  hipLaunchKernelGGL(im2col_conv3d_kernel, dim3(B * OT * OH * OW), dim3(256), 0, s, a, z, C, T, H, W, kt,
+                     kh, kw, st, sh, sw, OT, OH, OW, ld);
   return hipGetLastError();
 }
 

@@ -61,6 +61,8 @@ hipError_t launch_attention_decode(const float* q, float* kc, float* vc, float* 
 hipError_t launch_argmax(const float* logits, int n, float* part_val, int* part_idx,
                          unsigned int* counter, int64_t* token_out, int* pos_to_advance, int blocks,
                          hipStream_t s);
+hipError_t launch_im2col_conv3d(const float* a, float* z, int B, int C, int T, int H, int W, int kt,
+                                int kh, int kw, int st, int sh, int sw, int ld, hipStream_t s);
 hipError_t launch_set_int(int* p, int value, hipStream_t s);
 hipError_t launch_add_to_int(int* p, int delta, hipStream_t s);
 hipError_t launch_zero_u32(unsigned int* p, int n, hipStream_t s);
