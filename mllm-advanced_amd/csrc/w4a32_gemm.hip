@@ -389,23 +389,22 @@ static hipError_t launch_gemm_i8(float* y, const uint8_t* ws, const uint8_t* pac
   return hipGetLastError();
 }
 
-// All f16 configurations use a 128 x 128 output tile (1 KiB weight fragments shared through
-// LDS by the whole workgroup). With many tiles, 4 wavefronts per workgroup and three workgroups
-// per CU did best on MI355X; with few tiles, 8 wavefronts per workgroup (smaller wavefront
-// tiles, more wavefronts per SIMD to hide each other's stalls) did.
-static bool many_tiles(int M, int NT) {
-  const long tiles = (long)((M + 127) / 128) * ((NT + 7) / 8);
-  return tiles >= 1024;
-}
-
+// Tile shape by how many 128 x 128 tiles the problem has (measured on MI355X at M = 128..2048 over
+// the decoder and ViT shapes). A stage of 64 k costs a workgroup about the same time whatever
+// its tile size as long as it is alone on its CU, so few-tile problems take smaller tiles: more
+// workgroups, several per CU, which overlap each other's stalls. With many tiles the larger tile's
+// operand reuse wins; from 1024 tiles on, 4 wavefronts per workgroup and three workgroups per CU
+// did best, below that 8 wavefronts per workgroup.
 hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                        int kernel, hipStream_t s) {
   if (kernel == kKernelGemmI8 || (kernel == kKernelAuto && M <= 32)) {
     return launch_gemm_i8(y, ws, packed, M, K, N, s);
   }
-  const WeightGeom g = weight_geom(N, K);
-  if (many_tiles(M, g.NT)) return launch_f16<4, 1, 1, 4>(y, ws, packed, M, K, N, s);
-  return launch_f16<4, 2, 1, 2>(y, ws, packed, M, K, N, s);
+  const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+  if (tiles < 128) return launch_f16<2, 2, 1, 1>(y, ws, packed, M, K, N, s);   //  64 x  64
+  if (tiles < 512) return launch_f16<4, 1, 1, 2>(y, ws, packed, M, K, N, s);   // 128 x  64
+  if (tiles < 1024) return launch_f16<4, 2, 1, 2>(y, ws, packed, M, K, N, s);  // 128 x 128, 8 wavefronts
+  return launch_f16<4, 1, 1, 4>(y, ws, packed, M, K, N, s);                    // 128 x 128, 4 wavefronts
 }
 
 }  // namespace w4
