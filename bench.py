@@ -368,7 +368,7 @@ def main():
             "decode_ms_per_token": round(decode_ms / n_new, 4),
             "decode_tokens_per_s": round(n_new / (decode_ms * 1e-3), 1),
             "decode_weight_GBps": round(step_bytes / (decode_ms / n_new * 1e-3) / 1e9, 1),
-            "note": "one decode step = 171 launches (embedding, 28 x [add+norm+qkv, rope+cache, attention, o, "
+            "note": "one decode step = 143 launches (embedding, 28 x [add+norm+qkv, rope+cache+attention, o, "
                     "add+norm+gate/up+silu*mul, down], add+norm+lm_head, argmax), captured once and replayed; "
                     "positions and cache lengths are read from device memory",
         }

@@ -234,14 +234,16 @@ struct GroupArgs {
 // kPair: exactly two Linears of the same N (gate, up): a workgroup multiplies tile row nt of both
 //   and stores silu(y0) * y1 to y[0].
 template <int M, int kFusedR, bool kGrouped, int kCPW, bool kNorm, bool kPair>
-__global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(const GroupArgs ga,
-                                                          const float* __restrict__ x, int ldx,
-                                                          int K, int KC, const RowPrologue pro) {
+__global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
+    const float* __restrict__ x, int ldx, int K, int KC, const uint8_t* packed0, float* y0, int N0,
+    int W, const GroupArgs ga, const RowPrologue pro) {
+  // The leading scalar arguments (everything a single Linear needs) are preloaded into SGPRs by
+  // the dispatcher, so the first loads go out without waiting for the argument segment.
   extern __shared__ __align__(16) uint8_t smem[];
   constexpr int kSets = kPair ? 2 : 1;  // weight matrices a workgroup multiplies
-  const uint8_t* packed = ga.packed[0];
-  float* y = ga.y[0];
-  int N = ga.N[0], nt_first = 0;
+  const uint8_t* packed = packed0;
+  float* y = y0;
+  int N = N0, nt_first = 0;
   if (kGrouped) {
     // Which Linear this workgroup belongs to. All four table entries are fetched first (the
     // empty asm pins them in scalar registers) and then selected, so that the choice costs a
@@ -270,7 +272,7 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(const G
   const int NT = (N + kTileRows - 1) / kTileRows;
   const float* rsum = reinterpret_cast<const float*>(packed + (size_t)NT * KC * kTileBytes);
   const int Kp = KC * kTileK;
-  const int W = blockDim.x >> 6;
+  const int nthreads = 64 * W;  // the workgroup size, without a read of the hidden launch arguments
   int8_t* s_a = reinterpret_cast<int8_t*>(smem);                          // [M][Kp]
   float* s_red = reinterpret_cast<float*>(smem + (size_t)M * Kp);         // [W][kSets][M][16]
   float2* s_mm = reinterpret_cast<float2*>(s_red + W * kSets * M * 16);   // [W][M] (min, max)
@@ -289,7 +291,7 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(const G
     const float* row = x + (size_t)m * ldx;
 #pragma unroll
     for (int r = 0; r < kFusedR; ++r) {
-      const int c = threadIdx.x + r * blockDim.x;
+      const int c = threadIdx.x + r * nthreads;
       const int cc = c < groups ? c : groups - 1;  // a duplicate of a real element: harmless for min/max
       const float4 v0 = *reinterpret_cast<const float4*>(row + 8 * cc);
       const float4 v1 = *reinterpret_cast<const float4*>(row + 8 * cc + 4);
@@ -305,7 +307,7 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(const G
       const float* row = pro.delta + (size_t)m * ldx;
 #pragma unroll
       for (int r = 0; r < kFusedR; ++r) {
-        const int c = threadIdx.x + r * blockDim.x;
+        const int c = threadIdx.x + r * nthreads;
         const int cc = c < groups ? c : groups - 1;
         const float4 v0 = *reinterpret_cast<const float4*>(row + 8 * cc);
         const float4 v1 = *reinterpret_cast<const float4*>(row + 8 * cc + 4);
@@ -350,7 +352,7 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(const G
       float ss = 0.0f;
 #pragma unroll
       for (int r = 0; r < kFusedR; ++r) {
-        const int c = threadIdx.x + r * blockDim.x;
+        const int c = threadIdx.x + r * nthreads;
         if (pro.delta) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) xv[m][r][e] += dv[m][r][e];
@@ -371,7 +373,7 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(const G
     // the norm weight travels while the partial sums meet
 #pragma unroll
     for (int r = 0; r < kFusedR; ++r) {
-      const int c = threadIdx.x + r * blockDim.x;
+      const int c = threadIdx.x + r * nthreads;
       const int cc = c < groups ? c : groups - 1;
       const float4 v0 = *reinterpret_cast<const float4*>(pro.norm_w + 8 * cc);
       const float4 v1 = *reinterpret_cast<const float4*>(pro.norm_w + 8 * cc + 4);
@@ -424,7 +426,7 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(const G
   for (int m = 0; m < M; ++m) {
 #pragma unroll
     for (int r = 0; r < kFusedR; ++r) {
-      const int c = threadIdx.x + r * blockDim.x;
+      const int c = threadIdx.x + r * nthreads;
       if (c < grp_per_row) {
         uint2 out = quant_group8(xv[m][r], par[m]);
         if (c >= groups) out = make_uint2(0, 0);
@@ -480,8 +482,8 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(const G
   __syncthreads();
 
   //   y = (sum/16 + off * rsum[n]) * lhs_scale + bias[n], clamped to the finite f32 range
-  const bool prefetched = blockDim.x >= kOutputs;
-  for (int o = threadIdx.x; o < kOutputs; o += blockDim.x) {
+  const bool prefetched = nthreads >= kOutputs;
+  for (int o = threadIdx.x; o < kOutputs; o += nthreads) {
     const int m = o >> 4;
     const int n = kTileRows * nt + (o & 15);
     if (n < N) {
@@ -589,11 +591,11 @@ static hipError_t launch_fused_m(const GroupArgs& ga, const float* x, int ldx, i
   if (ga.count == 1 || kPair) {
     auto kern = gemv_fused_kernel<M, R, false, CPW, kNorm, kPair>;
     if (hipError_t e = raise_lds_limit(kern, lds, &raised1); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, grid, block, lds, s, ga, x, ldx, K, KC, pro);
+    hipLaunchKernelGGL(kern, grid, block, lds, s, x, ldx, K, KC, ga.packed[0], ga.y[0], ga.N[0], W, ga, pro);
   } else {
     auto kern = gemv_fused_kernel<M, R, true, CPW, kNorm, false>;
     if (hipError_t e = raise_lds_limit(kern, lds, &raisedg); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, grid, block, lds, s, ga, x, ldx, K, KC, pro);
+    hipLaunchKernelGGL(kern, grid, block, lds, s, x, ldx, K, KC, ga.packed[0], ga.y[0], ga.N[0], W, ga, pro);
   }
   return hipGetLastError();
 }

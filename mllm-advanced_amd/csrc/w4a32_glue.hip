@@ -209,44 +209,28 @@ __global__ __launch_bounds__(64) void rope_kv_kernel(float* __restrict__ q,
 }
 
 // ---------------------------------------------------------------------------------------------
-// Attention of one query vector per wavefront over the cached keys 0..pos (head_dim 128).
+// Prefill attention: one query vector per wavefront over the cached keys 0..pos (head_dim 128).
 //
 // A wavefront takes 64 keys at a time: lane = key for the scores (each lane walks its key's row,
 // q comes from LDS as a broadcast read), online softmax across chunks, then lane = 2 output
 // dims for P*V (one coalesced 512-byte row per key, the weight broadcast with v_readlane).
-//
-// kSplit = false (prefill): grid (Hq, M); query m sits at position pos0 + m; output written normalised.
-// kSplit = true  (decode, M = 1): grid (Hq, nsplit); every wavefront takes a contiguous share of
-//   the keys and leaves (max, sum, unnormalised acc[128]) in `part`; the last one to finish for a
-//   head (arrival counter, reset for the next launch) merges the shares and writes the output.
+// grid (Hq, M); query m sits at position pos0 + m.
 // ---------------------------------------------------------------------------------------------
 constexpr int kHeadDim = 128;
 constexpr int kPartStride = kHeadDim + 2;
 
-template <bool kSplit>
-__global__ __launch_bounds__(64) void attention_kernel(const float* __restrict__ q,
-                                                       const float* __restrict__ kc,
-                                                       const float* __restrict__ vc,
-                                                       float* __restrict__ out, int Hq, int Hkv,
-                                                       int max_seq, const int* __restrict__ d_pos0,
-                                                       int pos0, float scale, float* part,
-                                                       unsigned int* counters) {
+__global__ __launch_bounds__(64) void attention_prefill_kernel(const float* __restrict__ q,
+                                                               const float* __restrict__ kc,
+                                                               const float* __restrict__ vc,
+                                                               float* __restrict__ out, int Hq, int Hkv,
+                                                               int max_seq, const int* __restrict__ d_pos0,
+                                                               int pos0, float scale) {
   __shared__ __align__(16) float s_q[kHeadDim];
   const int h = blockIdx.x, lane = threadIdx.x;
   const int hk = h / (Hq / Hkv);
   if (d_pos0) pos0 = *d_pos0;
-  int m, begin, end;
-  if (kSplit) {
-    m = 0;
-    const int len = min(pos0 + 1, max_seq);
-    const int per = (len + (int)gridDim.y - 1) / (int)gridDim.y;
-    begin = min((int)blockIdx.y * per, len);
-    end = min(begin + per, len);
-  } else {
-    m = blockIdx.y;
-    begin = 0;
-    end = min(pos0 + m + 1, max_seq);
-  }
+  const int m = blockIdx.y;
+  const int end = min(pos0 + m + 1, max_seq);
   const float* qv = q + ((size_t)m * Hq + h) * kHeadDim;
   s_q[lane] = qv[lane];
   s_q[lane + 64] = qv[lane + 64];
@@ -257,7 +241,7 @@ __global__ __launch_bounds__(64) void attention_kernel(const float* __restrict__
   float run_max = -INFINITY, run_sum = 0.0f;
   float acc0 = 0.0f, acc1 = 0.0f;  // output dims 2*lane, 2*lane + 1
 
-  for (int base = begin; base < end; base += 64) {
+  for (int base = 0; base < end; base += 64) {
     const int key = base + lane;
     const bool valid = key < end;
     const float4* krow = reinterpret_cast<const float4*>(kbase + (size_t)(valid ? key : end - 1) * kHeadDim);
@@ -280,54 +264,27 @@ __global__ __launch_bounds__(64) void attention_kernel(const float* __restrict__
     acc1 *= corr;
     run_max = new_max;
     const int cnt = min(64, end - base);
-    for (int i = 0; i < cnt; ++i) {
-      const float pi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), i));
-      const float2 vv = *reinterpret_cast<const float2*>(vbase + (size_t)(base + i) * kHeadDim + 2 * lane);
-      acc0 += pi * vv.x;
-      acc1 += pi * vv.y;
+    for (int i0 = 0; i0 < cnt; i0 += 8) {
+      // eight rows requested before the first is used (rows past cnt repeat the last, weight 0)
+      float2 vv[8];
+      float pi[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = i0 + u < cnt ? i0 + u : cnt - 1;
+        vv[u] = *reinterpret_cast<const float2*>(vbase + (size_t)(base + i) * kHeadDim + 2 * lane);
+        const float w = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), i));
+        pi[u] = i0 + u < cnt ? w : 0.0f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        acc0 += pi[u] * vv[u].x;
+        acc1 += pi[u] * vv[u].y;
+      }
     }
   }
-
-  if (!kSplit) {
-    const float inv = 1.0f / run_sum;  // every query sees at least its own key
-    float* o = out + ((size_t)m * Hq + h) * kHeadDim;
-    *reinterpret_cast<float2*>(o + 2 * lane) = make_float2(acc0 * inv, acc1 * inv);
-    return;
-  }
-
-  // share of this wavefront
-  float* mine = part + ((size_t)h * gridDim.y + blockIdx.y) * kPartStride;
-  *reinterpret_cast<float2*>(mine + 2 + 2 * lane) = make_float2(acc0, acc1);
-  if (lane == 0) {
-    mine[0] = run_max;
-    mine[1] = run_sum;
-  }
-  __threadfence();
-  __shared__ unsigned int s_prev;
-  if (lane == 0) {
-    s_prev = __hip_atomic_fetch_add(counters + h, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  __syncthreads();
-  if (s_prev != gridDim.y - 1) return;
-  __threadfence();
-  // last arrival for this head: merge
-  const int ns = gridDim.y;
-  const float* all = part + (size_t)h * ns * kPartStride;
-  float gmax = -INFINITY;
-  for (int s = 0; s < ns; ++s) gmax = fmaxf(gmax, __builtin_nontemporal_load(all + (size_t)s * kPartStride));
-  float total = 0.0f, o0 = 0.0f, o1 = 0.0f;
-  for (int s = 0; s < ns; ++s) {
-    const float* ps = all + (size_t)s * kPartStride;
-    const float ms = __builtin_nontemporal_load(ps);
-    const float wgt = ms == -INFINITY ? 0.0f : expf(ms - gmax);  // an empty share has max = -inf
-    total += __builtin_nontemporal_load(ps + 1) * wgt;
-    o0 += __builtin_nontemporal_load(ps + 2 + 2 * lane) * wgt;
-    o1 += __builtin_nontemporal_load(ps + 3 + 2 * lane) * wgt;
-  }
-  const float inv = 1.0f / total;
-  float* o = out + (size_t)h * kHeadDim;
-  *reinterpret_cast<float2*>(o + 2 * lane) = make_float2(o0 * inv, o1 * inv);
-  if (lane == 0) counters[h] = 0;  // ready for the next launch
+  const float inv = 1.0f / run_sum;  // every query sees at least its own key
+  float* o = out + ((size_t)m * Hq + h) * kHeadDim;
+  *reinterpret_cast<float2*>(o + 2 * lane) = make_float2(acc0 * inv, acc1 * inv);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -380,10 +337,11 @@ __device__ __forceinline__ void softmax_merge_weights(float m, float m2, float& 
 // A lane holds dims 8*dl..8*dl+7; its RoPE partner dims (d +- 64) are read with a second load.
 template <int kGW, bool kRope>
 __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
-    const float* __restrict__ q, float* __restrict__ kc, float* __restrict__ vc,
-    float* __restrict__ out, int Hq, int Hkv, int max_seq, const int* __restrict__ d_pos0, int pos0,
-    float scale, float* part, unsigned int* counters, const float* __restrict__ k_new,
-    const float* __restrict__ v_new, const float* __restrict__ sin_t, const float* __restrict__ cos_t) {
+    const int* __restrict__ d_pos0, const float* __restrict__ q, const float* __restrict__ sin_t,
+    const float* __restrict__ cos_t, float* __restrict__ kc, float* __restrict__ vc, int Hq, int Hkv,
+    int max_seq, int pos0,  // up to here the arguments arrive preloaded in SGPRs: what the first loads need
+    int ns, float scale, const float* __restrict__ k_new, const float* __restrict__ v_new,
+    float* __restrict__ out, float* part, unsigned int* counters) {
   __shared__ float s_part[kDecWaves][kGW][kPartStride];
   __shared__ unsigned int s_prev;
   const int h0 = blockIdx.x * kGW;             // first query head of this group
@@ -395,7 +353,7 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
   if (pos0 >= max_seq) pos0 = max_seq - 1;     // the caller keeps the position inside the cache
   const int len = pos0 + 1;
   // keys of this workgroup, then of this wavefront (multiples of 4 so that slots stay aligned)
-  const int per_wg = ((len + (int)gridDim.y - 1) / (int)gridDim.y + 15) / 16 * 16;
+  const int per_wg = ((len + ns - 1) / ns + 15) / 16 * 16;
   const int per_wave = per_wg / kDecWaves;
   const int begin = min((int)blockIdx.y * per_wg + wave * per_wave, len);
   const int end = min(begin + per_wave, len);
@@ -553,8 +511,7 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
   __syncthreads();
 
   // the four wavefronts -> one share per head, thread t: head t / 128, dim t % 128
-  const int ns = gridDim.y;
-  for (int t = threadIdx.x; t < kGW * kHeadDim; t += blockDim.x) {
+    for (int t = threadIdx.x; t < kGW * kHeadDim; t += 64 * kDecWaves) {
     const int g = t / kHeadDim, d = t % kHeadDim;
     float mm = -INFINITY;
 #pragma unroll
@@ -580,10 +537,10 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
     s_prev = __hip_atomic_fetch_add(counters + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __syncthreads();
-  if (s_prev != gridDim.y - 1) return;
+  if (s_prev != (unsigned)ns - 1) return;
   // Last workgroup of this head group: merge the shares of all key slices. Every thread requests
   // all headers and its own dim of all shares at once (ns <= kMaxAttnSplit, loads independent).
-  for (int t = threadIdx.x; t < kGW * kHeadDim; t += blockDim.x) {
+  for (int t = threadIdx.x; t < kGW * kHeadDim; t += 64 * kDecWaves) {
     const int g = t / kHeadDim, d = t % kHeadDim;
     const float* all = part + (size_t)(h0 + g) * ns * kPartStride;
     float ms[kMaxAttnSplit], ls[kMaxAttnSplit], as[kMaxAttnSplit];
@@ -760,8 +717,8 @@ hipError_t launch_attention_prefill(const float* q, const float* kc, const float
                                     int M, int Hq, int Hkv, int max_seq, const int* d_pos0, int pos0,
                                     hipStream_t s) {
   const float scale = 1.0f / sqrtf((float)kHeadDim);
-  hipLaunchKernelGGL(attention_kernel<false>, dim3(Hq, M), dim3(64), 0, s, q, kc, vc, out, Hq, Hkv,
-                     max_seq, d_pos0, pos0, scale, nullptr, nullptr);
+  hipLaunchKernelGGL(attention_prefill_kernel, dim3(Hq, M), dim3(64), 0, s, q, kc, vc, out, Hq, Hkv,
+                     max_seq, d_pos0, pos0, scale);
   return hipGetLastError();
 }
 
@@ -776,8 +733,8 @@ hipError_t launch_attention_decode(const float* q, float* kc, float* vc, float* 
   if (nsplit > kMaxAttnSplit) return hipErrorInvalidValue;
 #define W4_ATTN(gw, rope)                                                                              \
   hipLaunchKernelGGL((attention_decode_kernel<gw, rope>), dim3(Hq / gw, nsplit), dim3(64 * kDecWaves), \
-                     0, s, q, kc, vc, out, Hq, Hkv, max_seq, d_pos0, pos0, scale, part, counters,      \
-                     k_new, v_new, sin_t, cos_t)
+                     0, s, d_pos0, q, sin_t, cos_t, kc, vc, Hq, Hkv, max_seq, pos0, nsplit, scale,     \
+                     k_new, v_new, out, part, counters)
   if (G % 2 == 0) {
     if (k_new) W4_ATTN(2, true); else W4_ATTN(2, false);
   } else if (G % 3 == 0) {
