@@ -235,8 +235,9 @@ struct GroupArgs {
 //   and stores silu(y0) * y1 to y[0].
 template <int M, int kFusedR, bool kGrouped, int kCPW, bool kNorm, bool kPair>
 __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
-    const float* __restrict__ x, int ldx, int K, int KC, const uint8_t* packed0, float* y0, int N0,
-    int W, const GroupArgs ga, const RowPrologue pro) {
+    const float* __restrict__ x, int ldx, int K, int KC, int W, const uint8_t* packed0, int N0,
+    const float* pro_delta, const float* pro_norm_w, float pro_eps, float* y0,  // 16 dwords: preloaded
+    float* pro_sum_out, const GroupArgs ga) {
   // The leading scalar arguments (everything a single Linear needs) are preloaded into SGPRs by
   // the dispatcher, so the first loads go out without waiting for the argument segment.
   extern __shared__ __align__(16) uint8_t smem[];
@@ -301,10 +302,10 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
     }
   }
   float dv[kNorm ? M : 1][kNorm ? kFusedR : 1][8];  // delta, then the norm weight
-  if (kNorm && pro.delta) {
+  if (kNorm && pro_delta) {
 #pragma unroll
     for (int m = 0; m < M; ++m) {
-      const float* row = pro.delta + (size_t)m * ldx;
+      const float* row = pro_delta + (size_t)m * ldx;
 #pragma unroll
       for (int r = 0; r < kFusedR; ++r) {
         const int c = threadIdx.x + r * nthreads;
@@ -353,11 +354,11 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
 #pragma unroll
       for (int r = 0; r < kFusedR; ++r) {
         const int c = threadIdx.x + r * nthreads;
-        if (pro.delta) {
+        if (pro_delta) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) xv[m][r][e] += dv[m][r][e];
-          if (pro.sum_out && blockIdx.x == 0 && c < groups) {
-            float* dst = pro.sum_out + (size_t)m * ldx + 8 * c;
+          if (pro_sum_out && blockIdx.x == 0 && c < groups) {
+            float* dst = pro_sum_out + (size_t)m * ldx + 8 * c;
             *reinterpret_cast<float4*>(dst) = make_float4(xv[m][r][0], xv[m][r][1], xv[m][r][2], xv[m][r][3]);
             *reinterpret_cast<float4*>(dst + 4) = make_float4(xv[m][r][4], xv[m][r][5], xv[m][r][6], xv[m][r][7]);
           }
@@ -375,8 +376,8 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
     for (int r = 0; r < kFusedR; ++r) {
       const int c = threadIdx.x + r * nthreads;
       const int cc = c < groups ? c : groups - 1;
-      const float4 v0 = *reinterpret_cast<const float4*>(pro.norm_w + 8 * cc);
-      const float4 v1 = *reinterpret_cast<const float4*>(pro.norm_w + 8 * cc + 4);
+      const float4 v0 = *reinterpret_cast<const float4*>(pro_norm_w + 8 * cc);
+      const float4 v1 = *reinterpret_cast<const float4*>(pro_norm_w + 8 * cc + 4);
       const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
 #pragma unroll
       for (int e = 0; e < 8; ++e) dv[0][r][e] = f[e];
@@ -386,7 +387,7 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
     for (int m = 0; m < M; ++m) {
       const float part = j < W ? s_ss[j * M + m] : 0.0f;
       const float total = row16_sum_all(part);
-      const float rstd = 1.0f / sqrtf(total / (float)K + pro.eps);
+      const float rstd = 1.0f / sqrtf(total / (float)K + pro_eps);
 #pragma unroll
       for (int r = 0; r < kFusedR; ++r) {
 #pragma unroll
@@ -591,11 +592,13 @@ static hipError_t launch_fused_m(const GroupArgs& ga, const float* x, int ldx, i
   if (ga.count == 1 || kPair) {
     auto kern = gemv_fused_kernel<M, R, false, CPW, kNorm, kPair>;
     if (hipError_t e = raise_lds_limit(kern, lds, &raised1); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, grid, block, lds, s, x, ldx, K, KC, ga.packed[0], ga.y[0], ga.N[0], W, ga, pro);
+    hipLaunchKernelGGL(kern, grid, block, lds, s, x, ldx, K, KC, W, ga.packed[0], ga.N[0], pro.delta, pro.norm_w,
+                       pro.eps, ga.y[0], pro.sum_out, ga);
   } else {
     auto kern = gemv_fused_kernel<M, R, true, CPW, kNorm, false>;
     if (hipError_t e = raise_lds_limit(kern, lds, &raisedg); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, grid, block, lds, s, x, ldx, K, KC, ga.packed[0], ga.y[0], ga.N[0], W, ga, pro);
+    hipLaunchKernelGGL(kern, grid, block, lds, s, x, ldx, K, KC, W, ga.packed[0], ga.N[0], pro.delta, pro.norm_w,
+                       pro.eps, ga.y[0], pro.sum_out, ga);
   }
   return hipGetLastError();
 }
