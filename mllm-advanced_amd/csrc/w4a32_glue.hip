@@ -323,13 +323,6 @@ __device__ __forceinline__ void row16_sum(float (&d)[kGW]) {
   asm volatile("s_nop 1");
 }
 
-// (m, l, acc) <- merge with (m2, l2, acc2): softmax partial results over disjoint key sets.
-__device__ __forceinline__ void softmax_merge_weights(float m, float m2, float& w1, float& w2, float& mn) {
-  mn = fmaxf(m, m2);
-  w1 = m == -INFINITY ? 0.0f : __expf(m - mn);
-  w2 = m2 == -INFINITY ? 0.0f : __expf(m2 - mn);
-}
-
 // kRope: q, k_new, v_new are the raw outputs of the q/k/v Linears for the token at position pos0.
 // The kernel rotates q itself, and the wavefront whose share contains key pos0 rotates k_new, uses
 // it and v_new in place of the (not yet written) cache row and - in the first head group of each KV
@@ -342,7 +335,7 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
     int max_seq, int pos0,  // up to here the arguments arrive preloaded in SGPRs: what the first loads need
     int ns, float scale, const float* __restrict__ k_new, const float* __restrict__ v_new,
     float* __restrict__ out, float* part, unsigned int* counters) {
-  __shared__ float s_part[kDecWaves][kGW][kPartStride];
+  __shared__ __align__(16) float s_part[4 * kDecWaves][kGW][kPartStride + 2];  // [wavefront x key slot]
   __shared__ unsigned int s_prev;
   const int h0 = blockIdx.x * kGW;             // first query head of this group
   const int G = Hq / Hkv;
@@ -381,6 +374,23 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
     }
   };
 
+  // The first block of K and V rows depends only on the position: it is requested before q, the
+  // RoPE factors and the new token's k, v, whose latency it then shares instead of following.
+  const float* kbase = kc + (size_t)hk * max_seq * kHeadDim + 8 * dl;
+  const float* vbase = vc + (size_t)hk * max_seq * kHeadDim + 8 * dl;
+  float kk[4][8], vv[4][8];
+  auto load_block = [&](int blk) {
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int key = blk + 4 * it + kq;
+      const int last = end > begin ? end - 1 : 0;
+      const size_t row = (size_t)(key < end ? key : last) * kHeadDim;
+      load8(kbase + row, kk[it]);
+      load8(vbase + row, vv[it]);
+    }
+  };
+  load_block(begin);
+
   float qr[kGW][8];
 #pragma unroll
   for (int g = 0; g < kGW; ++g) {
@@ -405,8 +415,6 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
       *reinterpret_cast<float4*>(vd + 4) = make_float4(vnew[4], vnew[5], vnew[6], vnew[7]);
     }
   }
-  const float* kbase = kc + (size_t)hk * max_seq * kHeadDim + 8 * dl;
-  const float* vbase = vc + (size_t)hk * max_seq * kHeadDim + 8 * dl;
 
   float m[kGW], l[kGW], acc[kGW][8];
 #pragma unroll
@@ -418,25 +426,7 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
   }
 
   for (int blk = begin; blk < end; blk += 16) {
-    float kk[4][8], vv[4][8];
-#pragma unroll
-    for (int it = 0; it < 4; ++it) {
-      const int key = blk + 4 * it + kq;
-      const size_t row = (size_t)(key < end ? key : end - 1) * kHeadDim;
-      const float4 a = *reinterpret_cast<const float4*>(kbase + row);
-      const float4 b = *reinterpret_cast<const float4*>(kbase + row + 4);
-      kk[it][0] = a.x; kk[it][1] = a.y; kk[it][2] = a.z; kk[it][3] = a.w;
-      kk[it][4] = b.x; kk[it][5] = b.y; kk[it][6] = b.z; kk[it][7] = b.w;
-    }
-#pragma unroll
-    for (int it = 0; it < 4; ++it) {
-      const int key = blk + 4 * it + kq;
-      const size_t row = (size_t)(key < end ? key : end - 1) * kHeadDim;
-      const float4 a = *reinterpret_cast<const float4*>(vbase + row);
-      const float4 b = *reinterpret_cast<const float4*>(vbase + row + 4);
-      vv[it][0] = a.x; vv[it][1] = a.y; vv[it][2] = a.z; vv[it][3] = a.w;
-      vv[it][4] = b.x; vv[it][5] = b.y; vv[it][6] = b.z; vv[it][7] = b.w;
-    }
+    if (blk != begin) load_block(blk);  // shares longer than 16 keys per wavefront (max_seq > 1024)
     if (has_new) {
 #pragma unroll
       for (int it = 0; it < 4; ++it) {
@@ -484,45 +474,39 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
     }
   }
 
-  // the four key slots of the wavefront -> lanes 0..15
+  // Every key slot of every wavefront leaves its share in LDS; thread t (head t / 128, dim t % 128)
+  // then merges the 16 of them. (Merging the four slots with cross-lane shuffles first cost three
+  // times as long as these LDS reads.)
 #pragma unroll
   for (int g = 0; g < kGW; ++g) {
-#pragma unroll
-    for (int off = 16; off <= 32; off <<= 1) {
-      const float m2 = __shfl_xor(m[g], off, 64);
-      const float l2 = __shfl_xor(l[g], off, 64);
-      float w1, w2, mn;
-      softmax_merge_weights(m[g], m2, w1, w2, mn);
-      l[g] = l[g] * w1 + l2 * w2;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) acc[g][i] = acc[g][i] * w1 + __shfl_xor(acc[g][i], off, 64) * w2;
-      m[g] = mn;
+    float* dst = &s_part[wave * 4 + kq][g][0];
+    if (dl == 0) {
+      dst[kHeadDim] = m[g];
+      dst[kHeadDim + 1] = l[g];
     }
-    if (kq == 0) {
-      float* dst = &s_part[wave][g][0];
-      if (dl == 0) {
-        dst[0] = m[g];
-        dst[1] = l[g];
-      }
-#pragma unroll
-      for (int i = 0; i < 8; ++i) dst[2 + 8 * dl + i] = acc[g][i];
-    }
+    *reinterpret_cast<float4*>(dst + 8 * dl) = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
+    *reinterpret_cast<float4*>(dst + 8 * dl + 4) = make_float4(acc[g][4], acc[g][5], acc[g][6], acc[g][7]);
   }
   __syncthreads();
 
-  // the four wavefronts -> one share per head, thread t: head t / 128, dim t % 128
-    for (int t = threadIdx.x; t < kGW * kHeadDim; t += 64 * kDecWaves) {
+  for (int t = threadIdx.x; t < kGW * kHeadDim; t += 64 * kDecWaves) {
     const int g = t / kHeadDim, d = t % kHeadDim;
+    float ms[4 * kDecWaves], ls[4 * kDecWaves], as[4 * kDecWaves];
+#pragma unroll
+    for (int w = 0; w < 4 * kDecWaves; ++w) {
+      ms[w] = s_part[w][g][kHeadDim];
+      ls[w] = s_part[w][g][kHeadDim + 1];
+      as[w] = s_part[w][g][d];
+    }
     float mm = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < kDecWaves; ++w) mm = fmaxf(mm, s_part[w][g][0]);
+    for (int w = 0; w < 4 * kDecWaves; ++w) mm = fmaxf(mm, ms[w]);
     float ll = 0.0f, a = 0.0f;
 #pragma unroll
-    for (int w = 0; w < kDecWaves; ++w) {
-      const float mw = s_part[w][g][0];
-      const float wt = mw == -INFINITY ? 0.0f : __expf(mw - mm);
-      ll += s_part[w][g][1] * wt;
-      a += s_part[w][g][2 + d] * wt;
+    for (int w = 0; w < 4 * kDecWaves; ++w) {
+      const float wt = ms[w] == -INFINITY ? 0.0f : __expf(ms[w] - mm);
+      ll += ls[w] * wt;
+      a += as[w] * wt;
     }
     float* mine = part + ((size_t)(h0 + g) * ns + blockIdx.y) * kPartStride;
     store_shared_across_wgs(mine + 2 + d, a);
