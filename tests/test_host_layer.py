@@ -10,6 +10,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HOST = os.path.join(ROOT, "mllm-advanced_amd", "host")
 BIN = os.path.join(HOST, "tests", "hip_linear_test")
+BIN_MODEL = os.path.join(HOST, "tests", "hip_qwen2_test")
 LIB = os.path.join(ROOT, "mllm-advanced_amd", "libmllm_hip_backend.so")
 
 
@@ -17,7 +18,7 @@ def test_backend_library_is_built_and_loads():
     assert os.path.exists(LIB), "run __graft_entry__.build()"
     ctypes.CDLL(os.path.join(ROOT, "mllm-advanced_amd", "libw4a32_hip.so"), mode=ctypes.RTLD_GLOBAL)
     ctypes.CDLL(LIB)
-    assert os.path.exists(BIN)
+    assert os.path.exists(BIN) and os.path.exists(BIN_MODEL)
 
 
 def test_container_structs_have_the_on_disk_sizes():
@@ -34,3 +35,50 @@ def test_cpp_operator_tests_pass(tmp_path):
     print(out.stderr[-2000:])
     assert out.returncode == 0, out.stdout[-2000:] + out.stderr[-2000:]
     assert "[ PASSED ]" in out.stdout
+
+
+@pytest.mark.gpu
+def test_cpp_model_generates_what_the_oracle_generates(tmp_path):
+    """The C++ model class writes a tiny Qwen2-shaped .mllm file under the reference's parameter
+    names, loads it and generates greedily (prefill in two slices, first step eager, the rest from a
+    HIP graph). The same file is read here and run through the numpy oracle, teacher-forced with the
+    tokens the binary printed: every printed token must be the oracle's greedy choice."""
+    import numpy as np
+
+    import decoder_oracle as do
+    from mllm_file import read
+
+    out = subprocess.run([BIN_MODEL, str(tmp_path)], capture_output=True, text=True, timeout=300)
+    print(out.stdout[-3000:])
+    print(out.stderr[-2000:])
+    assert out.returncode == 0 and "[ PASSED ]" in out.stdout
+    line = [l for l in out.stdout.splitlines() if l.startswith("TOKENS:")][0]
+    tokens = [int(t) for t in line.split()[1:]]
+    assert len(tokens) == 14
+
+    model_name, p = read(os.path.join(str(tmp_path), "tiny_qwen2.mllm"))
+    assert model_name == "tiny-qwen2" and p["model.embed_tokens.weight"].shape == (640, 256)
+    layers = []
+    for i in range(2):
+        b = f"model.layers.{i}."
+        layers.append({
+            "q": p[b + "self_attn.q_proj.weight"], "q_bias": p[b + "self_attn.q_proj.bias"],
+            "k": p[b + "self_attn.k_proj.weight"], "k_bias": p[b + "self_attn.k_proj.bias"],
+            "v": p[b + "self_attn.v_proj.weight"], "v_bias": p[b + "self_attn.v_proj.bias"],
+            "o": p[b + "self_attn.o_proj.weight"], "gate": p[b + "mlp.gate_proj.weight"],
+            "up": p[b + "mlp.up_proj.weight"], "down": p[b + "mlp.down_proj.weight"],
+            "attn_norm": p[b + "input_layernorm.weight"], "ffn_norm": p[b + "post_attention_layernorm.weight"]})
+    weights = {"embedding": p["model.embed_tokens.weight"], "final_norm": p["model.norm.weight"],
+               "lm_head": p["lm_head.weight"], "layers": layers}
+    ref = do.Decoder(weights, 2, 1, rope_theta=1e6, max_seq=64)
+    prompt = [3, 17, 100, 42, 7, 250, 611, 5, 98, 301, 77]
+    logits = ref.forward(prompt)
+    margins = []
+    for i, tok in enumerate(tokens):
+        top2 = np.sort(logits)[-2:]
+        margins.append(float(top2[1] - top2[0]))
+        # the oracle's choice, unless its two best logits are closer than the 2e-3 parity tolerance
+        assert do.greedy(logits) == tok or margins[-1] < 2e-3 * float(np.abs(logits).max()), (i, tok)
+        if i + 1 < len(tokens):
+            logits = ref.forward([tok])
+    assert max(margins) > 0.01        # the comparison was not vacuous
