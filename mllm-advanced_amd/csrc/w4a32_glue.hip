@@ -288,6 +288,165 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(const float* __re
 }
 
 // ---------------------------------------------------------------------------------------------
+// Prefill attention on the matrix cores, all in f32 (v_mfma_f32_32x32x2_f32): workgroup = one
+// head x 32 queries, its 4 wavefronts take the 32-key blocks round-robin and are merged through LDS.
+//
+// Both products are computed transposed so that a lane always stands for one QUERY:
+//   S^T = K Q^T   A = K block (lane: key l%32, dims 64*(l/32) + i), B = Q^T (lane: query l%32, same dims)
+//                 C: lane = query l%32, register v = key 8*(v/4) + 4*(l/32) + v%4 of the block
+//   O^T += V^T P^T  B = P^T = the softmaxed C registers as they are (step i uses register i: the
+//                 two k-slots of the instruction are then keys 8*(i/4) + i%4 and that + 4),
+//                 A = V^T (lane j = l%32 loads the float4 V[key][4j..4j+3]: component c feeds dim block c,
+//                 whose row j stands for dim 4j + c)
+//                 C: lane = query, register v of block c = dim 4*(8*(v/4) + 4*(l/32) + v%4) + c
+// so the online-softmax statistics and the rescaling of O are per-lane scalars, and no operand
+// needs a transpose.
+// ---------------------------------------------------------------------------------------------
+typedef float v16f32 __attribute__((ext_vector_type(16)));
+constexpr int kPfWaves = 4;
+
+__global__ __launch_bounds__(64 * kPfWaves) void attention_prefill_mfma_kernel(
+    const float* __restrict__ q, const float* __restrict__ kc, const float* __restrict__ vc,
+    float* __restrict__ out, int M, int Hq, int Hkv, int max_seq, const int* __restrict__ d_pos0,
+    int pos0, float scale) {
+  extern __shared__ __align__(16) float s_merge[];  // [kPfWaves - 1][66][64]: O^T registers, max, sum
+  const int h = blockIdx.x, qb = blockIdx.y;
+  const int hk = h / (Hq / Hkv);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int j = lane & 31, hh = lane >> 5;
+  if (d_pos0) pos0 = *d_pos0;
+
+  const int m_q = min(32 * qb + j, M - 1);           // this lane's query row (rows past M repeat the last)
+  const int q_pos = pos0 + m_q;                        // its position: it sees keys 0..q_pos
+  const int last_key = min(pos0 + min(32 * qb + 31, M - 1), max_seq - 1);
+  const int nkb = last_key / 32 + 1;                   // key blocks this query block touches
+
+  float qreg[64];
+  {
+    const float4* src = reinterpret_cast<const float4*>(q + ((size_t)m_q * Hq + h) * kHeadDim + 64 * hh);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float4 v = src[i];
+      qreg[4 * i] = v.x; qreg[4 * i + 1] = v.y; qreg[4 * i + 2] = v.z; qreg[4 * i + 3] = v.w;
+    }
+  }
+  const float* kbase = kc + (size_t)hk * max_seq * kHeadDim;
+  const float* vbase = vc + (size_t)hk * max_seq * kHeadDim;
+
+  v16f32 o[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[c][v] = 0.0f;
+  float run_max = -INFINITY, run_sum = 0.0f;
+
+  for (int kb = wave; kb < nkb; kb += kPfWaves) {
+    // S^T block
+    const int key_a = min(32 * kb + j, last_key);
+    const float4* ksrc = reinterpret_cast<const float4*>(kbase + (size_t)key_a * kHeadDim + 64 * hh);
+    v16f32 st;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) st[v] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float4 kv = ksrc[i];
+      st = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.x, qreg[4 * i], st, 0, 0, 0);
+      st = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.y, qreg[4 * i + 1], st, 0, 0, 0);
+      st = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.z, qreg[4 * i + 2], st, 0, 0, 0);
+      st = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.w, qreg[4 * i + 3], st, 0, 0, 0);
+    }
+    // V rows of this lane's 16 keys (both halves of the wavefront read whole 512-byte rows)
+    float4 vreg[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int key = min(32 * kb + 8 * (v >> 2) + 4 * hh + (v & 3), last_key);
+      vreg[v] = *reinterpret_cast<const float4*>(vbase + (size_t)key * kHeadDim + 4 * j);
+    }
+    // causal mask, online softmax (a query's 32 scores of the block sit in lanes j and j + 32)
+    float blk_max = -INFINITY;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int key = 32 * kb + 8 * (v >> 2) + 4 * hh + (v & 3);
+      st[v] = key <= q_pos ? st[v] * scale : -INFINITY;
+      blk_max = fmaxf(blk_max, st[v]);
+    }
+    blk_max = fmaxf(blk_max, __shfl_xor(blk_max, 32, 64));
+    const float new_max = fmaxf(run_max, blk_max);
+    // new_max = -inf only while every key so far was masked for this query: all weights 0
+    const float corr = run_max == -INFINITY ? 0.0f : __expf(run_max - new_max);
+    float psum = 0.0f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      st[v] = st[v] == -INFINITY ? 0.0f : __expf(st[v] - new_max);
+      psum += st[v];
+    }
+    psum += __shfl_xor(psum, 32, 64);
+    run_sum = run_sum * corr + psum;
+    run_max = new_max;
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o[c][v] *= corr;
+    // O^T += V^T P^T
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      o[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(vreg[i].x, st[i], o[0], 0, 0, 0);
+      o[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(vreg[i].y, st[i], o[1], 0, 0, 0);
+      o[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(vreg[i].z, st[i], o[2], 0, 0, 0);
+      o[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(vreg[i].w, st[i], o[3], 0, 0, 0);
+    }
+  }
+
+  // wavefronts 1..3 hand their (max, sum, O^T) to wavefront 0
+  if (wave > 0) {
+    float* dst = s_merge + (size_t)(wave - 1) * 66 * 64 + lane;
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) dst[(16 * c + v) * 64] = o[c][v];
+    dst[64 * 64] = run_max;
+    dst[65 * 64] = run_sum;
+  }
+  __syncthreads();
+  if (wave > 0) return;
+  float wmax[kPfWaves - 1], wsum[kPfWaves - 1];
+  float total_max = run_max;
+#pragma unroll
+  for (int w = 0; w < kPfWaves - 1; ++w) {
+    wmax[w] = s_merge[(size_t)w * 66 * 64 + 64 * 64 + lane];
+    wsum[w] = s_merge[(size_t)w * 66 * 64 + 65 * 64 + lane];
+    total_max = fmaxf(total_max, wmax[w]);
+  }
+  const float own_w = run_max == -INFINITY ? 0.0f : __expf(run_max - total_max);
+  float total_sum = run_sum * own_w;
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[c][v] *= own_w;
+#pragma unroll
+  for (int w = 0; w < kPfWaves - 1; ++w) {
+    const float wt = wmax[w] == -INFINITY ? 0.0f : __expf(wmax[w] - total_max);
+    total_sum += wsum[w] * wt;
+    const float* src = s_merge + (size_t)w * 66 * 64 + lane;
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o[c][v] += src[(16 * c + v) * 64] * wt;
+  }
+  // lane = query; register v of block c = dim 4*(8*(v/4) + 4*hh + v%4) + c: four blocks -> one float4
+  if (32 * qb + j < M) {
+    const float inv = 1.0f / total_sum;  // every query sees at least its own key
+    float* dst = out + ((size_t)(32 * qb + j) * Hq + h) * kHeadDim;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int row = 8 * (v >> 2) + 4 * hh + (v & 3);
+      *reinterpret_cast<float4*>(dst + 4 * row) =
+          make_float4(o[0][v] * inv, o[1][v] * inv, o[2][v] * inv, o[3][v] * inv);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // Decode attention (one query row): workgroup (x = group of kGW query heads that share a KV head,
 // y = slice of the cached keys), 4 wavefronts per workgroup, each taking a quarter of the slice
 // in blocks of 16 keys.
@@ -701,8 +860,14 @@ hipError_t launch_attention_prefill(const float* q, const float* kc, const float
                                     int M, int Hq, int Hkv, int max_seq, const int* d_pos0, int pos0,
                                     hipStream_t s) {
   const float scale = 1.0f / sqrtf((float)kHeadDim);
-  hipLaunchKernelGGL(attention_prefill_kernel, dim3(Hq, M), dim3(64), 0, s, q, kc, vc, out, Hq, Hkv,
-                     max_seq, d_pos0, pos0, scale);
+  if (M >= 16) {  // matrix-core kernel: 32 queries per workgroup
+    const size_t lds = sizeof(float) * (kPfWaves - 1) * 66 * 64;
+    hipLaunchKernelGGL(attention_prefill_mfma_kernel, dim3(Hq, (M + 31) / 32), dim3(64 * kPfWaves), lds, s,
+                       q, kc, vc, out, M, Hq, Hkv, max_seq, d_pos0, pos0, scale);
+  } else {
+    hipLaunchKernelGGL(attention_prefill_kernel, dim3(Hq, M), dim3(64), 0, s, q, kc, vc, out, Hq, Hkv,
+                       max_seq, d_pos0, pos0, scale);
+  }
   return hipGetLastError();
 }
 
