@@ -133,7 +133,6 @@ __device__ __forceinline__ uint4 dequant8(uint32_t w, h2 s, h2 s16) {
 }
 
 constexpr int kF16BK = 64;    // k per stage (two scale blocks, half of a weight tile chunk)
-constexpr int kF16Depth = 2;  // stages in flight between a global load and its use
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
@@ -148,20 +147,22 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 //
 //  * A (f16 activations) never touches LDS: the row quantiser already wrote it as 2 KiB chunks
 //    of 32 rows x 32 k, so the two operand loads of a block read one contiguous chunk (instead
-//    of 32 rows that lie K*2 bytes apart), into a register ring kF16Depth stages deep (a load
+//    of 32 rows that lie K*2 bytes apart), into a register ring DEPTH stages deep (a load
 //    has that many stages of MFMA work to land).
 //  * B (4-bit weights) is shared by the four wavefronts: its packed bytes are prefetched into
 //    a small register ring, dequantised once per workgroup to f16 and double-buffered in LDS
 //    as 1 KiB fragments in lane order (lane l at l*16: conflict-free 128-bit accesses).
 //  * One barrier per stage: it publishes the B buffer written during the previous stage and
 //    frees the one read during it.
-template <int WAVES_M, int WAVES_N, int WM, int WN>
+// DEPTH = stages between a global load and its use: 2 for the large tiles (registers), 4 for the
+// small ones, whose stages are short next to the memory latency.
+template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_f16_kernel(
     float* __restrict__ y, const _Float16* __restrict__ ah, const float* __restrict__ recip,
     const uint8_t* __restrict__ packed, const uint8_t* __restrict__ hscale,
     const float* __restrict__ rowmul, const float* __restrict__ bias, int M, int N, int K, int NT,
     int KC, int MB, int NB, int n_major) {
-  constexpr int D = kF16Depth;
+  constexpr int D = DEPTH;
   constexpr int NWAVES = WAVES_M * WAVES_N;
   constexpr int BM = 32 * WM * WAVES_M;
   constexpr int BN32 = WN * WAVES_N;           // 32-column fragments per workgroup and k-slice
@@ -353,7 +354,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_f16_kernel(
   }
 }
 
-template <int WAVES_M, int WAVES_N, int WM, int WN>
+template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH>
 static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                              hipStream_t s) {
   constexpr int BM = 32 * WM * WAVES_M, WNT = 2 * WN * WAVES_N;
@@ -364,7 +365,7 @@ static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed,
   // keep together what is more expensive to fetch eight times: the f16 activations (2 bytes per
   // element) or the packed weights (0.5625 bytes per element)
   const int n_major = (double)M * 2.0 <= (double)N * 0.5625 ? 1 : 0;
-  hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN>), dim3(grid),
+  hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH>), dim3(grid),
                      dim3(64 * WAVES_M * WAVES_N), 0, s, y,
                      reinterpret_cast<const _Float16*>(ws + w.ah_off),
                      reinterpret_cast<const float*>(ws + w.scale_off), packed,
@@ -401,10 +402,10 @@ hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M
     return launch_gemm_i8(y, ws, packed, M, K, N, s);
   }
   const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-  if (tiles < 128) return launch_f16<2, 2, 1, 1>(y, ws, packed, M, K, N, s);   //  64 x  64
-  if (tiles < 512) return launch_f16<4, 1, 1, 2>(y, ws, packed, M, K, N, s);   // 128 x  64
-  if (tiles < 1024) return launch_f16<4, 2, 1, 2>(y, ws, packed, M, K, N, s);  // 128 x 128, 8 wavefronts
-  return launch_f16<4, 1, 1, 4>(y, ws, packed, M, K, N, s);                    // 128 x 128, 4 wavefronts
+  if (tiles < 128) return launch_f16<2, 2, 1, 1, 8>(y, ws, packed, M, K, N, s);   //  64 x  64
+  if (tiles < 512) return launch_f16<4, 1, 1, 2, 2>(y, ws, packed, M, K, N, s);   // 128 x  64
+  if (tiles < 1024) return launch_f16<4, 2, 1, 2, 2>(y, ws, packed, M, K, N, s);  // 128 x 128, 8 wavefronts
+  return launch_f16<4, 1, 1, 4, 2>(y, ws, packed, M, K, N, s);                    // 128 x 128, 4 wavefronts
 }
 
 }  // namespace w4
