@@ -163,6 +163,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_f16_kernel(
     const float* __restrict__ rowmul, const float* __restrict__ bias, int M, int N, int K, int NT,
     int KC, int MB, int NB, int n_major) {
   constexpr int D = DEPTH;
+  static_assert(D % 2 == 0, "stage s uses LDS buffer s & 1: the unrolled ring must keep that parity");
   constexpr int NWAVES = WAVES_M * WAVES_N;
   constexpr int BM = 32 * WM * WAVES_M;
   constexpr int BN32 = WN * WAVES_N;           // 32-column fragments per workgroup and k-slice
