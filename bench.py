@@ -246,14 +246,23 @@ def main():
             else:
                 lins = [layer[idx] for layer in layers]
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            for l in lins:
-                L.w4a32_matmul(y_by_n[N].data_ptr(), x_by_k[K].data_ptr(), l.packed.data_ptr(),
-                               ws_by_k[K].data_ptr(), 1, K, N, sptr)
-            e0.record(stream)
-            for _ in range(reps):
+
+            def one_round(lins=lins, K=K, N=N):
                 for l in lins:
                     L.w4a32_matmul(y_by_n[N].data_ptr(), x_by_k[K].data_ptr(), l.packed.data_ptr(),
                                    ws_by_k[K].data_ptr(), 1, K, N, sptr)
+            one_round()
+            stream.synchronize()
+            run = one_round
+            if use_graph:      # as in the step: launch period on the device, not the host's call rate
+                g_shape = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g_shape, stream=stream):
+                    one_round()
+                run = g_shape.replay
+                run()
+            e0.record(stream)
+            for _ in range(reps):
+                run()
             e1.record(stream)
             stream.synchronize()
             us = e0.elapsed_time(e1) * 1e3 / (reps * len(lins))
