@@ -146,6 +146,11 @@ int w4a32_matmul_quantized_ex(float* d_y, const void* d_ws, const void* d_packed
       if (M <= w4::kGemvMaxM) return W4A32_ESHAPE;  // the f16 activation copy exists only for M > 8
       return from_hip(w4::launch_gemm(d_y, ws, pk, M, K, N, w4::kKernelGemmF16, s));
     default:
+      if (kernel >= W4A32_KERNEL_GEMM_F16_TILE0 &&
+          kernel < W4A32_KERNEL_GEMM_F16_TILE0 + W4A32_GEMM_F16_TILES) {
+        if (M <= w4::kGemvMaxM) return W4A32_ESHAPE;
+        return from_hip(w4::launch_gemm(d_y, ws, pk, M, K, N, kernel, s));
+      }
       return W4A32_EINVAL;
   }
 }

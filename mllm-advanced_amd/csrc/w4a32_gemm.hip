@@ -136,28 +136,29 @@ constexpr int kF16BK = 64;    // k per stage (two scale blocks, half of a weight
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-// v_mfma_f32_32x32x16_f16 (measured on MI355X: 2.1-2.2 PFLOP/s, twice the 16x16x32 shape).
-// Operands: lane l = 32*h + i holds 8 f16 of row/column i at "k-slot" h. Which k values a slot
-// stands for is free as long as A and B agree; here, inside a 32-k scale block, slice 0 is
-// k {0..7 | 16..23} for h = {0 | 1} and slice 1 is k {8..15 | 24..31}, so that one lane's two A
-// operands of a block are 32 contiguous bytes of its activation row.
+// v_mfma_f32_32x32x16_f16 (8 passes of 4 clocks; measured on MI355X: twice the rate of the
+// 16x16x32 shape). Operands: lane l = 32*h + i holds 8 f16 of row/column i at "k-slot" h. Which k
+// values a slot stands for is free as long as A and B agree; here, inside a 32-k scale block,
+// slice 0 is k {0..7 | 16..23} for h = {0 | 1} and slice 1 is k {8..15 | 24..31}, so that one
+// lane's two A operands of a block are 32 contiguous bytes of its activation row.
 //
-// Workgroup = 4 wavefronts stacked along M; wavefront w owns rows [32*WM*w, 32*WM*(w+1)) of
-// the BM x BN tile (BM = 128*WM, BN = 32*WN) and all BN columns.
+// Workgroup = WAVES_M x WAVES_N wavefronts on a BM x BN tile (BM = 32*WM*WAVES_M,
+// BN = 32*WN*WAVES_N); a wavefront owns WM x WN blocks of 32 x 32 outputs.
 //
 //  * A (f16 activations) never touches LDS: the row quantiser already wrote it as 2 KiB chunks
 //    of 32 rows x 32 k, so the two operand loads of a block read one contiguous chunk (instead
-//    of 32 rows that lie K*2 bytes apart), into a register ring DEPTH stages deep (a load
-//    has that many stages of MFMA work to land).
-//  * B (4-bit weights) is shared by the four wavefronts: its packed bytes are prefetched into
-//    a small register ring, dequantised once per workgroup to f16 and double-buffered in LDS
-//    as 1 KiB fragments in lane order (lane l at l*16: conflict-free 128-bit accesses).
+//    of 32 rows that lie K*2 bytes apart), into a register ring DEPTH stages deep.
+//  * B (4-bit weights) is shared by the wavefronts: its packed bytes are prefetched into a small
+//    register ring, dequantised once per workgroup to f16 and double-buffered in LDS as 1 KiB
+//    fragments in lane order (lane l at l*16: conflict-free 128-bit accesses).
 //  * One barrier per stage: it publishes the B buffer written during the previous stage and
 //    frees the one read during it.
-// DEPTH = stages between a global load and its use: 2 for the large tiles (registers), 4 for the
-// small ones, whose stages are short next to the memory latency.
-template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_f16_kernel(
+//  * What bounds a stage (measured): LDS moves 128 bytes per clock and CU, and a B fragment is
+//    read once per WM products, so WM = 1 costs 160 bytes per clock at the full product rate
+//    (reads + the tile's own writes): LDS-bound. WM = 2 needs 80. A is read once per WN products
+//    through the vector L1 (64 bytes per clock and CU): WN = 4 needs 32.
+template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH, int OCC>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
     float* __restrict__ y, const _Float16* __restrict__ ah, const float* __restrict__ recip,
     const uint8_t* __restrict__ packed, const uint8_t* __restrict__ hscale,
     const float* __restrict__ rowmul, const float* __restrict__ bias, int M, int N, int K, int NT,
@@ -171,11 +172,18 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_f16_kernel(
   static_assert(WNT % NWAVES == 0, "each wavefront dequantises WNT/NWAVES tile rows per stage");
   constexpr int B_UNITS = WNT / NWAVES;        // 8-byte pieces of packed B per thread per stage
   constexpr int kBufBytes = 4 * BN32 * 1024;   // one B stage: [4 k-slices][BN32 fragments]
+  constexpr int SL = 4;                        // k-slices of a stage
+  constexpr int AKB = 2;                       // activation k-blocks (32 k) of a stage
+  constexpr int kMfma = SL * WM * WN;          // products per wavefront and stage
+  constexpr int NDW = 2 * B_UNITS;             // packed dwords a thread dequantises per stage
+  constexpr int NSTEP = 4 * NDW;               // in four steps each
+  static_assert(2 * kBufBytes <= 65536, "static LDS");
 
   __shared__ __align__(16) uint8_t sB[2 * kBufBytes];
 
   const int t = threadIdx.x;
-  const int wave = t >> 6, lane = t & 63;
+  const int lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // scalar: what derives from it is too
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int g = lane >> 4, j = lane & 15;     // position inside a weight tile
   const int h = lane >> 5, i32 = lane & 31;   // position inside an MFMA operand / C tile
@@ -194,7 +202,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_f16_kernel(
   const int nt0 = nb * WNT;
   const int nstages = (K + kF16BK - 1) / kF16BK;
 
-  uint4 areg[D][2][WM][2];  // [ring slot][k-block][32-row tile][slice of the block]
+  uint4 areg[D][AKB][WM][2];  // [ring slot][k-block][32-row tile][slice of the block]
   uint2 breg[D][B_UNITS];
   uint32_t sreg[D][B_UNITS];
 
@@ -224,18 +232,15 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_f16_kernel(
   // numbers and k-blocks are clamped to valid addresses, and what must not contribute is
   // multiplied by a zero scale (padded stages) or meets the zero nibbles and zero scales that
   // pad every weight tile (k >= K).
-  auto load_a = [&](int s, uint4 (&dst)[2][WM][2]) {
+  auto load_a_kb = [&](int s, int kbl, uint4 (&dst)[AKB][WM][2]) {
     const int sc = s < nstages ? s : nstages - 1;
+    int blk = 2 * sc + kbl;
+    blk = blk < KB ? blk : KB - 1;
+    const int off = blk * 2048;
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      int blk = 2 * sc + kb;
-      blk = blk < KB ? blk : KB - 1;
-      const int off = blk * 2048;
-#pragma unroll
-      for (int a = 0; a < WM; ++a) {
-        dst[kb][a][0] = *reinterpret_cast<const uint4*>(a_ptr[a] + off);
-        dst[kb][a][1] = *reinterpret_cast<const uint4*>(a_ptr[a] + off + 16);
-      }
+    for (int a = 0; a < WM; ++a) {
+      dst[kbl][a][0] = *reinterpret_cast<const uint4*>(a_ptr[a] + off);
+      dst[kbl][a][1] = *reinterpret_cast<const uint4*>(a_ptr[a] + off + 16);
     }
   };
 
@@ -253,24 +258,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_f16_kernel(
 
   // Tile lane (g, j) of tile row ntl, block dd -> fragment (slice 2*dd + (g & 1), column tile
   // ntl / 2), operand lane 32*(g >> 1) + 16*(ntl & 1) + j.
-  // `s` is the stage the registers hold; a stage past the end (loaded from clamped addresses)
-  // gets scale 0. The mask is applied here, at use, so that the load itself has no consumer
-  // until D stages later.
-  auto store_b = [&](int s, int buf, const uint2 (&q)[B_UNITS], const uint32_t (&sc)[B_UNITS]) {
-    const uint32_t keep = s < nstages ? 0xFFFFFFFFu : 0u;
-    const h2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
-#pragma unroll
-    for (int u = 0; u < B_UNITS; ++u) {
-      const int ntl = wave + NWAVES * u;
-      const h2 s2 = __builtin_bit_cast(h2, sc[u] & keep);
-      const h2 s2_16 = s2 * sixteenth;
-      const h2 s_lo = {s2[0], s2[0]}, s_lo16 = {s2_16[0], s2_16[0]};
-      const h2 s_hi = {s2[1], s2[1]}, s_hi16 = {s2_16[1], s2_16[1]};
-      const int op_lane = 32 * (g >> 1) + 16 * (ntl & 1) + j;
-      uint8_t* base = sB + buf * kBufBytes + ((g & 1) * BN32 + (ntl >> 1)) * 1024 + 16 * op_lane;
-      *reinterpret_cast<uint4*>(base) = dequant8(q[u].x, s_lo, s_lo16);                    // block 0
-      *reinterpret_cast<uint4*>(base + 2 * BN32 * 1024) = dequant8(q[u].y, s_hi, s_hi16);  // block 1
-    }
+  auto frag_ptr = [&](int buf, int unit, int dd) {
+    const int ntl = wave + NWAVES * unit;
+    const int op_lane = 32 * (g >> 1) + 16 * (ntl & 1) + j;
+    return sB + buf * kBufBytes + ((2 * dd + (g & 1)) * BN32 + (ntl >> 1)) * 1024 + 16 * op_lane;
   };
 
   v16f acc[WM][WN];
@@ -281,43 +272,101 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_f16_kernel(
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
 
-  // Prologue: A stages 0..D-1 and B stages 0..D in flight; B stage 0 goes to LDS buffer 0.
-#pragma unroll
-  for (int p = 0; p < D; ++p) load_a(p, areg[p]);
+  // Prologue: A stages 0..D-1 and B stages 0..D in flight; B stage 0 goes to LDS buffer 0. The
+  // loads are issued in the loop's own order (per stage: B, then A): the compiler derives each
+  // wait in the loop from the fewest loads that can be younger than the one it needs on any way
+  // into the loop, so a prologue with another order makes the loop wait for newer loads than it
+  // uses.
   {
     uint2 q0[B_UNITS];
     uint32_t s0[B_UNITS];
     load_b(0, q0, s0);
 #pragma unroll
-    for (int p = 0; p < D; ++p) load_b(p + 1, breg[p], sreg[p]);  // ring slot p holds stage p+1
-    store_b(0, 0, q0, s0);
+    for (int p = 0; p < D; ++p) {
+      load_b(p + 1, breg[p], sreg[p]);  // ring slot p holds stage p+1
+#pragma unroll
+      for (int kbl = 0; kbl < AKB; ++kbl) load_a_kb(p, kbl, areg[p]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    const h2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+#pragma unroll
+    for (int u = 0; u < B_UNITS; ++u) {
+      const h2 s2 = __builtin_bit_cast(h2, s0[u]);
+      const h2 s2_16 = s2 * sixteenth;
+      *reinterpret_cast<uint4*>(frag_ptr(0, u, 0)) =
+          dequant8(q0[u].x, h2{s2[0], s2[0]}, h2{s2_16[0], s2_16[0]});
+      *reinterpret_cast<uint4*>(frag_ptr(0, u, 1)) =
+          dequant8(q0[u].y, h2{s2[1], s2[1]}, h2{s2_16[1], s2_16[1]});
+    }
   }
 
   // Stages are processed D at a time (ring slot u and LDS buffer u & 1 are then compile-time
   // constants); the stage count is rounded up to a multiple of D, extra stages multiply by 0.
+  //
+  // The order inside a stage is written out and fenced (sched_barrier) product by product: a
+  // product occupies the matrix pipe for 32 clocks but its issue slot for 4, so the same
+  // wavefront dequantises the next stage's weights, a few instructions at a time, and issues its
+  // LDS and global traffic in the gaps between its own products. (Left to the scheduler, all of a
+  // stage's dequantisation ran first and the products after it.)
   for (int s_base = 0; s_base < nstages; s_base += D) {
 #pragma unroll
     for (int u = 0; u < D; ++u) {
       const int s = s_base + u;
       __syncthreads();
-      // B of stage s+1 (ring slot u) -> the LDS buffer not being read; refill the slot
-      store_b(s + 1, (u + 1) & 1, breg[u], sreg[u]);
-      load_b(s + 1 + D, breg[u], sreg[u]);
-
-      // B fragments come from LDS one k-slice ahead of the MFMAs that use them.
       const uint8_t* bbuf = sB + (u & 1) * kBufBytes + 16 * lane;
       h8 bf[2][WN];
 #pragma unroll
       for (int b = 0; b < WN; ++b)
         bf[0][b] = *reinterpret_cast<const h8*>(bbuf + (wn * WN + b) * 1024);
+      __builtin_amdgcn_sched_barrier(0);  // requested first: their latency covers what follows
+      // Inputs of the dequantisation (stage s+1, ring slot u) move to temporaries, which frees the
+      // slot for its next load. A stage past the end (loaded from clamped addresses) gets scale 0.
+      uint32_t dx[NDW];
+      h2 dsc[NDW], dsc16[NDW];
+      {
+        const uint32_t keep = s + 1 < nstages ? 0xFFFFFFFFu : 0u;
+        const h2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
 #pragma unroll
-      for (int sl = 0; sl < 4; ++sl) {
-        if (sl < 3) {
-#pragma unroll
-          for (int b = 0; b < WN; ++b)
-            bf[(sl + 1) & 1][b] =
-                *reinterpret_cast<const h8*>(bbuf + ((sl + 1) * BN32 + wn * WN + b) * 1024);
+        for (int q = 0; q < B_UNITS; ++q) {
+          const h2 s2 = __builtin_bit_cast(h2, sreg[u][q] & keep);
+          const h2 s2_16 = s2 * sixteenth;
+          dsc[2 * q] = h2{s2[0], s2[0]};
+          dsc16[2 * q] = h2{s2_16[0], s2_16[0]};
+          dsc[2 * q + 1] = h2{s2[1], s2[1]};
+          dsc16[2 * q + 1] = h2{s2_16[1], s2_16[1]};
+          dx[2 * q] = breg[u][q].x ^ 0x88888888u;  // two's complement nibbles -> offset-8 nibbles
+          dx[2 * q + 1] = breg[u][q].y ^ 0x88888888u;
         }
+      }
+      load_b(s + 1 + D, breg[u], sreg[u]);
+      __builtin_amdgcn_sched_barrier(0);
+      // dequant8() cut into four steps per dword d (unit d / 2, scale block d % 2)
+      h2 dp[NDW];
+      uint32_t dxh[NDW];
+      uint4 dout[NDW];
+      auto dq_step = [&](int idx) {
+        const int d = idx >> 2, ph = idx & 3;
+        const h2 b1 = {(_Float16)1032.0f, (_Float16)1032.0f};
+        const h2 b16 = {(_Float16)1152.0f, (_Float16)1152.0f};
+        if (ph == 0) {
+          const h2 p0 = __builtin_bit_cast(h2, and_or(dx[d], 0x000F000Fu, 0x64006400u));
+          dp[d] = __builtin_bit_cast(h2, and_or(dx[d], 0x00F000F0u, 0x64006400u));
+          dout[d].x = __builtin_bit_cast(uint32_t, (p0 - b1) * dsc[d]);
+        } else if (ph == 1) {
+          dout[d].y = __builtin_bit_cast(uint32_t, (dp[d] - b16) * dsc16[d]);
+          dxh[d] = dx[d] >> 8;
+        } else if (ph == 2) {
+          const h2 p2 = __builtin_bit_cast(h2, and_or(dxh[d], 0x000F000Fu, 0x64006400u));
+          dp[d] = __builtin_bit_cast(h2, and_or(dxh[d], 0x00F000F0u, 0x64006400u));
+          dout[d].z = __builtin_bit_cast(uint32_t, (p2 - b1) * dsc[d]);
+        } else {
+          dout[d].w = __builtin_bit_cast(uint32_t, (dp[d] - b16) * dsc16[d]);
+          *reinterpret_cast<uint4*>(frag_ptr((u + 1) & 1, d >> 1, d & 1)) = dout[d];
+        }
+      };
+      int mi = 0;
+#pragma unroll
+      for (int sl = 0; sl < SL; ++sl) {
 #pragma unroll
         for (int b = 0; b < WN; ++b) {
 #pragma unroll
@@ -325,37 +374,75 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_f16_kernel(
             acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
                 __builtin_bit_cast(h8, areg[u][sl >> 1][a][sl & 1]), bf[sl & 1][b], acc[a][b], 0, 0,
                 0);
+            if (sl < SL - 1 && a == 0)  // the next slice's fragment b, one read per product
+              bf[(sl + 1) & 1][b] =
+                  *reinterpret_cast<const h8*>(bbuf + ((sl + 1) * BN32 + wn * WN + b) * 1024);
+#pragma unroll
+            for (int st = mi * NSTEP / kMfma; st < (mi + 1) * NSTEP / kMfma; ++st) dq_step(st);
+            ++mi;
+            __builtin_amdgcn_sched_barrier(0);
           }
         }
+        if (sl & 1) load_a_kb(s + D, sl >> 1, areg[u]);  // that k-block's registers are free now
       }
-      load_a(s + D, areg[u]);
     }
   }
 
-  // C layout of a 32x32 tile: lane (h, i32) holds column i32; register v holds row
-  // 8*(v/4) + 4*h + v%4.
+  // Everything the output transform reads is loaded before the first store: loads and stores
+  // retire through one in-order counter, so a load issued after a store would wait for that store
+  // to reach memory.
+  float rc[WM][16], rm[WN], bs[WN];
+#pragma unroll
+  for (int a = 0; a < WM; ++a) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int m = m0 + 32 * a + 8 * (v >> 2) + 4 * h + (v & 3);
+      rc[a][v] = recip[m < M ? m : M - 1];
+    }
+  }
 #pragma unroll
   for (int b = 0; b < WN; ++b) {
     const int n = 16 * nt0 + 32 * (wn * WN + b) + i32;
-    if (n >= N) continue;
-    const float rm = rowmul[n], bs = bias[n];
+    rm[b] = rowmul[n < N ? n : N - 1];
+    bs[b] = bias[n < N ? n : N - 1];
+  }
+
+  __builtin_amdgcn_sched_barrier(0);
+
+  // C layout of a 32x32 tile: lane (h, i32) holds column i32; register v holds row
+  // 8*(v/4) + 4*h + v%4. Stores go through a buffer descriptor that covers exactly this
+  // workgroup's valid rows: the hardware drops a store whose offset lies past the descriptor's
+  // size, so rows >= M need no branch (columns >= N get an offset past the end instead).
+  // Straight-line stores matter: with a branch around each one the compiler cannot count
+  // outstanding stores and waits for all of them before every use of a loaded factor (that made
+  // the epilogue of a 128 x 128 tile take 9 us instead of 1.7).
+  const int wg_m0 = mb * BM;
+  const int rows_valid = (M - wg_m0 < BM ? M - wg_m0 : BM);
+  const __amdgpu_buffer_rsrc_t out_rows = __builtin_amdgcn_make_buffer_rsrc(
+      y + (size_t)wg_m0 * N, 0, (int)((unsigned)rows_valid * (unsigned)N * 4u), 0x00020000);
+  const unsigned row_bytes = (unsigned)N * 4u;
+#pragma unroll
+  for (int b = 0; b < WN; ++b) {
+    constexpr int kPastEnd = 0x7FFFFFF0;
+    const int n = 16 * nt0 + 32 * (wn * WN + b) + i32;
 #pragma unroll
     for (int a = 0; a < WM; ++a) {
+      const unsigned row0 = (unsigned)(32 * WM * wm + 32 * a + 4 * h);
+      const unsigned off0 = row0 * row_bytes + (unsigned)n * 4u;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int m = m0 + 32 * a + 8 * (v >> 2) + 4 * h + (v & 3);
-        if (m < M) {
-          float val = acc[a][b][v] * rm;
-          val = __fmaf_rn(val, recip[m], bs);
-          val = fminf(fmaxf(val, -3.402823466e+38f), 3.402823466e+38f);
-          y[(size_t)m * N + n] = val;
-        }
+        float val = acc[a][b][v] * rm[b];
+        val = __fmaf_rn(val, rc[a][v], bs[b]);
+        val = fminf(fmaxf(val, -3.402823466e+38f), 3.402823466e+38f);
+        const unsigned dm = 8 * (v >> 2) + (v & 3);  // row offset from row0
+        const int off = n < N ? (int)(off0 + dm * row_bytes) : kPastEnd;
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), out_rows, off, 0, 0);
       }
     }
   }
 }
 
-template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH>
+template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH, int OCC>
 static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                              hipStream_t s) {
   constexpr int BM = 32 * WM * WAVES_M, WNT = 2 * WN * WAVES_N;
@@ -366,7 +453,7 @@ static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed,
   // keep together what is more expensive to fetch eight times: the f16 activations (2 bytes per
   // element) or the packed weights (0.5625 bytes per element)
   const int n_major = (double)M * 2.0 <= (double)N * 0.5625 ? 1 : 0;
-  hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH>), dim3(grid),
+  hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC>), dim3(grid),
                      dim3(64 * WAVES_M * WAVES_N), 0, s, y,
                      reinterpret_cast<const _Float16*>(ws + w.ah_off),
                      reinterpret_cast<const float*>(ws + w.scale_off), packed,
@@ -391,22 +478,43 @@ static hipError_t launch_gemm_i8(float* y, const uint8_t* ws, const uint8_t* pac
   return hipGetLastError();
 }
 
-// Tile shape by how many 128 x 128 tiles the problem has (measured on MI355X at M = 128..2048 over
-// the decoder and ViT shapes). A stage of 64 k costs a workgroup about the same time whatever
-// its tile size as long as it is alone on its CU, so few-tile problems take smaller tiles: more
-// workgroups, several per CU, which overlap each other's stalls. With many tiles the larger tile's
-// operand reuse wins; from 1024 tiles on, 4 wavefronts per workgroup and three workgroups per CU
-// did best, below that 8 wavefronts per workgroup.
+// Tile shapes of the f16 kernel (kKernelGemmF16Tile + index names one; kKernelGemmF16 chooses).
+//   0:  64 x  64, 4 wavefronts of 32 x 32, 8 stages of loads in flight
+//   1: 128 x  64, 4 wavefronts of 32 x 64
+//   2: 128 x 128, 4 wavefronts of 32 x 128, three workgroups per CU
+//   3: 256 x 128, 4 wavefronts of 64 x 128 (each B fragment feeds two products)
+static hipError_t launch_f16_tile(int tile, float* y, const uint8_t* ws, const uint8_t* packed, int M,
+                                  int K, int N, hipStream_t s) {
+  switch (tile) {
+    case 0: return launch_f16<2, 2, 1, 1, 8, 2>(y, ws, packed, M, K, N, s);
+    case 1: return launch_f16<4, 1, 1, 2, 2, 4>(y, ws, packed, M, K, N, s);
+    case 2: return launch_f16<4, 1, 1, 4, 2, 3>(y, ws, packed, M, K, N, s);
+    case 3: return launch_f16<4, 1, 2, 4, 2, 1>(y, ws, packed, M, K, N, s);
+  }
+  return hipErrorInvalidValue;
+}
+
+// Choice of tile shape, measured on MI355X at M = 128..8192 over the decoder and ViT shapes, by
+// the number of 128 x 128 tiles the problem has. A stage of 64 k costs a lone workgroup about the
+// same time whatever its tile size (barrier, first LDS round trip, dequantisation), so problems
+// with fewer tiles than CUs take the smaller tile and put two workgroups on a CU; with very
+// few tiles and a long K the 64 x 64 tile's four-fold workgroup count wins. From about one tile per
+// CU on, 128 x 128 with three resident workgroups per CU is best; with many tiles per CU the
+// 256 x 128 tile, which reads each B fragment from LDS once for two products.
 hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                        int kernel, hipStream_t s) {
   if (kernel == kKernelGemmI8 || (kernel == kKernelAuto && M <= 32)) {
     return launch_gemm_i8(y, ws, packed, M, K, N, s);
   }
+  if (kernel >= kKernelGemmF16Tile && kernel < kKernelGemmF16Tile + kGemmF16Tiles) {
+    return launch_f16_tile(kernel - kKernelGemmF16Tile, y, ws, packed, M, K, N, s);
+  }
   const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-  if (tiles < 128) return launch_f16<2, 2, 1, 1, 8>(y, ws, packed, M, K, N, s);   //  64 x  64
-  if (tiles < 512) return launch_f16<4, 1, 1, 2, 2>(y, ws, packed, M, K, N, s);   // 128 x  64
-  if (tiles < 1024) return launch_f16<4, 2, 1, 2, 2>(y, ws, packed, M, K, N, s);  // 128 x 128, 8 wavefronts
-  return launch_f16<4, 1, 1, 4, 2>(y, ws, packed, M, K, N, s);                    // 128 x 128, 4 wavefronts
+  int tile = 3;
+  if (tiles < 64 && K >= 4096) tile = 0;
+  else if (tiles < 160) tile = 1;
+  else if (tiles < 2048) tile = 2;
+  return launch_f16_tile(tile, y, ws, packed, M, K, N, s);
 }
 
 }  // namespace w4

@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include "w4a32_hip.h"
 #include "w4a32_layout.h"
 
 namespace w4 {
@@ -72,6 +73,8 @@ constexpr int kKernelAuto = 0;
 constexpr int kKernelGemv = 1;
 constexpr int kKernelGemmI8 = 2;
 constexpr int kKernelGemmF16 = 3;
+constexpr int kKernelGemmF16Tile = W4A32_KERNEL_GEMM_F16_TILE0;  // + index: that tile shape
+constexpr int kGemmF16Tiles = W4A32_GEMM_F16_TILES;
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
 

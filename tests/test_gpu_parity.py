@@ -272,18 +272,24 @@ def test_gemm_ragged_m(pkg, orc, m):
     assert max_abs_rel(y, ref) <= TIGHT
 
 
-@pytest.mark.parametrize("kernel", ["i8", "f16"])
+@pytest.mark.parametrize("kernel", ["i8", "f16", "f16:0", "f16:1", "f16:2", "f16:3"])
 @pytest.mark.parametrize("m,k,n", [(9, 32, 16), (40, 96, 50), (128, 1536, 256), (300, 1280, 3840),
                                    (512, 8960, 1536), (1024, 5120, 1280)])
 def test_gemm_each_kernel_matches_oracle(pkg, orc, kernel, m, k, n):
-    # both prefill kernels on the same inputs; K = 32 and 96 leave padding inside a stage
+    # both prefill kernels (and each tile shape of the f16 one) on the same inputs; K = 32 and 96
+    # leave padding inside a stage
     w = make_weights(n, k, seed=k)
     x = make_acts(m, k, seed=m, outlier_frac=0.02)
     bias = bias_for(n, True)
     u4, sc = orc.quant_rhs(w)
     packed = pkg.repack_native(dev(u4), dev(sc.view(np.int16)), dev(bias), n, k)
     ws = pkg.quant_lhs(dev(x))
-    sel = pkg.KERNEL_GEMM_I8 if kernel == "i8" else pkg.KERNEL_GEMM_F16
+    if kernel == "i8":
+        sel = pkg.KERNEL_GEMM_I8
+    elif kernel == "f16":
+        sel = pkg.KERNEL_GEMM_F16
+    else:  # every tile shape of the f16 kernel, whatever the size-based choice would be
+        sel = pkg.KERNEL_GEMM_F16_TILE0 + int(kernel.split(":")[1])
     y = host(pkg.matmul_quantized(ws, packed, m, k, n, kernel=sel))
     rows = np.unique(np.concatenate([np.arange(0, m, 41), [m - 1]]))
     ref = orc.linear(x[rows], u4, sc, bias=bias, threads=8)
