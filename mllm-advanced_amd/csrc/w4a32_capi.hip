@@ -190,8 +190,14 @@ int w4a32_matmul_grouped(float* const* d_y, const float* d_x, const void* const*
     for (int i = 0; i < count; ++i) pk[i] = static_cast<const uint8_t*>(d_packed[i]);
     return from_hip(w4::launch_gemv_group(d_y, d_x, K, pk, N, count, M, K, s));
   }
-  // other sizes: quantise the rows once, then one product per Linear
+  // other sizes: quantise the rows once, then one launch of the f16 kernel over all the Linears
+  // (M > 32) or one product per Linear
   if (int e = w4a32_quant_lhs(d_x, M, K, K, d_ws, stream)) return e;
+  if (M > 32) {
+    const uint8_t* pk[W4A32_MAX_GROUP];
+    for (int i = 0; i < count; ++i) pk[i] = static_cast<const uint8_t*>(d_packed[i]);
+    return from_hip(w4::launch_gemm_group(d_y, static_cast<const uint8_t*>(d_ws), pk, N, count, M, K, s));
+  }
   for (int i = 0; i < count; ++i) {
     if (int e = w4a32_matmul_quantized(d_y[i], d_ws, d_packed[i], M, K, N[i], stream)) return e;
   }

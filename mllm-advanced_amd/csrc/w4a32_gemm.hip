@@ -157,12 +157,24 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 //    read once per WM products, so WM = 1 costs 160 bytes per clock at the full product rate
 //    (reads + the tile's own writes): LDS-bound. WM = 2 needs 80. A is read once per WN products
 //    through the vector L1 (64 bytes per clock and CU): WN = 4 needs 32.
-template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH, int OCC>
+//
+// GROUPED: up to kMaxGemmGroup Linears on the same activation rows in one launch. Their column
+// blocks are numbered through (Linear i owns blocks nb_first[i] .. nb_first[i+1]-1); a workgroup
+// looks its Linear up and takes N, the blob and the output from the table.
+constexpr int kMaxGemmGroup = W4A32_MAX_GROUP;
+struct GemmGroup {
+  float* y[kMaxGemmGroup];
+  const uint8_t* packed[kMaxGemmGroup];
+  int N[kMaxGemmGroup];
+  int nb_first[kMaxGemmGroup + 1];  // entries past the last Linear hold the total
+};
+
+template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH, int OCC, bool GROUPED>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
-    float* __restrict__ y, const _Float16* __restrict__ ah, const float* __restrict__ recip,
-    const uint8_t* __restrict__ packed, const uint8_t* __restrict__ hscale,
-    const float* __restrict__ rowmul, const float* __restrict__ bias, int M, int N, int K, int NT,
-    int KC, int MB, int NB, int n_major) {
+    float* __restrict__ y_arg, const _Float16* __restrict__ ah, const float* __restrict__ recip,
+    const uint8_t* __restrict__ packed_arg, const uint8_t* __restrict__ hscale_arg,
+    const float* __restrict__ rowmul_arg, const float* __restrict__ bias_arg, int M, int N_arg, int K,
+    int NT_arg, int KC, int MB, int NB, int n_major, const GemmGroup grp) {
   constexpr int D = DEPTH;
   static_assert(D % 2 == 0, "stage s uses LDS buffer s & 1: the unrolled ring must keep that parity");
   constexpr int NWAVES = WAVES_M * WAVES_N;
@@ -197,7 +209,27 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
   const int tile = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
   if (tile >= total) return;  // whole workgroup: no barrier has been reached yet
   const int mb = n_major ? tile % MB : tile / NB;
-  const int nb = n_major ? tile / MB : tile % NB;
+  int nb = n_major ? tile / MB : tile % NB;
+  float* y = y_arg;
+  const uint8_t* packed = packed_arg;
+  const uint8_t* hscale = hscale_arg;
+  const float* rowmul = rowmul_arg;
+  const float* bias = bias_arg;
+  int N = N_arg, NT = NT_arg;
+  if constexpr (GROUPED) {
+    int gi = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxGemmGroup; ++i) gi = nb >= grp.nb_first[i] ? i : gi;
+    nb -= grp.nb_first[gi];
+    N = grp.N[gi];
+    const WeightGeom wgm = weight_geom(N, K);
+    NT = wgm.NT;
+    y = grp.y[gi];
+    packed = grp.packed[gi];
+    hscale = packed + wgm.hscale_off;
+    rowmul = reinterpret_cast<const float*>(packed + wgm.rowmul_off);
+    bias = reinterpret_cast<const float*>(packed + wgm.bias_off);
+  }
   const int m0 = mb * BM + 32 * WM * wm;
   const int nt0 = nb * WNT;
   const int nstages = (K + kF16BK - 1) / kF16BK;
@@ -251,8 +283,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
     const int offs = kc * kTileScaleBytes + 4 * half;
 #pragma unroll
     for (int u = 0; u < B_UNITS; ++u) {
-      q[u] = *reinterpret_cast<const uint2*>(bq_ptr[u] + offq);
-      sc[u] = *reinterpret_cast<const uint32_t*>(bs_ptr[u] + offs);
+      const u32x2 t2 = load_global<u32x2>(bq_ptr[u] + offq);  // (a table pointer is a generic one)
+      q[u] = make_uint2(t2.x, t2.y);
+      sc[u] = load_global<uint32_t>(bs_ptr[u] + offs);
     }
   };
 
@@ -403,8 +436,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
 #pragma unroll
   for (int b = 0; b < WN; ++b) {
     const int n = 16 * nt0 + 32 * (wn * WN + b) + i32;
-    rm[b] = rowmul[n < N ? n : N - 1];
-    bs[b] = bias[n < N ? n : N - 1];
+    rm[b] = load_global<float>(rowmul + (n < N ? n : N - 1));
+    bs[b] = load_global<float>(bias + (n < N ? n : N - 1));
   }
 
   __builtin_amdgcn_sched_barrier(0);
@@ -442,24 +475,45 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
   }
 }
 
+// One Linear (group == nullptr) or the Linears of `group`, whose column blocks add up to nb_total.
 template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH, int OCC>
 static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
-                             hipStream_t s) {
+                             const GemmGroup* group, const int* group_N, int count, hipStream_t s) {
   constexpr int BM = 32 * WM * WAVES_M, WNT = 2 * WN * WAVES_N;
-  const WeightGeom g = weight_geom(N, K);
   const WsGeom w = ws_geom(M, K);
-  const int NB = (g.NT + WNT - 1) / WNT, MB = (M + BM - 1) / BM;
+  const int MB = (M + BM - 1) / BM;
+  const _Float16* ah = reinterpret_cast<const _Float16*>(ws + w.ah_off);
+  const float* recip = reinterpret_cast<const float*>(ws + w.scale_off);
+  if (group) {
+    GemmGroup g = *group;
+    int nb = 0;
+    long n_total = 0;
+    for (int i = 0; i <= kMaxGemmGroup; ++i) {
+      g.nb_first[i] = nb;
+      if (i < count) {
+        nb += (weight_geom(group_N[i], K).NT + WNT - 1) / WNT;
+        n_total += group_N[i];
+      }
+    }
+    const int NB = nb;
+    const int n_major = (double)M * 2.0 <= (double)n_total * 0.5625 ? 1 : 0;
+    hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, true>),
+                       dim3(((MB * NB + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N), 0, s, nullptr, ah,
+                       recip, nullptr, nullptr, nullptr, nullptr, M, 0, K, 0,
+                       weight_geom(group_N[0], K).KC, MB, NB, n_major, g);
+    return hipGetLastError();
+  }
+  const WeightGeom g = weight_geom(N, K);
+  const int NB = (g.NT + WNT - 1) / WNT;
   const int grid = ((MB * NB + 7) / 8) * 8;
   // keep together what is more expensive to fetch eight times: the f16 activations (2 bytes per
   // element) or the packed weights (0.5625 bytes per element)
   const int n_major = (double)M * 2.0 <= (double)N * 0.5625 ? 1 : 0;
-  hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC>), dim3(grid),
-                     dim3(64 * WAVES_M * WAVES_N), 0, s, y,
-                     reinterpret_cast<const _Float16*>(ws + w.ah_off),
-                     reinterpret_cast<const float*>(ws + w.scale_off), packed,
-                     packed + g.hscale_off, reinterpret_cast<const float*>(packed + g.rowmul_off),
+  hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, false>), dim3(grid),
+                     dim3(64 * WAVES_M * WAVES_N), 0, s, y, ah, recip, packed, packed + g.hscale_off,
+                     reinterpret_cast<const float*>(packed + g.rowmul_off),
                      reinterpret_cast<const float*>(packed + g.bias_off), M, N, K, g.NT, g.KC, MB, NB,
-                     n_major);
+                     n_major, GemmGroup{});
   return hipGetLastError();
 }
 
@@ -484,14 +538,22 @@ static hipError_t launch_gemm_i8(float* y, const uint8_t* ws, const uint8_t* pac
 //   2: 128 x 128, 4 wavefronts of 32 x 128, three workgroups per CU
 //   3: 256 x 128, 4 wavefronts of 64 x 128 (each B fragment feeds two products)
 static hipError_t launch_f16_tile(int tile, float* y, const uint8_t* ws, const uint8_t* packed, int M,
-                                  int K, int N, hipStream_t s) {
+                                  int K, int N, const GemmGroup* group, const int* group_N, int count,
+                                  hipStream_t s) {
   switch (tile) {
-    case 0: return launch_f16<2, 2, 1, 1, 8, 2>(y, ws, packed, M, K, N, s);
-    case 1: return launch_f16<4, 1, 1, 2, 2, 4>(y, ws, packed, M, K, N, s);
-    case 2: return launch_f16<4, 1, 1, 4, 2, 3>(y, ws, packed, M, K, N, s);
-    case 3: return launch_f16<4, 1, 2, 4, 2, 1>(y, ws, packed, M, K, N, s);
+    case 0: return launch_f16<2, 2, 1, 1, 8, 2>(y, ws, packed, M, K, N, group, group_N, count, s);
+    case 1: return launch_f16<4, 1, 1, 2, 2, 4>(y, ws, packed, M, K, N, group, group_N, count, s);
+    case 2: return launch_f16<4, 1, 1, 4, 2, 3>(y, ws, packed, M, K, N, group, group_N, count, s);
+    case 3: return launch_f16<4, 1, 2, 4, 2, 1>(y, ws, packed, M, K, N, group, group_N, count, s);
   }
   return hipErrorInvalidValue;
+}
+
+static int choose_f16_tile(long tiles, int K) {
+  if (tiles < 64 && K >= 4096) return 0;
+  if (tiles < 160) return 1;
+  if (tiles < 2048) return 2;
+  return 3;
 }
 
 // Choice of tile shape, measured on MI355X at M = 128..8192 over the decoder and ViT shapes, by
@@ -507,14 +569,23 @@ hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M
     return launch_gemm_i8(y, ws, packed, M, K, N, s);
   }
   if (kernel >= kKernelGemmF16Tile && kernel < kKernelGemmF16Tile + kGemmF16Tiles) {
-    return launch_f16_tile(kernel - kKernelGemmF16Tile, y, ws, packed, M, K, N, s);
+    return launch_f16_tile(kernel - kKernelGemmF16Tile, y, ws, packed, M, K, N, nullptr, nullptr, 0, s);
   }
   const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-  int tile = 3;
-  if (tiles < 64 && K >= 4096) tile = 0;
-  else if (tiles < 160) tile = 1;
-  else if (tiles < 2048) tile = 2;
-  return launch_f16_tile(tile, y, ws, packed, M, K, N, s);
+  return launch_f16_tile(choose_f16_tile(tiles, K), y, ws, packed, M, K, N, nullptr, nullptr, 0, s);
+}
+
+hipError_t launch_gemm_group(float* const* y, const uint8_t* ws, const uint8_t* const* packed,
+                             const int* N, int count, int M, int K, hipStream_t s) {
+  GemmGroup g{};
+  long tiles = 0;
+  for (int i = 0; i < count; ++i) {
+    g.y[i] = y[i];
+    g.packed[i] = packed[i];
+    g.N[i] = N[i];
+    tiles += (long)((M + 127) / 128) * ((N[i] + 127) / 128);
+  }
+  return launch_f16_tile(choose_f16_tile(tiles, K), nullptr, ws, nullptr, M, K, 0, &g, N, count, s);
 }
 
 }  // namespace w4

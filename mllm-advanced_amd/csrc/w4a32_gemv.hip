@@ -189,17 +189,6 @@ __global__ __launch_bounds__(1024) void gemv_q_kernel(
   gemv_finish<M>(y, N, nt, W, acc, s_red, recip_m, negzp_m, rsum, bias, rs, bs);
 }
 
-// Loads and stores through pointers picked from the group table must say that they address global
-// memory: the compiler no longer knows, would emit flat instructions and, because those may
-// complete out of order with global ones, wait for every outstanding load at the first use of any.
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-#define W4_GLOBAL __attribute__((address_space(1)))
-template <typename T>
-__device__ __forceinline__ T load_global(const void* p) {
-  return *(const W4_GLOBAL T*)p;
-}
-
 // Up to kMaxGroup Linears that share their activation rows (and therefore K), run by one launch:
 // workgroup b serves tile row b - first[i] of Linear i, where first[] are running sums of tile rows.
 constexpr int kMaxGroup = 4;

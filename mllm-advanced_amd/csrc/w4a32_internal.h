@@ -40,6 +40,9 @@ hipError_t launch_gemv_decode(float* const* y, const float* x, const uint8_t* co
                               const float* norm_w, float eps, bool pair, hipStream_t s);
 hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                        int kernel, hipStream_t s);
+// several Linears on the same quantised rows in one launch of the f16 kernel (M > 32)
+hipError_t launch_gemm_group(float* const* y, const uint8_t* ws, const uint8_t* const* packed,
+                             const int* N, int count, int M, int K, hipStream_t s);
 
 // decoder operators (f32), w4a32_glue.hip
 hipError_t launch_embedding(const int64_t* ids, const float* table, int M, int D, int vocab,
@@ -77,5 +80,17 @@ constexpr int kKernelGemmF16Tile = W4A32_KERNEL_GEMM_F16_TILE0;  // + index: tha
 constexpr int kGemmF16Tiles = W4A32_GEMM_F16_TILES;
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+
+// Loads and stores through pointers picked from the group table must say that they address global
+// memory: the compiler no longer knows, would emit flat instructions and, because those may
+// complete out of order with global ones, wait for every outstanding load at the first use of any.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+#define W4_GLOBAL __attribute__((address_space(1)))
+template <typename T>
+__device__ __forceinline__ T load_global(const void* p) {
+  return *(const W4_GLOBAL T*)p;
+}
+
 
 }  // namespace w4

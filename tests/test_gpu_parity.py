@@ -195,10 +195,13 @@ def test_fused_decode_kernel_equals_two_step_path(pkg, orc, m, k, n):
 @pytest.mark.parametrize("m,k,ns", [(1, 1536, [1536, 256, 256]), (8, 1536, [1536, 256, 256]),
                                     (1, 1536, [8960, 8960]), (4, 1536, [8960, 8960]),
                                     (1, 8960, [1536]), (4, 8960, [1536, 50]), (12, 256, [64, 48, 16, 100]),
-                                    (2, 64, [40, 16])])
+                                    (2, 64, [40, 16]), (40, 256, [64, 48, 16, 100]),
+                                    (130, 96, [50, 16]), (300, 1536, [1536, 256, 256]),
+                                    (512, 1536, [8960, 8960]), (1024, 1280, [1280, 1280, 1280])])
 def test_grouped_linears_equal_separate_calls(pkg, m, k, ns):
     # q/k/v and gate/up take the same rows: one grouped call must give, bit for bit, what one
-    # w4a32_matmul per Linear gives (covers the one-launch path and the quantise-once fallback)
+    # w4a32_matmul per Linear gives (covers the one-launch decode path, the quantise-once fallback
+    # and, from M = 33 on, the prefill kernel's one launch over all the Linears)
     x = dev(make_acts(m, k, seed=7, outlier_frac=0.25))
     packed = [pkg.quant_pack_rhs(dev(make_weights(n, k, seed=10 + i)), dev(bias_for(n, True, seed=i)))
               for i, n in enumerate(ns)]
