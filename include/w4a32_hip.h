@@ -123,6 +123,16 @@ int w4a32_matmul_quantized(float* d_y, const void* d_ws, const void* d_packed, i
 int w4a32_matmul_quantized_ex(float* d_y, const void* d_ws, const void* d_packed, int M, int K,
                               int N, int kernel, void* stream);
 
+/* The same product for callers that can lend scratch memory: when the problem has few output
+ * tiles and a long K (down_proj at prefill sizes) each tile's k range is dealt to several
+ * workgroups, which leave partial sums in d_scratch; a second kernel adds them in a fixed order.
+ * w4a32_splitk_scratch_bytes() returns the bytes this needs, 0 when the library would not split the
+ * shape; with less scratch than that the call is w4a32_matmul_quantized(). The reference has no
+ * counterpart: its matmul splits M over threads only (kai_linear.cpp:366-396). */
+size_t w4a32_splitk_scratch_bytes(int M, int K, int N);
+int w4a32_matmul_quantized_splitk(float* d_y, const void* d_ws, const void* d_packed, int M, int K,
+                                  int N, void* d_scratch, size_t scratch_bytes, void* stream);
+
 /* The whole op = ...::matmul (kai_linear.cpp:350-398): quantise rows of d_x into d_ws,
  * then multiply. d_ws must hold w4a32_workspace_bytes(M, K). */
 int w4a32_matmul(float* d_y, const float* d_x, const void* d_packed, void* d_ws, int M, int K,

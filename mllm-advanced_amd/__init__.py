@@ -39,6 +39,8 @@ ABI = {
     "w4a32_export_lhs": (_ci, [_vp, _ci, _ci, _vp, _vp, _vp, _vp]),
     "w4a32_matmul_quantized": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a32_matmul_quantized_ex": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp]),
+    "w4a32_splitk_scratch_bytes": (_sz, [_ci, _ci, _ci]),
+    "w4a32_matmul_quantized_splitk": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a32_matmul": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a32_matmul_grouped": (_ci, [_vp, _vp, _vp, _vp, _ci, _vp, _ci, _ci, _vp]),
     # include/w4a32_decoder.h
@@ -226,6 +228,21 @@ def matmul_quantized(ws, packed, M, K, N, out=None, kernel=KERNEL_AUTO):
     y = out if out is not None else torch.empty((M, N), dtype=torch.float32, device="cuda")
     _check(lib().w4a32_matmul_quantized_ex(_ptr(y), _ptr(ws), _ptr(packed), M, K, N, kernel,
                                            _stream()), "w4a32_matmul_quantized_ex")
+    return y
+
+
+def matmul_quantized_splitk(ws, packed, M, K, N, scratch=None, out=None):
+    """matmul_quantized() with scratch memory lent for partial sums (allocated here when absent)."""
+    import torch
+
+    y = out if out is not None else torch.empty((M, N), dtype=torch.float32, device="cuda")
+    need = int(lib().w4a32_splitk_scratch_bytes(M, K, N))
+    if scratch is None and need:
+        scratch = _dev_empty(need)
+    _check(lib().w4a32_matmul_quantized_splitk(_ptr(y), _ptr(ws), _ptr(packed), M, K, N,
+                                               _ptr(scratch) if scratch is not None else None,
+                                               scratch.numel() * scratch.element_size() if scratch is not None else 0,
+                                               _stream()), "w4a32_matmul_quantized_splitk")
     return y
 
 

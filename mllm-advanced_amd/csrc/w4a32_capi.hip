@@ -155,6 +155,27 @@ int w4a32_matmul_quantized_ex(float* d_y, const void* d_ws, const void* d_packed
   }
 }
 
+size_t w4a32_splitk_scratch_bytes(int M, int K, int N) {
+  if (M <= 32 || shape_ok(N, K)) return 0;
+  const w4::SplitPlan p = w4::splitk_plan(M, K, N);
+  return p.parts > 1 ? (size_t)p.parts * M * N * sizeof(float) : 0;
+}
+
+int w4a32_matmul_quantized_splitk(float* d_y, const void* d_ws, const void* d_packed, int M, int K,
+                                  int N, void* d_scratch, size_t scratch_bytes, void* stream) {
+  const size_t need = w4a32_splitk_scratch_bytes(M, K, N);
+  if (need == 0 || !d_scratch || scratch_bytes < need) {
+    return w4a32_matmul_quantized(d_y, d_ws, d_packed, M, K, N, stream);
+  }
+  if (!d_y || !d_ws || !d_packed) return W4A32_EINVAL;
+  if (!aligned(d_ws, 256) || !aligned(d_packed, 16) || !aligned(d_y, 16) || !aligned(d_scratch, 16)) {
+    return W4A32_EINVAL;
+  }
+  return from_hip(w4::launch_gemm_splitk(d_y, static_cast<const uint8_t*>(d_ws),
+                                         static_cast<const uint8_t*>(d_packed), M, K, N,
+                                         static_cast<float*>(d_scratch), static_cast<hipStream_t>(stream)));
+}
+
 int w4a32_matmul_quantized(float* d_y, const void* d_ws, const void* d_packed, int M, int K, int N,
                            void* stream) {
   return w4a32_matmul_quantized_ex(d_y, d_ws, d_packed, M, K, N, W4A32_KERNEL_AUTO, stream);

@@ -156,7 +156,15 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
       W4_TRY(w4a32_matmul_grouped(ys, xn, ps, ns, 2, ws, M, H, stream));
     }
     W4_TRY(from_hip(w4::launch_silu_mul(gate, up, act, (size_t)M * I, s)));
-    W4_TRY(w4a32_matmul(delta, act, lw.down, ws, M, I, H, stream));
+    if (M > 32) {
+      // few output tiles, long K: split-K, with the partial sums in the gate and up buffers,
+      // which are dead once `act` holds silu(gate) * up
+      W4_TRY(w4a32_quant_lhs(act, M, I, I, ws, stream));
+      const size_t lend = g.up_off - g.gate_off + sizeof(float) * (size_t)c->max_batch_tokens * I;
+      W4_TRY(w4a32_matmul_quantized_splitk(delta, ws, lw.down, M, I, H, gate, lend, stream));
+    } else {
+      W4_TRY(w4a32_matmul(delta, act, lw.down, ws, M, I, H, stream));
+    }
   }
   // Only the last row feeds the head: h_last += delta_last; xn_last = norm(h_last)
   const size_t last = (size_t)(M - 1) * H;

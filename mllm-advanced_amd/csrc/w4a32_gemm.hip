@@ -161,6 +161,12 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 // GROUPED: up to kMaxGemmGroup Linears on the same activation rows in one launch. Their column
 // blocks are numbered through (Linear i owns blocks nb_first[i] .. nb_first[i+1]-1); a workgroup
 // looks its Linear up and takes N, the blob and the output from the table.
+//
+// SPLITK: `ksplit` workgroups share a tile, each takes a contiguous range of the stages and stores
+// its raw f32 sums to part[ks][M][N]; splitk_reduce_kernel adds the parts in a fixed order and
+// applies the output transform. For problems with few tiles and a long K (down_proj at M <= 512:
+// 48 tiles of 128 x 128 for 256 CUs, 140 stages each).
+constexpr int kModePlain = 0, kModeGrouped = 1, kModeSplitK = 2;
 constexpr int kMaxGemmGroup = W4A32_MAX_GROUP;
 struct GemmGroup {
   float* y[kMaxGemmGroup];
@@ -169,12 +175,14 @@ struct GemmGroup {
   int nb_first[kMaxGemmGroup + 1];  // entries past the last Linear hold the total
 };
 
-template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH, int OCC, bool GROUPED>
+template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH, int OCC, int MODE>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
     float* __restrict__ y_arg, const _Float16* __restrict__ ah, const float* __restrict__ recip,
     const uint8_t* __restrict__ packed_arg, const uint8_t* __restrict__ hscale_arg,
     const float* __restrict__ rowmul_arg, const float* __restrict__ bias_arg, int M, int N_arg, int K,
-    int NT_arg, int KC, int MB, int NB, int n_major, const GemmGroup grp) {
+    int NT_arg, int KC, int MB, int NB, int n_major, int ksplit, float* __restrict__ part,
+    const GemmGroup grp) {
+  constexpr bool GROUPED = MODE == kModeGrouped, SPLITK = MODE == kModeSplitK;
   constexpr int D = DEPTH;
   static_assert(D % 2 == 0, "stage s uses LDS buffer s & 1: the unrolled ring must keep that parity");
   constexpr int NWAVES = WAVES_M * WAVES_N;
@@ -204,10 +212,15 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
   // XCD owns one contiguous run of tiles; the run is ordered so that neighbours share the larger
   // operand (n_major: all row blocks of a weight column block together, weights fetched by one
   // XCD only; otherwise all column blocks of a row block together).
-  const int total = MB * NB;
+  const int total = MB * NB * (SPLITK ? ksplit : 1);
   const int per_xcd = (total + 7) >> 3;
-  const int tile = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+  int tile = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
   if (tile >= total) return;  // whole workgroup: no barrier has been reached yet
+  int ks = 0;
+  if constexpr (SPLITK) {
+    ks = tile % ksplit;
+    tile /= ksplit;
+  }
   const int mb = n_major ? tile % MB : tile / NB;
   int nb = n_major ? tile / MB : tile % NB;
   float* y = y_arg;
@@ -232,7 +245,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
   }
   const int m0 = mb * BM + 32 * WM * wm;
   const int nt0 = nb * WNT;
-  const int nstages = (K + kF16BK - 1) / kF16BK;
+  // this workgroup's stages: [s_begin, nstages)
+  int s_begin = 0, nstages = (K + kF16BK - 1) / kF16BK;
+  if constexpr (SPLITK) {
+    s_begin = (int)((long)ks * nstages / ksplit);
+    nstages = (int)((long)(ks + 1) * nstages / ksplit);
+  }
 
   uint4 areg[D][AKB][WM][2];  // [ring slot][k-block][32-row tile][slice of the block]
   uint2 breg[D][B_UNITS];
@@ -305,7 +323,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
 
-  // Prologue: A stages 0..D-1 and B stages 0..D in flight; B stage 0 goes to LDS buffer 0. The
+  // Prologue: the first D stages of A and D+1 of B in flight; the first B stage goes to LDS buffer 0. The
   // loads are issued in the loop's own order (per stage: B, then A): the compiler derives each
   // wait in the loop from the fewest loads that can be younger than the one it needs on any way
   // into the loop, so a prologue with another order makes the loop wait for newer loads than it
@@ -313,12 +331,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
   {
     uint2 q0[B_UNITS];
     uint32_t s0[B_UNITS];
-    load_b(0, q0, s0);
+    load_b(s_begin, q0, s0);
 #pragma unroll
     for (int p = 0; p < D; ++p) {
-      load_b(p + 1, breg[p], sreg[p]);  // ring slot p holds stage p+1
+      load_b(s_begin + p + 1, breg[p], sreg[p]);  // ring slot p holds the stage after slot p's A
 #pragma unroll
-      for (int kbl = 0; kbl < AKB; ++kbl) load_a_kb(p, kbl, areg[p]);
+      for (int kbl = 0; kbl < AKB; ++kbl) load_a_kb(s_begin + p, kbl, areg[p]);
     }
     __builtin_amdgcn_sched_barrier(0);
     const h2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
@@ -341,7 +359,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
   // wavefront dequantises the next stage's weights, a few instructions at a time, and issues its
   // LDS and global traffic in the gaps between its own products. (Left to the scheduler, all of a
   // stage's dequantisation ran first and the products after it.)
-  for (int s_base = 0; s_base < nstages; s_base += D) {
+  for (int s_base = s_begin; s_base < nstages; s_base += D) {
 #pragma unroll
     for (int u = 0; u < D; ++u) {
       const int s = s_base + u;
@@ -451,8 +469,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
   // the epilogue of a 128 x 128 tile take 9 us instead of 1.7).
   const int wg_m0 = mb * BM;
   const int rows_valid = (M - wg_m0 < BM ? M - wg_m0 : BM);
+  float* out_base = SPLITK ? part + ((size_t)ks * M + wg_m0) * N : y + (size_t)wg_m0 * N;
   const __amdgpu_buffer_rsrc_t out_rows = __builtin_amdgcn_make_buffer_rsrc(
-      y + (size_t)wg_m0 * N, 0, (int)((unsigned)rows_valid * (unsigned)N * 4u), 0x00020000);
+      out_base, 0, (int)((unsigned)rows_valid * (unsigned)N * 4u), 0x00020000);
   const unsigned row_bytes = (unsigned)N * 4u;
 #pragma unroll
   for (int b = 0; b < WN; ++b) {
@@ -464,9 +483,11 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
       const unsigned off0 = row0 * row_bytes + (unsigned)n * 4u;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        float val = acc[a][b][v] * rm[b];
-        val = __fmaf_rn(val, rc[a][v], bs[b]);
-        val = fminf(fmaxf(val, -3.402823466e+38f), 3.402823466e+38f);
+        float val = acc[a][b][v];
+        if constexpr (!SPLITK) {
+          val = __fmaf_rn(val * rm[b], rc[a][v], bs[b]);
+          val = fminf(fmaxf(val, -3.402823466e+38f), 3.402823466e+38f);
+        }
         const unsigned dm = 8 * (v >> 2) + (v & 3);  // row offset from row0
         const int off = n < N ? (int)(off0 + dm * row_bytes) : kPastEnd;
         __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), out_rows, off, 0, 0);
@@ -475,10 +496,46 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
   }
 }
 
+// y[m][n] = transform(part[0][m][n] + part[1][m][n] + ...), four columns per thread when N allows.
+template <int VEC>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(
+    float* __restrict__ y, const float* __restrict__ part, int ksplit, int M, int N,
+    const float* __restrict__ recip, const float* __restrict__ rowmul, const float* __restrict__ bias) {
+  const size_t total = (size_t)M * N;
+  const size_t e = ((size_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+  if (e >= total) return;
+  const int m = (int)(e / N), n = (int)(e % N);
+  float sum[VEC];
+  if constexpr (VEC == 4) {
+    const float4 p = *reinterpret_cast<const float4*>(part + e);
+    sum[0] = p.x; sum[1] = p.y; sum[2] = p.z; sum[3] = p.w;
+    for (int k = 1; k < ksplit; ++k) {
+      const float4 q = *reinterpret_cast<const float4*>(part + (size_t)k * total + e);
+      sum[0] += q.x; sum[1] += q.y; sum[2] += q.z; sum[3] += q.w;
+    }
+  } else {
+    sum[0] = part[e];
+    for (int k = 1; k < ksplit; ++k) sum[0] += part[(size_t)k * total + e];
+  }
+  const float rc = recip[m];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    float val = __fmaf_rn(sum[i] * rowmul[n + i], rc, bias[n + i]);
+    sum[i] = fminf(fmaxf(val, -3.402823466e+38f), 3.402823466e+38f);
+  }
+  if constexpr (VEC == 4) {
+    *reinterpret_cast<float4*>(y + e) = make_float4(sum[0], sum[1], sum[2], sum[3]);
+  } else {
+    y[e] = sum[0];
+  }
+}
+
 // One Linear (group == nullptr) or the Linears of `group`, whose column blocks add up to nb_total.
+// ksplit > 1: the stages of every tile are dealt to ksplit workgroups (partial sums in `part`).
 template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH, int OCC>
 static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
-                             const GemmGroup* group, const int* group_N, int count, hipStream_t s) {
+                             const GemmGroup* group, const int* group_N, int count, int ksplit,
+                             float* part, hipStream_t s) {
   constexpr int BM = 32 * WM * WAVES_M, WNT = 2 * WN * WAVES_N;
   const WsGeom w = ws_geom(M, K);
   const int MB = (M + BM - 1) / BM;
@@ -497,23 +554,39 @@ static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed,
     }
     const int NB = nb;
     const int n_major = (double)M * 2.0 <= (double)n_total * 0.5625 ? 1 : 0;
-    hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, true>),
+    hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModeGrouped>),
                        dim3(((MB * NB + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N), 0, s, nullptr, ah,
                        recip, nullptr, nullptr, nullptr, nullptr, M, 0, K, 0,
-                       weight_geom(group_N[0], K).KC, MB, NB, n_major, g);
+                       weight_geom(group_N[0], K).KC, MB, NB, n_major, 1, nullptr, g);
     return hipGetLastError();
   }
   const WeightGeom g = weight_geom(N, K);
   const int NB = (g.NT + WNT - 1) / WNT;
-  const int grid = ((MB * NB + 7) / 8) * 8;
   // keep together what is more expensive to fetch eight times: the f16 activations (2 bytes per
   // element) or the packed weights (0.5625 bytes per element)
   const int n_major = (double)M * 2.0 <= (double)N * 0.5625 ? 1 : 0;
-  hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, false>), dim3(grid),
-                     dim3(64 * WAVES_M * WAVES_N), 0, s, y, ah, recip, packed, packed + g.hscale_off,
-                     reinterpret_cast<const float*>(packed + g.rowmul_off),
-                     reinterpret_cast<const float*>(packed + g.bias_off), M, N, K, g.NT, g.KC, MB, NB,
-                     n_major, GemmGroup{});
+  const float* rowmul = reinterpret_cast<const float*>(packed + g.rowmul_off);
+  const float* bias = reinterpret_cast<const float*>(packed + g.bias_off);
+  if (ksplit > 1) {
+    hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModeSplitK>),
+                       dim3(((MB * NB * ksplit + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N), 0, s, y, ah,
+                       recip, packed, packed + g.hscale_off, rowmul, bias, M, N, K, g.NT, g.KC, MB, NB,
+                       n_major, ksplit, part, GemmGroup{});
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+    const size_t total = (size_t)M * N;
+    if (N % 4 == 0) {
+      hipLaunchKernelGGL(splitk_reduce_kernel<4>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256),
+                         0, s, y, part, ksplit, M, N, recip, rowmul, bias);
+    } else {
+      hipLaunchKernelGGL(splitk_reduce_kernel<1>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                         s, y, part, ksplit, M, N, recip, rowmul, bias);
+    }
+    return hipGetLastError();
+  }
+  hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModePlain>),
+                     dim3(((MB * NB + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N), 0, s, y, ah, recip,
+                     packed, packed + g.hscale_off, rowmul, bias, M, N, K, g.NT, g.KC, MB, NB, n_major,
+                     1, nullptr, GemmGroup{});
   return hipGetLastError();
 }
 
@@ -539,12 +612,16 @@ static hipError_t launch_gemm_i8(float* y, const uint8_t* ws, const uint8_t* pac
 //   3: 256 x 128, 4 wavefronts of 64 x 128 (each B fragment feeds two products)
 static hipError_t launch_f16_tile(int tile, float* y, const uint8_t* ws, const uint8_t* packed, int M,
                                   int K, int N, const GemmGroup* group, const int* group_N, int count,
-                                  hipStream_t s) {
+                                  int ksplit, float* part, hipStream_t s) {
   switch (tile) {
-    case 0: return launch_f16<2, 2, 1, 1, 8, 2>(y, ws, packed, M, K, N, group, group_N, count, s);
-    case 1: return launch_f16<4, 1, 1, 2, 2, 4>(y, ws, packed, M, K, N, group, group_N, count, s);
-    case 2: return launch_f16<4, 1, 1, 4, 2, 3>(y, ws, packed, M, K, N, group, group_N, count, s);
-    case 3: return launch_f16<4, 1, 2, 4, 2, 1>(y, ws, packed, M, K, N, group, group_N, count, s);
+    case 0:
+      return launch_f16<2, 2, 1, 1, 8, 2>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
+    case 1:
+      return launch_f16<4, 1, 1, 2, 2, 4>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
+    case 2:
+      return launch_f16<4, 1, 1, 4, 2, 3>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
+    case 3:
+      return launch_f16<4, 1, 2, 4, 2, 1>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
   }
   return hipErrorInvalidValue;
 }
@@ -569,10 +646,12 @@ hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M
     return launch_gemm_i8(y, ws, packed, M, K, N, s);
   }
   if (kernel >= kKernelGemmF16Tile && kernel < kKernelGemmF16Tile + kGemmF16Tiles) {
-    return launch_f16_tile(kernel - kKernelGemmF16Tile, y, ws, packed, M, K, N, nullptr, nullptr, 0, s);
+    return launch_f16_tile(kernel - kKernelGemmF16Tile, y, ws, packed, M, K, N, nullptr, nullptr, 0, 1,
+                           nullptr, s);
   }
   const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-  return launch_f16_tile(choose_f16_tile(tiles, K), y, ws, packed, M, K, N, nullptr, nullptr, 0, s);
+  return launch_f16_tile(choose_f16_tile(tiles, K), y, ws, packed, M, K, N, nullptr, nullptr, 0, 1,
+                         nullptr, s);
 }
 
 hipError_t launch_gemm_group(float* const* y, const uint8_t* ws, const uint8_t* const* packed,
@@ -585,7 +664,29 @@ hipError_t launch_gemm_group(float* const* y, const uint8_t* ws, const uint8_t* 
     g.N[i] = N[i];
     tiles += (long)((M + 127) / 128) * ((N[i] + 127) / 128);
   }
-  return launch_f16_tile(choose_f16_tile(tiles, K), nullptr, ws, nullptr, M, K, 0, &g, N, count, s);
+  return launch_f16_tile(choose_f16_tile(tiles, K), nullptr, ws, nullptr, M, K, 0, &g, N, count, 1,
+                         nullptr, s);
+}
+
+// Split-K: tile shape and number of parts for a problem (parts == 1: not worth splitting).
+// Measured on MI355X (down_proj, K = 8960, N = 1536): M = 128: 44 -> 19 us, 256: 48 -> 21,
+// 512: 51 -> 30, 2048: 95 -> 80; at K = 1536 and K = 5120 the second kernel and the partial sums'
+// traffic cost what the shorter loops gain, so only long K qualifies.
+SplitPlan splitk_plan(int M, int K, int N) {
+  SplitPlan p{2, 1};
+  const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+  const int nstages = (K + kF16BK - 1) / kF16BK;
+  if (M <= 32 || nstages < 96 || tiles > 256) return p;
+  long parts = (640 + tiles / 2) / tiles;
+  parts = parts < 2 ? 2 : parts > 10 ? 10 : parts;
+  p.parts = (int)parts;
+  return p;
+}
+
+hipError_t launch_gemm_splitk(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
+                              float* part, hipStream_t s) {
+  const SplitPlan p = splitk_plan(M, K, N);
+  return launch_f16_tile(p.tile, y, ws, packed, M, K, N, nullptr, nullptr, 0, p.parts, part, s);
 }
 
 }  // namespace w4

@@ -40,6 +40,14 @@ hipError_t launch_gemv_decode(float* const* y, const float* x, const uint8_t* co
                               const float* norm_w, float eps, bool pair, hipStream_t s);
 hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                        int kernel, hipStream_t s);
+// the f16 kernel with every tile's k range dealt to several workgroups (partial sums in `part`,
+// which holds parts * M * N floats), then a reduction; for few tiles and a long K
+struct SplitPlan {
+  int tile, parts;
+};
+SplitPlan splitk_plan(int M, int K, int N);
+hipError_t launch_gemm_splitk(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
+                              float* part, hipStream_t s);
 // several Linears on the same quantised rows in one launch of the f16 kernel (M > 32)
 hipError_t launch_gemm_group(float* const* y, const uint8_t* ws, const uint8_t* const* packed,
                              const int* N, int count, int M, int K, hipStream_t s);

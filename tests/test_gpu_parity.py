@@ -300,6 +300,32 @@ def test_gemm_each_kernel_matches_oracle(pkg, orc, kernel, m, k, n):
     assert err <= GEMM_TOL and err <= TIGHT, (kernel, err)
 
 
+@pytest.mark.parametrize("m,k,n", [(512, 8960, 1536), (100, 8960, 50), (300, 6144, 272), (64, 256, 64)])
+def test_splitk_matches_oracle_and_plain(pkg, orc, m, k, n):
+    # few tiles and a long K: the k range of a tile is dealt to several workgroups and the parts are
+    # added by a second kernel; the last shape is one the library does not split (falls through)
+    w = make_weights(n, k, seed=n)
+    x = make_acts(m, k, seed=m, outlier_frac=0.02)
+    bias = bias_for(n, True)
+    u4, sc = orc.quant_rhs(w)
+    packed = pkg.repack_native(dev(u4), dev(sc.view(np.int16)), dev(bias), n, k)
+    ws = pkg.quant_lhs(dev(x))
+    split = int(pkg.lib().w4a32_splitk_scratch_bytes(m, k, n)) > 0
+    assert split == (k >= 6144)
+    y = host(pkg.matmul_quantized_splitk(ws, packed, m, k, n))
+    plain = host(pkg.matmul_quantized(ws, packed, m, k, n))
+    rows = np.unique(np.concatenate([np.arange(0, m, 37), [m - 1]]))
+    ref = orc.linear(x[rows], u4, sc, bias=bias, threads=8)
+    assert max_abs_rel(y[rows], ref) <= TIGHT
+    assert max_abs_rel(y, plain) <= 1e-6          # same products, another f32 summation order
+    if not split:
+        assert np.array_equal(y, plain)
+    # too little scratch: the plain kernel runs
+    import torch
+    tiny = torch.empty((16,), dtype=torch.uint8, device="cuda")
+    assert np.array_equal(host(pkg.matmul_quantized_splitk(ws, packed, m, k, n, scratch=tiny)), plain)
+
+
 def test_f16_kernel_with_wide_scale_range(pkg, orc):
     # rows whose block scales differ by many octaves, and rows that are tiny or huge overall:
     # the per-row power-of-two normalisation must keep the f16 operands exact
