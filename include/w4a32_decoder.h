@@ -34,6 +34,19 @@ int w4a32_op_rmsnorm(const float* d_h, const float* d_delta, const float* d_weig
 int w4a32_op_add(const float* d_a, const float* d_b, float* d_out, size_t n, void* stream);
 int w4a32_op_silu_mul(const float* d_gate, const float* d_up, float* d_out, size_t n, void* stream);
 
+/* The two operators above with the row quantiser of the Linear that reads their result behind them
+ * (w4a32_quant_lhs, include/w4a32_hip.h): the f32 rows they would write are never stored, the
+ * quantised rows go to d_ws for w4a32_matmul_quantized*(). For M > 8 rows of K <= 16384 values.
+ *   norm:     h_out = h + delta (skipped when d_delta is NULL; d_h_out may alias d_h), then the
+ *             rows h_out * (w * 1/sqrt(mean(h_out^2) + eps)) are quantised;
+ *   silu_mul: the rows silu(gate) * up are quantised.
+ * The reference runs RMSNormOp / the MLP's elementwise ops and the Linear's own row quantiser as
+ * separate passes (RMSNormOp.cpp:36-76, modeling_ds_qwen2.hpp:47-54, kai_linear.cpp:358-362). */
+int w4a32_quant_lhs_norm(const float* d_h, const float* d_delta, const float* d_weight, float eps,
+                         float* d_h_out, int M, int K, void* d_ws, void* stream);
+int w4a32_quant_lhs_silu_mul(const float* d_gate, const float* d_up, int M, int K, void* d_ws,
+                             void* stream);
+
 /* sin/cos tables [max_pos][head_dim/2]: theta = pos / base^(2d/head_dim).
  * precompute_normal_hf_sin_cos, mllm/Backends/Arm/Kernels/rope.cpp:20-37. */
 int w4a32_op_rope_table(float* d_sin, float* d_cos, int max_pos, int head_dim, float base,

@@ -149,6 +149,12 @@ int w4a32_matmul(float* d_y, const float* d_x, const void* d_packed, void* d_ws,
 int w4a32_matmul_grouped(float* const* d_y, const float* d_x, const void* const* d_packed,
                          const int* N, int count, void* d_ws, int M, int K, void* stream);
 
+/* The grouped product on rows that are already quantised into d_ws (w4a32_quant_lhs or one of the
+ * fused quantisers of w4a32_decoder.h): at M > 32 one launch of the prefill kernel over all the
+ * Linears, else one product per Linear. */
+int w4a32_matmul_quantized_grouped(float* const* d_y, const void* d_ws, const void* const* d_packed,
+                                   const int* N, int count, int M, int K, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

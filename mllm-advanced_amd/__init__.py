@@ -39,6 +39,9 @@ ABI = {
     "w4a32_export_lhs": (_ci, [_vp, _ci, _ci, _vp, _vp, _vp, _vp]),
     "w4a32_matmul_quantized": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a32_matmul_quantized_ex": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp]),
+    "w4a32_matmul_quantized_grouped": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
+    "w4a32_quant_lhs_norm": (_ci, [_vp, _vp, _vp, ctypes.c_float, _vp, _ci, _ci, _vp, _vp]),
+    "w4a32_quant_lhs_silu_mul": (_ci, [_vp, _vp, _ci, _ci, _vp, _vp]),
     "w4a32_splitk_scratch_bytes": (_sz, [_ci, _ci, _ci]),
     "w4a32_matmul_quantized_splitk": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a32_matmul": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
@@ -208,6 +211,29 @@ def quant_lhs(x, ws=None):
     if ws is None:
         ws = _dev_empty(workspace_bytes(M, K))
     _check(lib().w4a32_quant_lhs(_ptr(x), M, K, x.stride(0), _ptr(ws), _stream()), "w4a32_quant_lhs")
+    return ws
+
+
+def quant_lhs_norm(h, weight, eps, delta=None, ws=None):
+    """Residual add + RMSNorm + row quantiser in one launch: returns (ws, h + delta or None)."""
+    import torch
+
+    M, K = h.shape
+    if ws is None:
+        ws = _dev_empty(workspace_bytes(M, K))
+    h_out = torch.empty_like(h) if delta is not None else None
+    _check(lib().w4a32_quant_lhs_norm(_ptr(h), _ptr(delta), _ptr(weight), eps, _ptr(h_out), M, K,
+                                      _ptr(ws), _stream()), "w4a32_quant_lhs_norm")
+    return ws, h_out
+
+
+def quant_lhs_silu_mul(gate, up, ws=None):
+    """silu(gate) * up + row quantiser in one launch."""
+    M, K = gate.shape
+    if ws is None:
+        ws = _dev_empty(workspace_bytes(M, K))
+    _check(lib().w4a32_quant_lhs_silu_mul(_ptr(gate), _ptr(up), M, K, _ptr(ws), _stream()),
+           "w4a32_quant_lhs_silu_mul")
     return ws
 
 

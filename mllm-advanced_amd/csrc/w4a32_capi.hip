@@ -214,10 +214,24 @@ int w4a32_matmul_grouped(float* const* d_y, const float* d_x, const void* const*
   // other sizes: quantise the rows once, then one launch of the f16 kernel over all the Linears
   // (M > 32) or one product per Linear
   if (int e = w4a32_quant_lhs(d_x, M, K, K, d_ws, stream)) return e;
-  if (M > 32) {
+  return w4a32_matmul_quantized_grouped(d_y, d_ws, d_packed, N, count, M, K, stream);
+}
+
+int w4a32_matmul_quantized_grouped(float* const* d_y, const void* d_ws, const void* const* d_packed,
+                                   const int* N, int count, int M, int K, void* stream) {
+  if (!d_y || !d_ws || !d_packed || !N) return W4A32_EINVAL;
+  if (count < 1 || count > W4A32_MAX_GROUP || M <= 0) return W4A32_EINVAL;
+  for (int i = 0; i < count; ++i) {
+    if (int e = shape_ok(N[i], K)) return e;
+    if (!d_y[i] || !d_packed[i]) return W4A32_EINVAL;
+    if (!aligned(d_packed[i], 16) || !aligned(d_y[i], 4)) return W4A32_EINVAL;
+  }
+  if (!aligned(d_ws, 256)) return W4A32_EINVAL;
+  if (M > 32 && count > 1) {
     const uint8_t* pk[W4A32_MAX_GROUP];
     for (int i = 0; i < count; ++i) pk[i] = static_cast<const uint8_t*>(d_packed[i]);
-    return from_hip(w4::launch_gemm_group(d_y, static_cast<const uint8_t*>(d_ws), pk, N, count, M, K, s));
+    return from_hip(w4::launch_gemm_group(d_y, static_cast<const uint8_t*>(d_ws), pk, N, count, M, K,
+                                          static_cast<hipStream_t>(stream)));
   }
   for (int i = 0; i < count; ++i) {
     if (int e = w4a32_matmul_quantized(d_y[i], d_ws, d_packed[i], M, K, N[i], stream)) return e;

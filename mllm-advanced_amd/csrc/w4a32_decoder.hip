@@ -127,14 +127,22 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
     const w4a32_layer_weights& lw = w->layers[l];
     float* kc = reinterpret_cast<float*>(st + g.kcache_off) + (size_t)l * g.cache_layer;
     float* vc = reinterpret_cast<float*>(st + g.vcache_off) + (size_t)l * g.cache_layer;
+    // Prefill sizes: the operator in front of a Linear runs inside that Linear's row quantiser.
+    const bool fuse_rows = M > 32 && w4::quant_rows_fusable(std::max(H, I));
     // h += mlp output of the previous layer; xn = norm(h)
-    W4_TRY(from_hip(w4::launch_rmsnorm(h, l == 0 ? nullptr : delta, lw.attn_norm, M, H, c->rms_eps, h,
-                                       xn, s)));
     {
       float* ys[3] = {q, k, v};
       const void* ps[3] = {lw.q, lw.k, lw.v};
       const int ns[3] = {qd, kvd, kvd};
-      W4_TRY(w4a32_matmul_grouped(ys, xn, ps, ns, 3, ws, M, H, stream));
+      if (fuse_rows) {
+        W4_TRY(w4a32_quant_lhs_norm(h, l == 0 ? nullptr : delta, lw.attn_norm, c->rms_eps, h, M, H, ws,
+                                    stream));
+        W4_TRY(w4a32_matmul_quantized_grouped(ys, ws, ps, ns, 3, M, H, stream));
+      } else {
+        W4_TRY(from_hip(w4::launch_rmsnorm(h, l == 0 ? nullptr : delta, lw.attn_norm, M, H, c->rms_eps,
+                                           h, xn, s)));
+        W4_TRY(w4a32_matmul_grouped(ys, xn, ps, ns, 3, ws, M, H, stream));
+      }
     }
     W4_TRY(from_hip(w4::launch_rope_kv(q, k, v, sin_t, cos_t, kc, vc, M, Hq, Hkv, D, c->max_seq, d_pos,
                                        0, s)));
@@ -148,21 +156,31 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
     }
     W4_TRY(w4a32_matmul(delta, attn, lw.o, ws, M, qd, H, stream));
     // h += attention output; xn = norm(h)
-    W4_TRY(from_hip(w4::launch_rmsnorm(h, delta, lw.ffn_norm, M, H, c->rms_eps, h, xn, s)));
     {
       float* ys[2] = {gate, up};
       const void* ps[2] = {lw.gate, lw.up};
       const int ns[2] = {I, I};
-      W4_TRY(w4a32_matmul_grouped(ys, xn, ps, ns, 2, ws, M, H, stream));
+      if (fuse_rows) {
+        W4_TRY(w4a32_quant_lhs_norm(h, delta, lw.ffn_norm, c->rms_eps, h, M, H, ws, stream));
+        W4_TRY(w4a32_matmul_quantized_grouped(ys, ws, ps, ns, 2, M, H, stream));
+      } else {
+        W4_TRY(from_hip(w4::launch_rmsnorm(h, delta, lw.ffn_norm, M, H, c->rms_eps, h, xn, s)));
+        W4_TRY(w4a32_matmul_grouped(ys, xn, ps, ns, 2, ws, M, H, stream));
+      }
     }
-    W4_TRY(from_hip(w4::launch_silu_mul(gate, up, act, (size_t)M * I, s)));
     if (M > 32) {
+      if (fuse_rows) {
+        W4_TRY(w4a32_quant_lhs_silu_mul(gate, up, M, I, ws, stream));
+      } else {
+        W4_TRY(from_hip(w4::launch_silu_mul(gate, up, act, (size_t)M * I, s)));
+        W4_TRY(w4a32_quant_lhs(act, M, I, I, ws, stream));
+      }
       // few output tiles, long K: split-K, with the partial sums in the gate and up buffers,
-      // which are dead once `act` holds silu(gate) * up
-      W4_TRY(w4a32_quant_lhs(act, M, I, I, ws, stream));
+      // which are dead once the quantised rows of silu(gate) * up exist
       const size_t lend = g.up_off - g.gate_off + sizeof(float) * (size_t)c->max_batch_tokens * I;
       W4_TRY(w4a32_matmul_quantized_splitk(delta, ws, lw.down, M, I, H, gate, lend, stream));
     } else {
+      W4_TRY(from_hip(w4::launch_silu_mul(gate, up, act, (size_t)M * I, s)));
       W4_TRY(w4a32_matmul(delta, act, lw.down, ws, M, I, H, stream));
     }
   }
@@ -288,6 +306,25 @@ int w4a32_op_silu_mul(const float* d_gate, const float* d_up, float* d_out, size
   if (!d_gate || !d_up || !d_out || n == 0) return W4A32_EINVAL;
   if (n % 4 != 0) return W4A32_ESHAPE;
   return from_hip(w4::launch_silu_mul(d_gate, d_up, d_out, n, S(stream)));
+}
+
+int w4a32_quant_lhs_norm(const float* d_h, const float* d_delta, const float* d_weight, float eps,
+                         float* d_h_out, int M, int K, void* d_ws, void* stream) {
+  if (!d_h || !d_weight || !d_ws || M <= 0 || K <= 0) return W4A32_EINVAL;
+  if (d_delta && !d_h_out) return W4A32_EINVAL;
+  if (K % 32 != 0 || M <= w4::kGemvMaxM || !w4::quant_rows_fusable(K)) return W4A32_ESHAPE;
+  if ((reinterpret_cast<uintptr_t>(d_ws) & 255) != 0) return W4A32_EINVAL;
+  return from_hip(w4::launch_quant_lhs_norm(d_h, d_delta, d_weight, eps, d_h_out, M, K,
+                                            static_cast<uint8_t*>(d_ws), S(stream)));
+}
+
+int w4a32_quant_lhs_silu_mul(const float* d_gate, const float* d_up, int M, int K, void* d_ws,
+                             void* stream) {
+  if (!d_gate || !d_up || !d_ws || M <= 0 || K <= 0) return W4A32_EINVAL;
+  if (K % 32 != 0 || M <= w4::kGemvMaxM || !w4::quant_rows_fusable(K)) return W4A32_ESHAPE;
+  if ((reinterpret_cast<uintptr_t>(d_ws) & 255) != 0) return W4A32_EINVAL;
+  return from_hip(w4::launch_quant_lhs_silu_mul(d_gate, d_up, M, K, static_cast<uint8_t*>(d_ws),
+                                                S(stream)));
 }
 
 int w4a32_op_rope_table(float* d_sin, float* d_cos, int max_pos, int head_dim, float base, void* stream) {

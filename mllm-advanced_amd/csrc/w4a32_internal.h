@@ -20,6 +20,13 @@ hipError_t launch_dequant(const uint8_t* packed, int N, int K, float* out, hipSt
 
 // activations (every forward)
 hipError_t launch_quant_lhs(const float* x, int M, int K, int ldx, uint8_t* ws, hipStream_t s);
+// the quantiser with the operator that produces its rows in front (prefill sizes): residual add +
+// RMSNorm, or silu(gate) * up; K must satisfy quant_rows_fusable()
+bool quant_rows_fusable(int K);
+hipError_t launch_quant_lhs_norm(const float* h, const float* delta, const float* norm_w, float eps,
+                                 float* h_out, int M, int K, uint8_t* ws, hipStream_t s);
+hipError_t launch_quant_lhs_silu_mul(const float* gate, const float* up, int M, int K, uint8_t* ws,
+                                     hipStream_t s);
 
 // products
 hipError_t launch_gemv(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,

@@ -42,6 +42,48 @@ def test_embedding_rmsnorm_add_silu(pkg):
     assert max_abs_rel(pkg.op_silu_mul(a, b).cpu().numpy(), ref.cpu().numpy()) < 1e-5
 
 
+@pytest.mark.parametrize("M,K", [(40, 1536), (512, 1536), (33, 8960), (9, 96), (64, 16384)])
+def test_fused_row_quantisers_match_separate_operators(pkg, M, K):
+    # norm + quantiser and silu*mul + quantiser in one launch against operator, then quantiser
+    g = torch.Generator(device="cuda").manual_seed(M + K)
+    h = torch.randn((M, K), generator=g, device="cuda") * 2
+    d = torch.randn((M, K), generator=g, device="cuda")
+    w = 1 + 0.1 * torch.randn((K,), generator=g, device="cuda")
+    for delta in (None, d):
+        ws, h_out = pkg.quant_lhs_norm(h, w, 1e-6, delta=delta)
+        if delta is None:
+            y = pkg.op_rmsnorm(h, w, 1e-6)
+        else:
+            h_ref, y = pkg.op_rmsnorm(h, w, 1e-6, delta=delta)
+            assert torch.equal(h_out, h_ref)
+        aq, recip, nzp = pkg.export_lhs(ws, M, K)
+        aq0, recip0, nzp0 = pkg.export_lhs(pkg.quant_lhs(y), M, K)
+        # the sum of squares is taken in another order: the normalised row may differ in its last
+        # bit, which moves a value that sits on a rounding boundary by one step
+        assert torch.allclose(recip, recip0, rtol=1e-6, atol=0)
+        assert int((nzp - nzp0).abs().max()) <= 1
+        diff = (aq.int() - aq0.int()).abs()
+        assert int(diff.max()) <= 1 and float((diff > 0).float().mean()) < 2e-3
+        deq = (aq.float() + nzp.float()[:, None]) * recip[:, None]
+        assert float((deq - y).abs().max()) <= 1.01 * float(recip.max())
+    gate = torch.randn((M, K), generator=g, device="cuda") * 3
+    up = torch.randn((M, K), generator=g, device="cuda")
+    a1 = pkg.export_lhs(pkg.quant_lhs_silu_mul(gate, up), M, K)
+    a0 = pkg.export_lhs(pkg.quant_lhs(pkg.op_silu_mul(gate, up)), M, K)
+    for x1, x0 in zip(a1, a0):
+        assert torch.equal(x1, x0)          # elementwise: the same arithmetic, bit for bit
+
+
+def test_fused_row_quantisers_reject_what_they_do_not_take(pkg):
+    h = torch.zeros((8, 64), device="cuda")
+    w = torch.ones((64,), device="cuda")
+    with pytest.raises(RuntimeError):
+        pkg.quant_lhs_norm(h, w, 1e-6)                     # decode sizes use w4a32_decode_linear
+    big = torch.zeros((16, 16416), device="cuda")
+    with pytest.raises(RuntimeError):
+        pkg.quant_lhs_silu_mul(big, big)                   # row too long for the register kernel
+
+
 def test_rope_table_and_kv_append(pkg):
     import decoder_oracle as do
 
