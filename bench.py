@@ -234,6 +234,36 @@ def main():
                                        "GBps": round(step_bytes / (ms_single * 1e-3) / 1e9, 1)},
              "product_only_ms_per_step": round(ms_prod, 4)}
 
+    # ---- the same pass on 4 and 8 rows (batched decode): same launches, same weight bytes
+    batched = {}
+    for Mb in (4, 8):
+        xb = {K: torch.randn((Mb, K), generator=xgen, device="cuda") for K in (1536, 8960)}
+        wsb = {K: torch.empty(pkg.workspace_bytes(Mb, K), dtype=torch.uint8, device="cuda")
+               for K in (1536, 8960)}
+        yb = {N: torch.empty((Mb, N), device="cuda") for N in (256, 1536, 8960, 151936)}
+        yb2 = {256: torch.empty((Mb, 256), device="cuda"), 8960: torch.empty((Mb, 8960), device="cuda")}
+        calls_b = []
+        for layer in layers:
+            q, k, v, o, gate, up, down = layer
+            calls_b.append((group_args([q, k, v], [yb[1536], yb[256], yb2[256]]), 1536))
+            calls_b.append((group_args([o], [yb[1536]]), 1536))
+            calls_b.append((group_args([gate, up], [yb[8960], yb2[8960]]), 1536))
+            calls_b.append((group_args([down], [yb[1536]]), 8960))
+        calls_b.append((group_args([lm_head], [yb[151936]]), 1536))
+
+        def batched_pass(calls_b=calls_b, xb=xb, wsb=wsb, Mb=Mb):
+            for (ya, pa, na, cnt), K in calls_b:
+                rc = L.w4a32_matmul_grouped(ya, xb[K].data_ptr(), pa, na, cnt, wsb[K].data_ptr(), Mb, K, sptr)
+                if rc:
+                    raise pkg.W4A32Error(f"w4a32_matmul_grouped M={Mb} -> {rc}")
+        ms_b, _ = timed(batched_pass, args.steps, args.warmup, use_graph)
+        bytes_b = sum(algorithmic_bytes(Mb, l.K, l.N, l.has_bias) for l in step_linears)
+        batched[f"M{Mb}"] = {"ms_per_step": round(ms_b, 4), "GBps": round(bytes_b / (ms_b * 1e-3) / 1e9, 1),
+                             "rows_per_s": round(Mb * 1e3 / ms_b, 1),
+                             "flop_equiv_TFLOPs": round(sum(2.0 * Mb * l.K * l.N for l in step_linears)
+                                                        / (ms_b * 1e-3) / 1e12, 2)}
+    extra["decode_pass_batched"] = batched
+
     # ---- per-shape decode figures (product kernel, weights rotated over the 28 layers)
     per_shape = {}
     reps = 20
@@ -316,9 +346,46 @@ def main():
                     tot_flop += flop
                     tot_ms += times[0]
                     tot_kms += times[1]
+                # The layer's Linears as a prefill issues them: rows quantised once per input, q,k,v and
+                # gate,up each as one grouped launch, down with its k range split over workgroups
+                # (partial sums in lent scratch).
+                lay = layers[0]
+                xh = torch.randn((M, 1536), generator=xgen, device="cuda")
+                xi = torch.randn((M, 8960), generator=xgen, device="cuda")
+                ws_h = torch.empty(pkg.workspace_bytes(M, 1536), dtype=torch.uint8, device="cuda")
+                ws_i = torch.empty(pkg.workspace_bytes(M, 8960), dtype=torch.uint8, device="cuda")
+                yq, yk, yv = (torch.empty((M, n), device="cuda") for n in (1536, 256, 256))
+                yg, yu = (torch.empty((M, 8960), device="cuda") for _ in range(2))
+                yo = torch.empty((M, 1536), device="cuda")
+                scratch = torch.empty(max(16, int(L.w4a32_splitk_scratch_bytes(M, 8960, 1536))),
+                                      dtype=torch.uint8, device="cuda")
+
+                def issued():
+                    pkg.quant_lhs(xh, ws_h)
+                    pkg.matmul_quantized_grouped(ws_h, [lay[0].packed, lay[1].packed, lay[2].packed],
+                                                 [1536, 256, 256], M, 1536, outs=[yq, yk, yv])
+                    pkg.quant_lhs(xh, ws_h)
+                    pkg.matmul_quantized(ws_h, lay[3].packed, M, 1536, 1536, out=yo)
+                    pkg.quant_lhs(xh, ws_h)
+                    pkg.matmul_quantized_grouped(ws_h, [lay[4].packed, lay[5].packed], [8960, 8960], M,
+                                                 1536, outs=[yg, yu])
+                    pkg.quant_lhs(xi, ws_i)
+                    pkg.matmul_quantized_splitk(ws_i, lay[6].packed, M, 8960, 1536, scratch=scratch, out=yo)
+                for _ in range(3):
+                    issued()
+                e0 = torch.cuda.Event(enable_timing=True)
+                e1 = torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for _ in range(20):
+                    issued()
+                e1.record(stream)
+                stream.synchronize()
+                issued_ms = e0.elapsed_time(e1) / 20
                 prefill[f"M{M}"] = {"per_shape": per,
                                     "layer_TFLOPs": round(tot_flop / (tot_ms * 1e-3) / 1e12, 1),
-                                    "layer_kernel_TFLOPs": round(tot_flop / (tot_kms * 1e-3) / 1e12, 1)}
+                                    "layer_kernel_TFLOPs": round(tot_flop / (tot_kms * 1e-3) / 1e12, 1),
+                                    "layer_as_issued_ms": round(issued_ms, 4),
+                                    "layer_as_issued_TFLOPs": round(tot_flop / (issued_ms * 1e-3) / 1e12, 1)}
         extra["prefill"] = prefill
         best = prefill["M2048"]["per_shape"]["gate_proj"]["kernel_TFLOPs"]
         extra["prefill_roofline"] = {"bound": "mfma", "kernel": "gemm_f16_kernel (v_mfma_f32_32x32x16_f16)",

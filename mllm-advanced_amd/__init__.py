@@ -257,6 +257,20 @@ def matmul_quantized(ws, packed, M, K, N, out=None, kernel=KERNEL_AUTO):
     return y
 
 
+def matmul_quantized_grouped(ws, packed_list, Ns, M, K, outs=None):
+    """Several Linears on rows already quantised into ws (one launch at M > 32)."""
+    import torch
+
+    n = len(Ns)
+    ys = outs if outs is not None else [torch.empty((M, N), dtype=torch.float32, device="cuda") for N in Ns]
+    yarr = (ctypes.c_void_p * n)(*[y.data_ptr() for y in ys])
+    parr = (ctypes.c_void_p * n)(*[p.data_ptr() for p in packed_list])
+    narr = (ctypes.c_int * n)(*Ns)
+    _check(lib().w4a32_matmul_quantized_grouped(yarr, _ptr(ws), parr, narr, n, M, K, _stream()),
+           "w4a32_matmul_quantized_grouped")
+    return ys
+
+
 def matmul_quantized_splitk(ws, packed, M, K, N, scratch=None, out=None):
     """matmul_quantized() with scratch memory lent for partial sums (allocated here when absent)."""
     import torch

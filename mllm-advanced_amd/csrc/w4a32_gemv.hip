@@ -25,6 +25,15 @@
 // Arithmetic per 8 weights (one dword): two mask ops give int8 vectors of 16*q, two
 // v_dot4_i32_i8 give 16 * sum a_q*q exactly, one cvt + one fma apply the block scale in f32.
 // The 1/16 and the activation offset (off * rsum[n]) are folded in once per output.
+//
+// From three rows on (kDecodeMfmaMinM) the dot products of a scale block come from ONE
+// v_mfma_i32_16x16x32_i8 instead of 2*M v_dot4: the tile dword of all 64 lanes, expanded by the
+// same two mask ops, is its B operand (column = lane % 16, k-slice = lane / 16), the A operand is
+// 8 bytes of activation row lane % 16 (rows past M repeat the last one; their results are not
+// used). Lane (g, j) then holds the exact block sums of rows 4g..4g+3 for column j, already
+// summed over the four k-groups; cvt + fma apply the block scale as before, so every output is
+// the same f32 expression in the same order as on the dot4 path. The instruction count per chunk
+// no longer grows with M (M = 8: 130 -> 45 per wavefront).
 #include <algorithm>
 
 #include "w4a32_internal.h"
@@ -32,15 +41,68 @@
 
 namespace w4 {
 
+typedef int v4i_t __attribute__((ext_vector_type(4)));
+constexpr int kDecodeMfmaMinM = 3;
+constexpr bool decode_mfma(int M) { return M >= kDecodeMfmaMinM; }
+// accumulators per lane: one per row (a partial over this lane's k-group) or, on the MFMA path,
+// rows 4g..4g+3 of column j
+constexpr int decode_acc(int M) { return decode_mfma(M) ? 4 : M; }
+
+// One scale block (tile dword wv, scale sv) against the M int8 rows at a_base (+ m * Kp); a_base
+// already points at this lane's k-group.
+template <int M>
+__device__ __forceinline__ void block_products(uint32_t wv, float sv, const int8_t* a_base, int Kp,
+                                               int j, float (&acc)[decode_acc(M)]) {
+  const uint32_t lo = (wv << 4) & 0xF0F0F0F0u;  // 16*q at k offsets 0..3
+  const uint32_t hi = wv & 0xF0F0F0F0u;         // 16*q at k offsets 4..7
+  if constexpr (decode_mfma(M)) {
+    const long b64 = (long)(((unsigned long)hi << 32) | lo);
+    const long a64 = *reinterpret_cast<const long*>(a_base + (size_t)(j < M ? j : M - 1) * Kp);
+    v4i_t c = {0, 0, 0, 0};
+    c = __builtin_amdgcn_mfma_i32_16x16x32_i8(a64, b64, c, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[r] = __fmaf_rn((float)c[r], sv, acc[r]);
+  } else {
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      const int2 a = *reinterpret_cast<const int2*>(a_base + (size_t)m * Kp);
+      int dot = __builtin_amdgcn_sdot4(a.x, (int)lo, 0, false);
+      dot = __builtin_amdgcn_sdot4(a.y, (int)hi, dot, false);
+      acc[m] = __fmaf_rn((float)dot, sv, acc[m]);
+    }
+  }
+}
+
+// The sums of a wavefront, complete over its k-groups, to s_dst[m * 16 + j].
+template <int M>
+__device__ __forceinline__ void store_row_sums(float (&acc)[decode_acc(M)], float* s_dst, int lane) {
+  const int g = lane >> 4, j = lane & 15;
+  if constexpr (decode_mfma(M)) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = 4 * g + r;
+      if (m < M) s_dst[m * 16 + j] = acc[r];
+    }
+  } else {
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      float v = acc[m];
+      v += __shfl_xor(v, 16, 64);
+      v += __shfl_xor(v, 32, 64);
+      if (lane < 16) s_dst[m * 16 + lane] = v;
+    }
+  }
+}
+
 // Streams this wavefront's chunks of tile row `tiles` against the int8 rows in LDS and leaves
 // the per-(m, j) sums over the whole workgroup in s_red[m*16 + j] order via a final reduction.
 template <int M>
 __device__ __forceinline__ void gemv_accumulate(const uint8_t* __restrict__ tiles, int KC, int Kp,
                                                 const int8_t* s_a, uint4 wq, uint2 sc, int kc,
-                                                int W, int lane, float (&acc)[M]) {
+                                                int W, int lane, float (&acc)[decode_acc(M)]) {
   const int g = lane >> 4, j = lane & 15;
 #pragma unroll
-  for (int m = 0; m < M; ++m) acc[m] = 0.0f;
+  for (int m = 0; m < decode_acc(M); ++m) acc[m] = 0.0f;
 
   while (kc < KC) {
     const int kn = kc + W;
@@ -55,26 +117,11 @@ __device__ __forceinline__ void gemv_accumulate(const uint8_t* __restrict__ tile
                          __uint_as_float(sc.y << 16), __uint_as_float(sc.y & 0xFFFF0000u)};
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-      const int lo = (int)((wv[d] << 4) & 0xF0F0F0F0u);  // 16*q at k offsets 0..3
-      const int hi = (int)(wv[d] & 0xF0F0F0F0u);         // 16*q at k offsets 4..7
-      const int8_t* a_base = s_a + kTileK * kc + kBlockLen * d + 8 * g;
-#pragma unroll
-      for (int m = 0; m < M; ++m) {
-        const int2 a = *reinterpret_cast<const int2*>(a_base + (size_t)m * Kp);
-        int dot = __builtin_amdgcn_sdot4(a.x, lo, 0, false);
-        dot = __builtin_amdgcn_sdot4(a.y, hi, dot, false);
-        acc[m] = __fmaf_rn((float)dot, sv[d], acc[m]);
-      }
+      block_products<M>(wv[d], sv[d], s_a + kTileK * kc + kBlockLen * d + 8 * g, Kp, j, acc);
     }
     kc = kn;
     wq = wq_n;
     sc = sc_n;
-  }
-  // Sum the four k-groups of a row (lanes j, j+16, j+32, j+48).
-#pragma unroll
-  for (int m = 0; m < M; ++m) {
-    acc[m] += __shfl_xor(acc[m], 16, 64);
-    acc[m] += __shfl_xor(acc[m], 32, 64);
   }
 }
 
@@ -87,15 +134,12 @@ constexpr int kMaxWaves = 16;  // wavefronts per workgroup, at most
 // stride over the outputs and fetch them here.
 template <int M>
 __device__ __forceinline__ void gemv_finish(float* __restrict__ y, int N, int nt, int W,
-                                            const float (&acc)[M], float* s_red,
+                                            float (&acc)[decode_acc(M)], float* s_red,
                                             const float (&recip_m)[M], const int (&negzp_m)[M],
                                             const float* __restrict__ rsum,
                                             const float* __restrict__ bias, float rs, float bs) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  if (lane < 16) {
-#pragma unroll
-    for (int m = 0; m < M; ++m) s_red[(wave * M + m) * 16 + lane] = acc[m];
-  }
+  store_row_sums<M>(acc, s_red + wave * M * 16, lane);
   __syncthreads();
   const bool prefetched = blockDim.x >= 16 * M;
   for (int o = threadIdx.x; o < 16 * M; o += blockDim.x) {
@@ -177,7 +221,7 @@ __global__ __launch_bounds__(1024) void gemv_q_kernel(
   }
   __syncthreads();
 
-  float acc[M];
+  float acc[decode_acc(M)];
   gemv_accumulate<M>(tiles, KC, Kp, s_a, wq, sc, wave, W, lane, acc);
   float recip_m[M];
   int negzp_m[M];
@@ -426,11 +470,11 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
   }
   __syncthreads();
 
-  float acc[kSets][M];
+  float acc[kSets][decode_acc(M)];
 #pragma unroll
   for (int st = 0; st < kSets; ++st)
 #pragma unroll
-    for (int m = 0; m < M; ++m) acc[st][m] = 0.0f;
+    for (int m = 0; m < decode_acc(M); ++m) acc[st][m] = 0.0f;
 #pragma unroll
   for (int i = 0; i < kCPW; ++i) {
     const bool valid = wave + i * W < KC;
@@ -438,37 +482,17 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
       const int8_t* a_base = s_a + kTileK * kc + kBlockLen * d + 8 * g;
-      int2 a[M];
-#pragma unroll
-      for (int m = 0; m < M; ++m) a[m] = *reinterpret_cast<const int2*>(a_base + (size_t)m * Kp);
 #pragma unroll
       for (int st = 0; st < kSets; ++st) {
-        const uint32_t wv = wq[st][i][d];
         const uint32_t sw = sc[st][i][d >> 1];
         const uint32_t sbits = valid ? ((d & 1) ? (sw & 0xFFFF0000u) : (sw << 16)) : 0u;
-        const float sv = __uint_as_float(sbits);
-        const int lo = (int)((wv << 4) & 0xF0F0F0F0u);  // 16*q at k offsets 0..3
-        const int hi = (int)(wv & 0xF0F0F0F0u);         // 16*q at k offsets 4..7
-#pragma unroll
-        for (int m = 0; m < M; ++m) {
-          int dot = __builtin_amdgcn_sdot4(a[m].x, lo, 0, false);
-          dot = __builtin_amdgcn_sdot4(a[m].y, hi, dot, false);
-          acc[st][m] = __fmaf_rn((float)dot, sv, acc[st][m]);
-        }
+        block_products<M>(wq[st][i][d], __uint_as_float(sbits), a_base, Kp, j, acc[st]);
       }
     }
   }
-  // Sum the four k-groups of a row (lanes j, j+16, j+32, j+48), then across wavefronts via LDS.
+  // The sums of the four k-groups of a row, then across wavefronts via LDS.
 #pragma unroll
-  for (int st = 0; st < kSets; ++st) {
-#pragma unroll
-    for (int m = 0; m < M; ++m) {
-      float v = acc[st][m];
-      v += __shfl_xor(v, 16, 64);
-      v += __shfl_xor(v, 32, 64);
-      if (lane < 16) s_red[((wave * kSets + st) * M + m) * 16 + lane] = v;
-    }
-  }
+  for (int st = 0; st < kSets; ++st) store_row_sums<M>(acc[st], s_red + (wave * kSets + st) * M * 16, lane);
   __syncthreads();
 
   //   y = (sum/16 + off * rsum[n]) * lhs_scale + bias[n], clamped to the finite f32 range
@@ -726,9 +750,9 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
       rs = rsum[n];
       bs = bias[n];
     }
-    float acc[M];
+    float acc[decode_acc(M)];
 #pragma unroll
-    for (int m = 0; m < M; ++m) acc[m] = 0.0f;
+    for (int m = 0; m < decode_acc(M); ++m) acc[m] = 0.0f;
 
     for (int b = 0; b < batches; ++b) {
       // request the next batch (of this tile row, or the first of the next one) ...
@@ -758,16 +782,7 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
                                __uint_as_float(sc_cur[i].y & 0xFFFF0000u)};
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
-            const int lo = (int)((wv[d] << 4) & 0xF0F0F0F0u);
-            const int hi = (int)(wv[d] & 0xF0F0F0F0u);
-            const int8_t* a_base = s_a + kTileK * kc + kBlockLen * d + 8 * g;
-#pragma unroll
-            for (int m = 0; m < M; ++m) {
-              const int2 a = *reinterpret_cast<const int2*>(a_base + (size_t)m * Kp);
-              int dot = __builtin_amdgcn_sdot4(a.x, lo, 0, false);
-              dot = __builtin_amdgcn_sdot4(a.y, hi, dot, false);
-              acc[m] = __fmaf_rn((float)dot, sv[d], acc[m]);
-            }
+            block_products<M>(wv[d], sv[d], s_a + kTileK * kc + kBlockLen * d + 8 * g, Kp, j, acc);
           }
         }
       }
@@ -777,18 +792,37 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
         sc_cur[i] = sc_nxt[i];
       }
     }
+    if constexpr (decode_mfma(M)) {
+      // lane (g, j) holds rows 4g..4g+3 of column j; rsum / bias of the column sit in lane j
+      const float rsj = __shfl(rs, j, 64), bsj = __shfl(bs, j, 64);
+      if (n < N) {
 #pragma unroll
-    for (int m = 0; m < M; ++m) {
-      acc[m] += __shfl_xor(acc[m], 16, 64);
-      acc[m] += __shfl_xor(acc[m], 32, 64);
-    }
-    if (lane < 16 && n < N) {
+        for (int m = 0; m < M; ++m) {  // compile-time row index: negzp_m / recip_m stay in registers
+          if ((m >> 2) == g) {
+            float sum = acc[0];
+#pragma unroll
+            for (int r = 1; r < 4; ++r) sum = (m & 3) == r ? acc[r] : sum;
+            float v = __fmaf_rn((float)negzp_m[m], rsj, sum * 0.0625f);
+            v = __fmaf_rn(v, recip_m[m], bsj);
+            v = fminf(fmaxf(v, -3.402823466e+38f), 3.402823466e+38f);
+            y[(size_t)m * N + n] = v;
+          }
+        }
+      }
+    } else {
 #pragma unroll
       for (int m = 0; m < M; ++m) {
-        float v = __fmaf_rn((float)negzp_m[m], rs, acc[m] * 0.0625f);
-        v = __fmaf_rn(v, recip_m[m], bs);
-        v = fminf(fmaxf(v, -3.402823466e+38f), 3.402823466e+38f);
-        y[(size_t)m * N + n] = v;
+        acc[m] += __shfl_xor(acc[m], 16, 64);
+        acc[m] += __shfl_xor(acc[m], 32, 64);
+      }
+      if (lane < 16 && n < N) {
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+          float v = __fmaf_rn((float)negzp_m[m], rs, acc[m] * 0.0625f);
+          v = __fmaf_rn(v, recip_m[m], bs);
+          v = fminf(fmaxf(v, -3.402823466e+38f), 3.402823466e+38f);
+          y[(size_t)m * N + n] = v;
+        }
       }
     }
   }
