@@ -90,6 +90,19 @@ int w4a32_unpack_native(const void* d_packed, int N, int K, uint8_t* d_u4, uint1
  * (tests/Arm/KaiLinearTest.hpp:355-361 unpack, :340 scale). */
 int w4a32_dequant(const void* d_packed, int N, int K, float* d_out, void* stream);
 
+/* PARITY UNPINNED. The weight blob that the reference's Arm quantizer stores in a .mllm file
+ * (KaiQuantizationPass.cpp:172-184: the output of kai_run_rhs_pack_nxk_qsi4c32p_qsu4c32s1s0 called
+ * at kai_linear.cpp:331-344) back to the native arrays of w4a32_repack_native(), so that such a
+ * file loads without re-quantising. nr, kr, sr are the tile's (nr 4 or 8; kr/sr 8 for the
+ * ...p4x8 / ...p8x8 tiles, 4 for ...p4x4). The packing routine is KleidiAI's, which the reference
+ * tree does not contain: the layout is restated from its published loop and checked only against
+ * this repository's own restatement (oracle/kai_blob.py).
+ * w4a32_kai_blob_bytes(): ceil(N/nr)*nr * (K/32 * 18 + 8), what quant_pack_rhs_size returns
+ * (kai_linear.cpp:302-309); 0 for an unsupported shape. d_bias may be NULL. */
+size_t w4a32_kai_blob_bytes(int N, int K, int nr);
+int w4a32_unpack_kai(const void* d_kai_blob, int N, int K, int nr, int kr, int sr, uint8_t* d_u4,
+                     uint16_t* d_scales, float* d_bias, void* stream);
+
 /* ---- online: one forward ------------------------------------------------------------ */
 
 /* Per-row asymmetric int8 quantisation of the activations into the workspace

@@ -42,6 +42,8 @@ ABI = {
     "w4a32_matmul_quantized_grouped": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a32_quant_lhs_norm": (_ci, [_vp, _vp, _vp, ctypes.c_float, _vp, _ci, _ci, _vp, _vp]),
     "w4a32_quant_lhs_silu_mul": (_ci, [_vp, _vp, _ci, _ci, _vp, _vp]),
+    "w4a32_kai_blob_bytes": (_sz, [_ci, _ci, _ci]),
+    "w4a32_unpack_kai": (_ci, [_vp, _ci, _ci, _ci, _ci, _ci, _vp, _vp, _vp, _vp]),
     "w4a32_splitk_scratch_bytes": (_sz, [_ci, _ci, _ci]),
     "w4a32_matmul_quantized_splitk": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a32_matmul": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
@@ -235,6 +237,18 @@ def quant_lhs_silu_mul(gate, up, ws=None):
     _check(lib().w4a32_quant_lhs_silu_mul(_ptr(gate), _ptr(up), M, K, _ptr(ws), _stream()),
            "w4a32_quant_lhs_silu_mul")
     return ws
+
+
+def unpack_kai(blob, N, K, nr, kr, sr):
+    """Blob of the reference's Arm quantizer (parity unpinned) -> native u4, bf16 scales, bias."""
+    import torch
+
+    u4 = torch.empty((N, K // 2), dtype=torch.uint8, device="cuda")
+    scales = torch.empty((N, K // 32), dtype=torch.int16, device="cuda")
+    bias = torch.empty((N,), dtype=torch.float32, device="cuda")
+    _check(lib().w4a32_unpack_kai(_ptr(blob), N, K, nr, kr, sr, _ptr(u4), _ptr(scales), _ptr(bias),
+                                  _stream()), "w4a32_unpack_kai")
+    return u4, scales, bias
 
 
 def export_lhs(ws, M, K):

@@ -91,6 +91,22 @@ int w4a32_unpack_native(const void* d_packed, int N, int K, uint8_t* d_u4, uint1
                                     d_bias, static_cast<hipStream_t>(stream)));
 }
 
+size_t w4a32_kai_blob_bytes(int N, int K, int nr) {
+  if (shape_ok(N, K) || (nr != 4 && nr != 8)) return 0;
+  return (size_t)((N + nr - 1) / nr) * nr * ((size_t)(K / 32) * 18 + 8);
+}
+
+int w4a32_unpack_kai(const void* d_kai_blob, int N, int K, int nr, int kr, int sr, uint8_t* d_u4,
+                     uint16_t* d_scales, float* d_bias, void* stream) {
+  if (int e = shape_ok(N, K)) return e;
+  if (!d_kai_blob || !d_u4 || !d_scales) return W4A32_EINVAL;
+  if ((nr != 4 && nr != 8) || sr <= 0 || kr <= 0 || kr % sr != 0) return W4A32_EINVAL;
+  const int seg = kr / sr;
+  if (seg != 4 && seg != 8 && seg != 16) return W4A32_EINVAL;  // a segment divides half a block
+  return from_hip(w4::launch_unpack_kai(static_cast<const uint8_t*>(d_kai_blob), N, K, nr, kr, sr, d_u4,
+                                        d_scales, d_bias, static_cast<hipStream_t>(stream)));
+}
+
 int w4a32_dequant(const void* d_packed, int N, int K, float* d_out, void* stream) {
   if (int e = shape_ok(N, K)) return e;
   if (!d_packed || !d_out) return W4A32_EINVAL;

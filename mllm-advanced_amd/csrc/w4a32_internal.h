@@ -17,6 +17,9 @@ hipError_t launch_repack(const uint8_t* u4, const uint16_t* scales, const float*
 hipError_t launch_unpack(const uint8_t* packed, int N, int K, uint8_t* u4, uint16_t* scales,
                          float* bias, hipStream_t s);
 hipError_t launch_dequant(const uint8_t* packed, int N, int K, float* out, hipStream_t s);
+// blob of the reference's Arm quantizer (KleidiAI packing, parity unpinned) -> native arrays
+hipError_t launch_unpack_kai(const uint8_t* blob, int N, int K, int nr, int kr, int sr, uint8_t* u4,
+                             uint16_t* scales, float* bias, hipStream_t s);
 
 // activations (every forward)
 hipError_t launch_quant_lhs(const float* x, int M, int K, int ldx, uint8_t* ws, hipStream_t s);

@@ -208,6 +208,50 @@ __global__ __launch_bounds__(64) void unpack_kernel(const uint8_t* __restrict__ 
   }
 }
 
+// [parity unpinned] The blob the reference's Arm quantizer stores (output of
+// kai_run_rhs_pack_nxk_qsi4c32p_qsu4c32s1s0, called at kai_linear.cpp:331-344) back to the native
+// arrays. KleidiAI is not part of the reference tree; the layout is restated from its published
+// packing loop: rows in groups of nr; per group and 32-block nr*16 data bytes, where byte i belongs
+// to segment i / (nr*seg), row (i / seg) % nr, position t = i % seg (seg = kr/sr), low nibble =
+// weight k = seg*segment + t of the block, high nibble = k + 16, the byte XORed with 0x88; then nr
+// bf16 scales; after the group's blocks nr f32 row sums (not used here) and nr f32 biases.
+// One thread per (row, block).
+__global__ __launch_bounds__(256) void unpack_kai_kernel(const uint8_t* __restrict__ blob, int N,
+                                                         int K, int nr, int seg,
+                                                         uint8_t* __restrict__ u4,
+                                                         uint16_t* __restrict__ scales,
+                                                         float* __restrict__ bias) {
+  const int nb = K / kBlockLen;
+  const long id = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= (long)N * nb) return;
+  const int n = (int)(id / nb), b = (int)(id % nb);
+  const int grp = n / nr, r = n % nr;
+  const size_t group_bytes = (size_t)nr * ((size_t)nb * 18 + 8);
+  const uint8_t* gbase = blob + (size_t)grp * group_bytes;
+  const uint8_t* data = gbase + (size_t)b * nr * 18;
+  uint8_t lo[16], hi[16];  // u4 at k = 0..15 and 16..31 of the block
+#pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    const int s = k / seg, t = k % seg;
+    const uint8_t v = data[(s * nr + r) * seg + t] ^ 0x88;
+    lo[k] = v & 0xF;
+    hi[k] = v >> 4;
+  }
+  uint8_t* dst = u4 + (size_t)n * (K / 2) + 16 * b;  // native: byte k/2, low nibble = even k
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    dst[i] = (uint8_t)(lo[2 * i] | (lo[2 * i + 1] << 4));
+    dst[8 + i] = (uint8_t)(hi[2 * i] | (hi[2 * i + 1] << 4));
+  }
+  const uint8_t* sp = data + nr * 16 + 2 * r;
+  scales[(size_t)n * nb + b] = (uint16_t)(sp[0] | (sp[1] << 8));
+  if (b == 0 && bias) {
+    const uint8_t* bp = gbase + (size_t)nb * nr * 18 + 4 * nr + 4 * r;
+    const uint32_t bits = bp[0] | (bp[1] << 8) | (bp[2] << 16) | ((uint32_t)bp[3] << 24);
+    bias[n] = __uint_as_float(bits);
+  }
+}
+
 __global__ __launch_bounds__(256) void copy_bias_kernel(const float* __restrict__ src, int N,
                                                         float* __restrict__ dst) {
   const int n = blockIdx.x * blockDim.x + threadIdx.x;
@@ -282,6 +326,14 @@ hipError_t launch_unpack(const uint8_t* packed, int N, int K, uint8_t* u4, uint1
   if (e != hipSuccess || !bias) return e;
   hipLaunchKernelGGL(copy_bias_kernel, dim3((N + 255) / 256), dim3(256), 0, s,
                      reinterpret_cast<const float*>(packed + g.bias_off), N, bias);
+  return hipGetLastError();
+}
+
+hipError_t launch_unpack_kai(const uint8_t* blob, int N, int K, int nr, int kr, int sr, uint8_t* u4,
+                             uint16_t* scales, float* bias, hipStream_t s) {
+  const long items = (long)N * (K / kBlockLen);
+  hipLaunchKernelGGL(unpack_kai_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, blob, N,
+                     K, nr, kr / sr, u4, scales, bias);
   return hipGetLastError();
 }
 

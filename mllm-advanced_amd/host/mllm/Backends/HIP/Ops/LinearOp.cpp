@@ -22,9 +22,20 @@ void checkHip(hipError_t e, const char* what) {
   if (e != hipSuccess) MLLM_ERROR_EXIT(kHipError, "%s failed: %s", what, hipGetErrorString(e));
 }
 
-// [KAI-recall, unpinned] size of the blob the reference's Arm quantizer writes for nr | N:
-// per row K/2 nibble bytes + K/32 bf16 scales + f32 row sum + f32 bias.
-size_t kleidiaiBlobBytes(int N, int K) { return (size_t)N * (K / 2 + K / 32 * 2 + 8); }
+// Packing parameters of the reference's six W4A32 tiles (ukernel table kai_linear.cpp:123-218): nr
+// from "qsi4c32p<nr>x..", kr / sr from the micro-kernel family (p4x8, p8x8: 16 / 2; p4x4: 8 / 2).
+// [parity unpinned: KleidiAI, which defines them, is not part of the reference tree]
+struct KaiTile {
+  int nr, kr, sr;
+};
+KaiTile kaiTile(LinearOpImplType t) {
+  switch (static_cast<int>(t)) {
+    case 4:
+    case 7: return {8, 16, 2};
+    case 8: return {4, 8, 2};
+    default: return {4, 16, 2};
+  }
+}
 
 }  // namespace
 
@@ -77,12 +88,22 @@ void HipLinearOp::load(const std::shared_ptr<ParameterLoader>& ploader) {
                                                       w4a32_native_scale_bytes(N, K));
     check(w4a32_repack_native(u4, sc, bias, N, K, packed.ptr<void>(), stream), "w4a32_repack_native");
     hb.synchronize();
-  } else if (weight_.dtype() == kInt8 && weight_.numel() == kleidiaiBlobBytes(N, K)) {
-    MLLM_ERROR_EXIT(kCoreError, "%s.weight looks like a KleidiAI-packed blob (%zu bytes). Its byte "
-                    "layout depends on the Arm tile and is not defined by the reference's own "
-                    "sources; re-quantize from the f32 model with this backend's quantizer.",
-                    name().c_str(), weight_.numel());
-    return;
+  } else if (const KaiTile kt = kaiTile(cargo_.impl_type_);
+             weight_.dtype() == kInt8 && weight_.numel() == w4a32_kai_blob_bytes(N, K, kt.nr)) {
+    // The blob the reference's Arm quantizer wrote for this tile (KaiQuantizationPass.cpp:172-184):
+    // un-interleave it to the native arrays, then repack. Its bias sits inside the blob (the
+    // file's <name>.bias is a 1-byte placeholder). Layout restated from KleidiAI: parity unpinned.
+    Tensor blob = toDevice(weight_);
+    const size_t u4_bytes = w4a32_native_u4_bytes(N, K), sc_bytes = w4a32_native_scale_bytes(N, K);
+    Tensor tmp = Tensor::empty({static_cast<int32_t>(u4_bytes + sc_bytes + (size_t)N * sizeof(float))},
+                               kInt8, kHIP).alloc();
+    uint8_t* u4 = tmp.ptr<uint8_t>();
+    auto* sc = reinterpret_cast<uint16_t*>(u4 + u4_bytes);
+    auto* bias = reinterpret_cast<float*>(u4 + u4_bytes + sc_bytes);
+    check(w4a32_unpack_kai(blob.ptr<void>(), N, K, kt.nr, kt.kr, kt.sr, u4, sc, bias, stream),
+          "w4a32_unpack_kai");
+    check(w4a32_repack_native(u4, sc, bias, N, K, packed.ptr<void>(), stream), "w4a32_repack_native");
+    hb.synchronize();
   } else {
     MLLM_ERROR_EXIT(kShapeError, "%s.weight: expected f32 [%d,%d] or an int8 W4 blob of %zu bytes, "
                     "got %s with %zu elements", name().c_str(), N, K, nativeBlobBytes(N, K),

@@ -16,8 +16,10 @@ class HipLinearOp final : public LinearOp {
   //   * kInt8 [bytes] in this build's row-major W4 format: out*in/2 nibble bytes, out*in/32 bf16
   //     scales, out f32 bias values (what quantizeLinearForFile() emits; the bias tensor in the
   //     file is then a 1-byte placeholder, as in the reference's quantised files).
-  // A blob in KleidiAI's packed layout (what the reference's Arm quantizer writes) is refused
-  // with an explanatory error.
+  //   * int8 [ceil(out/nr)*nr * (in/32 * 18 + 8)]: the blob the reference's Arm quantizer writes for
+  //     the op's tile (KleidiAI's packed layout, nr rows interleaved); it is un-interleaved on the
+  //     device and repacked. That layout is restated from KleidiAI's published packing loop, which
+  //     the reference tree does not contain: parity unpinned.
   void load(const std::shared_ptr<ParameterLoader>& ploader) override;
 
   void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;

@@ -189,6 +189,41 @@ static void testQuantizedFile(const char* dir) {
   EXPECT(maxAbsRel(y_b, ref) <= 1e-3);
 }
 
+// A file that holds, for three of the reference's tiles, the same quantised layer twice: as the blob
+// the reference's Arm quantizer would store (KleidiAI's interleaved layout, written by the python
+// restatement of that layout: parity unpinned) and as this backend's row-major blob. Both must load
+// to the same device weights: identical outputs.
+static void testKaiFile(const char* dir) {
+  const std::string path = std::string(dir) + "/kai_layers.mllm";
+  if (FILE* f = std::fopen(path.c_str(), "rb")) {
+    std::fclose(f);
+  } else {
+    std::printf("[ SKIP ] no %s\n", path.c_str());
+    return;
+  }
+  std::printf("[ RUN ] load blobs in the Arm quantizer's layout\n");
+  struct Case { int tile, N, K; };
+  const Case cases[] = {{5, 50, 256}, {7, 56, 96}, {8, 13, 64}, {3, 256, 1536}};
+  auto loaded = mllm::load(path);
+  const int M = 3;
+  for (const auto& c : cases) {
+    const auto impl = static_cast<LinearOpImplType>(c.tile);
+    auto op_k = makeLinear("kai" + std::to_string(c.tile), c.K, c.N, true, impl);
+    auto op_n = makeLinear("nat" + std::to_string(c.tile), c.K, c.N, true, impl);
+    op_k->load(loaded);
+    op_n->load(loaded);
+    auto x = normal((size_t)M * c.K, 1.0f, 40 + c.tile);
+    auto y_k = calculate(op_k, {M, c.K}, x, nullptr);
+    auto y_n = calculate(op_n, {M, c.K}, x, nullptr);
+    double mx = 0;
+    for (float v : y_n) mx = std::max(mx, (double)std::fabs(v));
+    std::printf("  tile %d N=%d K=%d: outputs %s, max |y| %.3g\n", c.tile, c.N, c.K,
+                y_k == y_n ? "identical" : "DIFFER", mx);
+    EXPECT(y_k == y_n);
+    EXPECT(mx > 0);
+  }
+}
+
 static void testImplTypeStrings() {
   std::printf("[ RUN ] implType strings\n");
   using C = LinearOpCargo;
@@ -222,9 +257,9 @@ static void testErrors() {
   expectThrow("missing parameter", [&] { makeLinear("nope", 64, 64, false)->load(params); });
   expectThrow("K % 32 != 0", [&] { makeLinear("a", 48, 64, false)->load(params); });
   expectThrow("wrong weight shape", [&] { makeLinear("a", 64, 32, false)->load(params); });
-  std::vector<int8_t> kai((size_t)64 * (64 / 2 + 64 / 32 * 2 + 8), 0);
-  params->insert("k.weight", hostTensor({(int32_t)kai.size()}, kInt8, kai.data()));
-  expectThrow("KleidiAI-packed blob", [&] { makeLinear("k", 64, 64, false)->load(params); });
+  std::vector<int8_t> odd((size_t)64 * (64 / 2 + 64 / 32 * 2 + 8) + 3, 0);
+  params->insert("k.weight", hostTensor({(int32_t)odd.size()}, kInt8, odd.data()));
+  expectThrow("int8 blob of no known size", [&] { makeLinear("k", 64, 64, false)->load(params); });
   expectThrow("forward before load", [&] {
     auto op = makeLinear("a", 64, 64, false);
     std::vector<float> x(64, 1.0f);
@@ -252,6 +287,7 @@ int main(int argc, char** argv) {
   testReferenceProtocol();
   testFromF32File(dir);
   testQuantizedFile(dir);
+  testKaiFile(dir);
   hip::currentHipBackend().synchronize();
   ctx.shutdown();
   std::printf(g_failed ? "[ FAILED ] %d expectation(s)\n" : "[ PASSED ]%.0d\n", g_failed);

@@ -38,6 +38,37 @@ def test_cpp_operator_tests_pass(tmp_path):
 
 
 @pytest.mark.gpu
+def test_cpp_operator_loads_the_arm_quantizers_blob(tmp_path):
+    """Writes a .mllm file that holds each test layer twice: as the interleaved blob the reference's
+    Arm quantizer stores (python restatement of KleidiAI's packing: parity unpinned) and as this
+    backend's row-major blob; the C++ test loads both through HipLinearOp::load and demands identical
+    outputs."""
+    import numpy as np
+
+    import kai_blob
+    from mllm_file import write
+
+    params = {}
+    rng = np.random.default_rng(5)
+    for tile, N, K in [(5, 50, 256), (7, 56, 96), (8, 13, 64), (3, 256, 1536)]:
+        nr, kr, sr = kai_blob.TILE_PARAMS[tile]
+        u4 = rng.integers(0, 256, size=(N, K // 2), dtype=np.uint8)
+        scales = ((rng.standard_normal((N, K // 32)) * 0.01).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+        bias = rng.standard_normal(N).astype(np.float32)
+        params[f"kai{tile}.weight"] = kai_blob.pack(u4, scales, bias, nr, kr, sr).view(np.int8)
+        params[f"kai{tile}.bias"] = np.zeros(1, dtype=np.int8)          # KaiQuantizationPass.cpp:180-184
+        native = np.concatenate([u4.ravel(), scales.ravel().view(np.uint8), bias.view(np.uint8)])
+        params[f"nat{tile}.weight"] = native.view(np.int8)
+        params[f"nat{tile}.bias"] = np.zeros(1, dtype=np.int8)
+    write(os.path.join(str(tmp_path), "kai_layers.mllm"), "kai-blobs", params)
+    out = subprocess.run([BIN, str(tmp_path)], capture_output=True, text=True, timeout=300)
+    print(out.stdout[-3000:])
+    print(out.stderr[-2000:])
+    assert out.returncode == 0 and "[ PASSED ]" in out.stdout
+    assert out.stdout.count("outputs identical") == 4 and "[ SKIP ]" not in out.stdout
+
+
+@pytest.mark.gpu
 def test_cpp_model_generates_what_the_oracle_generates(tmp_path):
     """The C++ model class writes a tiny Qwen2-shaped .mllm file under the reference's parameter
     names, loads it and generates greedily (prefill in two slices, first step eager, the rest from a
