@@ -303,8 +303,9 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(const float* __re
 // needs a transpose.
 // ---------------------------------------------------------------------------------------------
 typedef float v16f32 __attribute__((ext_vector_type(16)));
-constexpr int kPfWaves = 4;
-
+// kPfWaves wavefronts per workgroup: 4, or 8 for long prompts (two wavefronts per SIMD overlap each
+// other's loads and dependent MFMA chains; the merge area then takes 118 KB of LDS).
+template <int kPfWaves>
 __global__ __launch_bounds__(64 * kPfWaves) void attention_prefill_mfma_kernel(
     const float* __restrict__ q, const float* __restrict__ kc, const float* __restrict__ vc,
     float* __restrict__ out, int M, int Hq, int Hkv, int max_seq, const int* __restrict__ d_pos0,
@@ -860,10 +861,23 @@ hipError_t launch_attention_prefill(const float* q, const float* kc, const float
                                     int M, int Hq, int Hkv, int max_seq, const int* d_pos0, int pos0,
                                     hipStream_t s) {
   const float scale = 1.0f / sqrtf((float)kHeadDim);
-  if (M >= 16) {  // matrix-core kernel: 32 queries per workgroup
-    const size_t lds = sizeof(float) * (kPfWaves - 1) * 66 * 64;
-    hipLaunchKernelGGL(attention_prefill_mfma_kernel, dim3(Hq, (M + 31) / 32), dim3(64 * kPfWaves), lds, s,
-                       q, kc, vc, out, M, Hq, Hkv, max_seq, d_pos0, pos0, scale);
+  if (M >= 256) {  // matrix-core kernel, 32 queries per workgroup; many key blocks: 8 wavefronts
+    constexpr int W = 8;
+    const size_t lds = sizeof(float) * (W - 1) * 66 * 64;
+    static bool raised = false;
+    if (!raised) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_prefill_mfma_kernel<W>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return e;
+      raised = true;
+    }
+    hipLaunchKernelGGL(attention_prefill_mfma_kernel<W>, dim3(Hq, (M + 31) / 32), dim3(64 * W), lds, s, q,
+                       kc, vc, out, M, Hq, Hkv, max_seq, d_pos0, pos0, scale);
+  } else if (M >= 16) {
+    constexpr int W = 4;
+    const size_t lds = sizeof(float) * (W - 1) * 66 * 64;
+    hipLaunchKernelGGL(attention_prefill_mfma_kernel<W>, dim3(Hq, (M + 31) / 32), dim3(64 * W), lds, s, q,
+                       kc, vc, out, M, Hq, Hkv, max_seq, d_pos0, pos0, scale);
   } else {
     hipLaunchKernelGGL(attention_prefill_kernel, dim3(Hq, M), dim3(64), 0, s, q, kc, vc, out, Hq, Hkv,
                        max_seq, d_pos0, pos0, scale);

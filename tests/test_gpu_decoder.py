@@ -137,7 +137,8 @@ def test_attention_prefill_and_decode(pkg, Hq, Hkv):
             o = torch.nn.functional.scaled_dot_product_attention(tq, tk, tv, attn_mask=mask)
         return o[0].permute(1, 0, 2).reshape(M, Hq * D)
 
-    for M, pos0 in [(1, 0), (5, 0), (70, 0), (33, 100), (130, 0)]:
+    # 16 rows and more run on the matrix cores, 256 and more with 8 wavefronts per workgroup
+    for M, pos0 in [(1, 0), (5, 0), (70, 0), (33, 100), (130, 0), (256, 0), (300, 200), (512, 512)]:
         q = torch.randn((M, Hq * D), generator=g, device="cuda")
         out = pkg.op_attention(q, kc, vc, Hq, Hkv, D, pos0)
         assert max_abs_rel(out.cpu().numpy(), ref(q, pos0).cpu().numpy()) < 2e-5, (M, pos0)
