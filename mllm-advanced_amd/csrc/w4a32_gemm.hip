@@ -175,7 +175,7 @@ struct GemmGroup {
   int nb_first[kMaxGemmGroup + 1];  // entries past the last Linear hold the total
 };
 
-template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH, int OCC, int MODE>
+template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH, int OCC, int MODE, int BE>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
     float* __restrict__ y_arg, const _Float16* __restrict__ ah, const float* __restrict__ recip,
     const uint8_t* __restrict__ packed_arg, const uint8_t* __restrict__ hscale_arg,
@@ -184,7 +184,11 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
     const GemmGroup grp) {
   constexpr bool GROUPED = MODE == kModeGrouped, SPLITK = MODE == kModeSplitK;
   constexpr int D = DEPTH;
-  static_assert(D % 2 == 0, "stage s uses LDS buffer s & 1: the unrolled ring must keep that parity");
+  // BE = stages per barrier (1 or 2). The loop is unrolled U stages at a time so that ring slots and
+  // LDS buffers are compile-time constants.
+  static_assert(BE == 1 || (BE == 2 && D == 2), "two stages per barrier are built for a ring of two");
+  constexpr int U = BE == 2 ? 4 : D;
+  static_assert(U % (2 * BE) == 0, "the unrolled stages must cover whole pairs of LDS buffer sets");
   constexpr int NWAVES = WAVES_M * WAVES_N;
   constexpr int BM = 32 * WM * WAVES_M;
   constexpr int BN32 = WN * WAVES_N;           // 32-column fragments per workgroup and k-slice
@@ -197,9 +201,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
   constexpr int kMfma = SL * WM * WN;          // products per wavefront and stage
   constexpr int NDW = 2 * B_UNITS;             // packed dwords a thread dequantises per stage
   constexpr int NSTEP = 4 * NDW;               // in four steps each
-  static_assert(2 * kBufBytes <= 65536, "static LDS");
+  constexpr int kLdsBufs = 2 * BE;             // two sets (read / being written) of BE stage buffers
+  static_assert(kLdsBufs * kBufBytes <= 65536, "static LDS");
 
-  __shared__ __align__(16) uint8_t sB[2 * kBufBytes];
+  __shared__ __align__(16) uint8_t sB[kLdsBufs * kBufBytes];
 
   const int t = threadIdx.x;
   const int lane = t & 63;
@@ -328,26 +333,33 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
   // wait in the loop from the fewest loads that can be younger than the one it needs on any way
   // into the loop, so a prologue with another order makes the loop wait for newer loads than it
   // uses.
+  // B runs BE stages ahead of the products: the first BE stages go to the first buffer set here, and
+  // ring slot p holds stage p + BE.
   {
-    uint2 q0[B_UNITS];
-    uint32_t s0[B_UNITS];
-    load_b(s_begin, q0, s0);
+    uint2 q0[BE][B_UNITS];
+    uint32_t s0[BE][B_UNITS];
+#pragma unroll
+    for (int e = 0; e < BE; ++e) load_b(s_begin + e, q0[e], s0[e]);
 #pragma unroll
     for (int p = 0; p < D; ++p) {
-      load_b(s_begin + p + 1, breg[p], sreg[p]);  // ring slot p holds the stage after slot p's A
+      load_b(s_begin + p + BE, breg[p], sreg[p]);
 #pragma unroll
       for (int kbl = 0; kbl < AKB; ++kbl) load_a_kb(s_begin + p, kbl, areg[p]);
     }
     __builtin_amdgcn_sched_barrier(0);
     const h2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
 #pragma unroll
-    for (int u = 0; u < B_UNITS; ++u) {
-      const h2 s2 = __builtin_bit_cast(h2, s0[u]);
-      const h2 s2_16 = s2 * sixteenth;
-      *reinterpret_cast<uint4*>(frag_ptr(0, u, 0)) =
-          dequant8(q0[u].x, h2{s2[0], s2[0]}, h2{s2_16[0], s2_16[0]});
-      *reinterpret_cast<uint4*>(frag_ptr(0, u, 1)) =
-          dequant8(q0[u].y, h2{s2[1], s2[1]}, h2{s2_16[1], s2_16[1]});
+    for (int e = 0; e < BE; ++e) {
+      const uint32_t keep = s_begin + e < nstages ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+      for (int u = 0; u < B_UNITS; ++u) {
+        const h2 s2 = __builtin_bit_cast(h2, s0[e][u] & keep);
+        const h2 s2_16 = s2 * sixteenth;
+        *reinterpret_cast<uint4*>(frag_ptr(e, u, 0)) =
+            dequant8(q0[e][u].x, h2{s2[0], s2[0]}, h2{s2_16[0], s2_16[0]});
+        *reinterpret_cast<uint4*>(frag_ptr(e, u, 1)) =
+            dequant8(q0[e][u].y, h2{s2[1], s2[1]}, h2{s2_16[1], s2_16[1]});
+      }
     }
   }
 
@@ -359,37 +371,49 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
   // wavefront dequantises the next stage's weights, a few instructions at a time, and issues its
   // LDS and global traffic in the gaps between its own products. (Left to the scheduler, all of a
   // stage's dequantisation ran first and the products after it.)
-  for (int s_base = s_begin; s_base < nstages; s_base += D) {
+  //
+  // With BE = 2 the barrier comes every second stage (four LDS buffers): the stage behind it finds its
+  // first fragments requested under the previous stage's last products, and a lone workgroup on a CU
+  // pays the barrier and that LDS round trip half as often.
+  h8 bf[2][WN];
+  for (int s_base = s_begin; s_base < nstages; s_base += U) {
 #pragma unroll
-    for (int u = 0; u < D; ++u) {
+    for (int u = 0; u < U; ++u) {
       const int s = s_base + u;
-      __syncthreads();
-      const uint8_t* bbuf = sB + (u & 1) * kBufBytes + 16 * lane;
-      h8 bf[2][WN];
+      constexpr int kSlotMask = D - 1;
+      static_assert((D & (D - 1)) == 0, "ring slot = stage mod D by masking");
+      const int slot = u & kSlotMask;
+      const int rbuf = ((u / BE) & 1) * BE + u % BE;                    // buffer this stage reads
+      const int wbuf = (((u + BE) / BE) & 1) * BE + (u + BE) % BE;      // buffer of stage s + BE
+      const uint8_t* bbuf = sB + rbuf * kBufBytes + 16 * lane;
+      if (u % BE == 0) {
+        __syncthreads();
 #pragma unroll
-      for (int b = 0; b < WN; ++b)
-        bf[0][b] = *reinterpret_cast<const h8*>(bbuf + (wn * WN + b) * 1024);
-      __builtin_amdgcn_sched_barrier(0);  // requested first: their latency covers what follows
-      // Inputs of the dequantisation (stage s+1, ring slot u) move to temporaries, which frees the
-      // slot for its next load. A stage past the end (loaded from clamped addresses) gets scale 0.
+        for (int b = 0; b < WN; ++b)
+          bf[0][b] = *reinterpret_cast<const h8*>(bbuf + (wn * WN + b) * 1024);
+        __builtin_amdgcn_sched_barrier(0);  // requested first: their latency covers what follows
+      }
+      // Inputs of the dequantisation (stage s + BE, in this stage's ring slot) move to temporaries,
+      // which frees the slot for its next load. A stage past the end (loaded from clamped addresses)
+      // gets scale 0.
       uint32_t dx[NDW];
       h2 dsc[NDW], dsc16[NDW];
       {
-        const uint32_t keep = s + 1 < nstages ? 0xFFFFFFFFu : 0u;
+        const uint32_t keep = s + BE < nstages ? 0xFFFFFFFFu : 0u;
         const h2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
 #pragma unroll
         for (int q = 0; q < B_UNITS; ++q) {
-          const h2 s2 = __builtin_bit_cast(h2, sreg[u][q] & keep);
+          const h2 s2 = __builtin_bit_cast(h2, sreg[slot][q] & keep);
           const h2 s2_16 = s2 * sixteenth;
           dsc[2 * q] = h2{s2[0], s2[0]};
           dsc16[2 * q] = h2{s2_16[0], s2_16[0]};
           dsc[2 * q + 1] = h2{s2[1], s2[1]};
           dsc16[2 * q + 1] = h2{s2_16[1], s2_16[1]};
-          dx[2 * q] = breg[u][q].x ^ 0x88888888u;  // two's complement nibbles -> offset-8 nibbles
-          dx[2 * q + 1] = breg[u][q].y ^ 0x88888888u;
+          dx[2 * q] = breg[slot][q].x ^ 0x88888888u;  // two's complement nibbles -> offset-8 nibbles
+          dx[2 * q + 1] = breg[slot][q].y ^ 0x88888888u;
         }
       }
-      load_b(s + 1 + D, breg[u], sreg[u]);
+      load_b(s + BE + D, breg[slot], sreg[slot]);
       __builtin_amdgcn_sched_barrier(0);
       // dequant8() cut into four steps per dword d (unit d / 2, scale block d % 2)
       h2 dp[NDW];
@@ -412,7 +436,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
           dout[d].z = __builtin_bit_cast(uint32_t, (p2 - b1) * dsc[d]);
         } else {
           dout[d].w = __builtin_bit_cast(uint32_t, (dp[d] - b16) * dsc16[d]);
-          *reinterpret_cast<uint4*>(frag_ptr((u + 1) & 1, d >> 1, d & 1)) = dout[d];
+          *reinterpret_cast<uint4*>(frag_ptr(wbuf, d >> 1, d & 1)) = dout[d];
         }
       };
       int mi = 0;
@@ -423,18 +447,20 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
 #pragma unroll
           for (int a = 0; a < WM; ++a) {
             acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                __builtin_bit_cast(h8, areg[u][sl >> 1][a][sl & 1]), bf[sl & 1][b], acc[a][b], 0, 0,
-                0);
+                __builtin_bit_cast(h8, areg[slot][sl >> 1][a][sl & 1]), bf[sl & 1][b], acc[a][b], 0,
+                0, 0);
             if (sl < SL - 1 && a == 0)  // the next slice's fragment b, one read per product
               bf[(sl + 1) & 1][b] =
                   *reinterpret_cast<const h8*>(bbuf + ((sl + 1) * BN32 + wn * WN + b) * 1024);
+            if (sl == SL - 1 && a == 0 && (u + 1) % BE != 0)  // no barrier ahead: the next stage's first
+              bf[0][b] = *reinterpret_cast<const h8*>(bbuf + kBufBytes + (wn * WN + b) * 1024);
 #pragma unroll
             for (int st = mi * NSTEP / kMfma; st < (mi + 1) * NSTEP / kMfma; ++st) dq_step(st);
             ++mi;
             __builtin_amdgcn_sched_barrier(0);
           }
         }
-        if (sl & 1) load_a_kb(s + D, sl >> 1, areg[u]);  // that k-block's registers are free now
+        if (sl & 1) load_a_kb(s + D, sl >> 1, areg[slot]);  // that k-block's registers are free now
       }
     }
   }
@@ -532,7 +558,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(
 
 // One Linear (group == nullptr) or the Linears of `group`, whose column blocks add up to nb_total.
 // ksplit > 1: the stages of every tile are dealt to ksplit workgroups (partial sums in `part`).
-template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH, int OCC>
+template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH, int OCC, int BE = 1>
 static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                              const GemmGroup* group, const int* group_N, int count, int ksplit,
                              float* part, hipStream_t s) {
@@ -554,7 +580,7 @@ static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed,
     }
     const int NB = nb;
     const int n_major = (double)M * 2.0 <= (double)n_total * 0.5625 ? 1 : 0;
-    hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModeGrouped>),
+    hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModeGrouped, BE>),
                        dim3(((MB * NB + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N), 0, s, nullptr, ah,
                        recip, nullptr, nullptr, nullptr, nullptr, M, 0, K, 0,
                        weight_geom(group_N[0], K).KC, MB, NB, n_major, 1, nullptr, g);
@@ -568,7 +594,7 @@ static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed,
   const float* rowmul = reinterpret_cast<const float*>(packed + g.rowmul_off);
   const float* bias = reinterpret_cast<const float*>(packed + g.bias_off);
   if (ksplit > 1) {
-    hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModeSplitK>),
+    hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModeSplitK, BE>),
                        dim3(((MB * NB * ksplit + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N), 0, s, y, ah,
                        recip, packed, packed + g.hscale_off, rowmul, bias, M, N, K, g.NT, g.KC, MB, NB,
                        n_major, ksplit, part, GemmGroup{});
@@ -583,7 +609,7 @@ static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed,
     }
     return hipGetLastError();
   }
-  hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModePlain>),
+  hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModePlain, BE>),
                      dim3(((MB * NB + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N), 0, s, y, ah, recip,
                      packed, packed + g.hscale_off, rowmul, bias, M, N, K, g.NT, g.KC, MB, NB, n_major,
                      1, nullptr, GemmGroup{});
@@ -610,6 +636,8 @@ static hipError_t launch_gemm_i8(float* y, const uint8_t* ws, const uint8_t* pac
 //   1: 128 x  64, 4 wavefronts of 32 x 64
 //   2: 128 x 128, 4 wavefronts of 32 x 128, three workgroups per CU
 //   3: 256 x 128, 4 wavefronts of 64 x 128 (each B fragment feeds two products)
+//   4: 128 x  64 with one barrier per two stages (long K, few tiles: 12-15 % over shape 1; on the
+//      128 x 128 tile the same change measured no gain)
 static hipError_t launch_f16_tile(int tile, float* y, const uint8_t* ws, const uint8_t* packed, int M,
                                   int K, int N, const GemmGroup* group, const int* group_N, int count,
                                   int ksplit, float* part, hipStream_t s) {
@@ -622,13 +650,15 @@ static hipError_t launch_f16_tile(int tile, float* y, const uint8_t* ws, const u
       return launch_f16<4, 1, 1, 4, 2, 3>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
     case 3:
       return launch_f16<4, 1, 2, 4, 2, 1>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
+    case 4:
+      return launch_f16<4, 1, 1, 2, 2, 3, 2>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
   }
   return hipErrorInvalidValue;
 }
 
 static int choose_f16_tile(long tiles, int K) {
   if (tiles < 64 && K >= 4096) return 0;
-  if (tiles < 160) return 1;
+  if (tiles < 160) return K >= 4096 ? 4 : 1;
   if (tiles < 2048) return 2;
   return 3;
 }
