@@ -28,6 +28,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the decode pass, measured with hardware counters (not re-measured by a
+# bench run: the counters need the profiler); algorithmic bytes per launch are 7,732,011.
+PASS_TRAFFIC_BYTES_PER_LAUNCH = 7_993_476
 LAYERS = 28
 # name, K, N, bias, count per layer
 LAYER_LINEARS = [
@@ -207,7 +210,10 @@ def main():
     roof_bytes = step_bytes / n_launch
     achieved = roof_bytes / (roof_avg_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": PASS_TRAFFIC_BYTES_PER_LAUNCH,
+                "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over this pass's 113 launches "
+                                  "(3889.3 / 27.6 KiB per dispatch), scaled x2.00 / x1.00 by the same counters' "
+                                  "reading for a 256 MiB copy; profiles/traffic_fetch_write_decode_prefill.md",
                 "kernel": "gemv_fused_kernel<1,R> (R=1 for K=1536, R=2 for K=8960); lm_head runs "
                           "gemv_wide_kernel<1,true>",
                 "launches_per_step": n_launch, "avg_launch_us": round(roof_avg_us, 3),
