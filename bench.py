@@ -561,7 +561,16 @@ def main():
                                "gate,up) are issued as one grouped call",
                    "M": 1, "linears": len(step_linears), "launches": n_launch,
                    "algorithmic_bytes_per_step": step_bytes},
-        "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
+        "roofline": roofline, "cpu_baseline": cpu,
+        # the other two figures the headline metric names, measured in the same run (details in extra)
+        "also": {"prefill_gemm_TFLOPs_M512_gate_proj": (extra.get("prefill_roofline") or {}).get(
+                     "M512_gate_proj_kernel_TFLOPs"),
+                 "prefill_layer_TFLOPs_M512_as_issued": ((extra.get("prefill") or {}).get("M512") or {}).get(
+                     "layer_as_issued_TFLOPs"),
+                 "decoder_tokens_per_s_batch1": (extra.get("decoder_config4") or {}).get("decode_tokens_per_s"),
+                 "decoder_prefill_tokens_per_s_512": (extra.get("decoder_config4") or {}).get(
+                     "prefill_tokens_per_s")},
+        "extra": extra,
     }
     print(json.dumps(out))
 
