@@ -187,7 +187,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
   // BE = stages per barrier (1 or 2). The loop is unrolled U stages at a time so that ring slots and
   // LDS buffers are compile-time constants.
   static_assert(BE == 1 || (BE == 2 && D == 2), "two stages per barrier are built for a ring of two");
-  constexpr int U = BE == 2 ? 4 : D;
+  constexpr int U = BE == 2 ? 4 : (D < 2 ? 2 : D);
   static_assert(U % (2 * BE) == 0, "the unrolled stages must cover whole pairs of LDS buffer sets");
   constexpr int NWAVES = WAVES_M * WAVES_N;
   constexpr int BM = 32 * WM * WAVES_M;
@@ -635,7 +635,9 @@ static hipError_t launch_gemm_i8(float* y, const uint8_t* ws, const uint8_t* pac
 //   0:  64 x  64, 4 wavefronts of 32 x 32, 8 stages of loads in flight
 //   1: 128 x  64, 4 wavefronts of 32 x 64
 //   2: 128 x 128, 4 wavefronts of 32 x 128, three workgroups per CU
-//   3: 256 x 128, 4 wavefronts of 64 x 128 (each B fragment feeds two products)
+//   3: 256 x 128, 4 wavefronts of 64 x 128 (each B fragment feeds two products: half the LDS reads
+//      per product), loads one stage ahead only, which keeps it at 224 registers: two workgroups
+//      per CU (with two stages ahead and one workgroup per CU it never beat shape 2)
 //   4: 128 x  64 with one barrier per two stages (long K, few tiles: 12-15 % over shape 1; on the
 //      128 x 128 tile the same change measured no gain)
 static hipError_t launch_f16_tile(int tile, float* y, const uint8_t* ws, const uint8_t* packed, int M,
@@ -649,7 +651,7 @@ static hipError_t launch_f16_tile(int tile, float* y, const uint8_t* ws, const u
     case 2:
       return launch_f16<4, 1, 1, 4, 2, 3>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
     case 3:
-      return launch_f16<4, 1, 2, 4, 2, 1>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
+      return launch_f16<4, 1, 2, 4, 1, 2>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
     case 4:
       return launch_f16<4, 1, 1, 2, 2, 3, 2>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
   }
@@ -659,17 +661,18 @@ static hipError_t launch_f16_tile(int tile, float* y, const uint8_t* ws, const u
 static int choose_f16_tile(long tiles, int K) {
   if (tiles < 64 && K >= 4096) return 0;
   if (tiles < 160) return K >= 4096 ? 4 : 1;
-  if (tiles < 2048) return 2;
-  return 3;
+  if (tiles >= 1400 || (K >= 4096 && tiles >= 320)) return 3;
+  return 2;
 }
 
 // Choice of tile shape, measured on MI355X at M = 128..8192 over the decoder and ViT shapes, by
 // the number of 128 x 128 tiles the problem has. A stage of 64 k costs a lone workgroup about the
-// same time whatever its tile size (barrier, first LDS round trip, dequantisation), so problems
-// with fewer tiles than CUs take the smaller tile and put two workgroups on a CU; with very
-// few tiles and a long K the 64 x 64 tile's four-fold workgroup count wins. From about one tile per
-// CU on, 128 x 128 with three resident workgroups per CU is best; with many tiles per CU the
-// 256 x 128 tile, which reads each B fragment from LDS once for two products.
+// same time whatever its tile size, so problems with fewer tiles than CUs take the smaller tile and
+// put two workgroups on a CU; with very few tiles and a long K the 64 x 64 tile's four-fold
+// workgroup count wins. From about one tile per CU on, 128 x 128 with three resident workgroups per
+// CU is best, but there LDS bandwidth bounds it (each B fragment feeds one product); with many
+// tiles per CU (gate_proj from M = 3072 on, down_proj from 4096 on) the 256 x 128 tile is 10-17 %
+// faster (gate_proj at M = 8192: 270 -> 227 us, 1.0 PFLOP/s).
 hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                        int kernel, hipStream_t s) {
   if (kernel == kKernelGemmI8 || (kernel == kKernelAuto && M <= 32)) {
