@@ -175,8 +175,8 @@ struct GemmGroup {
   int nb_first[kMaxGemmGroup + 1];  // entries past the last Linear hold the total
 };
 
-template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH, int OCC, int MODE, int BE>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
+template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH, int OCC, int MODE, int BE, int WK>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_kernel(
     float* __restrict__ y_arg, const _Float16* __restrict__ ah, const float* __restrict__ recip,
     const uint8_t* __restrict__ packed_arg, const uint8_t* __restrict__ hscale_arg,
     const float* __restrict__ rowmul_arg, const float* __restrict__ bias_arg, int M, int N_arg, int K,
@@ -189,27 +189,37 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
   static_assert(BE == 1 || (BE == 2 && D == 2), "two stages per barrier are built for a ring of two");
   constexpr int U = BE == 2 ? 4 : (D < 2 ? 2 : D);
   static_assert(U % (2 * BE) == 0, "the unrolled stages must cover whole pairs of LDS buffer sets");
-  constexpr int NWAVES = WAVES_M * WAVES_N;
+  static_assert(WK == 1 || (WK == 2 && WM == 1), "k-halves: built for one 32-row block per wavefront");
+  constexpr int NWAVES = WAVES_M * WAVES_N * WK;
   constexpr int BM = 32 * WM * WAVES_M;
   constexpr int BN32 = WN * WAVES_N;           // 32-column fragments per workgroup and k-slice
   constexpr int WNT = 2 * BN32;                // 16-row weight tile rows per workgroup
-  static_assert(WNT % NWAVES == 0, "each wavefront dequantises WNT/NWAVES tile rows per stage");
-  constexpr int B_UNITS = WNT / NWAVES;        // 8-byte pieces of packed B per thread per stage
+  // Wavefront w dequantises tile rows w, w + NWAVES, ... of the stage. When that does not come out even,
+  // the surplus units repeat a valid row's loads and write to a spare fragment nobody reads.
+  constexpr int B_UNITS = (WNT + NWAVES - 1) / NWAVES;  // 8-byte pieces of packed B per thread per stage
+  constexpr bool kSpareUnits = WNT % NWAVES != 0;
   constexpr int kBufBytes = 4 * BN32 * 1024;   // one B stage: [4 k-slices][BN32 fragments]
-  constexpr int SL = 4;                        // k-slices of a stage
-  constexpr int AKB = 2;                       // activation k-blocks (32 k) of a stage
+  constexpr int SL = 4 / WK;                   // k-slices of a stage that one wavefront multiplies
+  constexpr int AKB = 2 / WK;                  // activation k-blocks (32 k) of a stage, likewise
   constexpr int kMfma = SL * WM * WN;          // products per wavefront and stage
   constexpr int NDW = 2 * B_UNITS;             // packed dwords a thread dequantises per stage
   constexpr int NSTEP = 4 * NDW;               // in four steps each
   constexpr int kLdsBufs = 2 * BE;             // two sets (read / being written) of BE stage buffers
-  static_assert(kLdsBufs * kBufBytes <= 65536, "static LDS");
+  constexpr int kSpareOff = kLdsBufs * kBufBytes;
+  constexpr int kLdsBytes = kSpareOff + (kSpareUnits ? 1024 : 0);
+  static_assert(kLdsBytes <= 65536, "static LDS");
+  static_assert(WK == 1 || kSpareOff >= NWAVES * 4096, "the k-halves meet through the stage buffers");
 
-  __shared__ __align__(16) uint8_t sB[kLdsBufs * kBufBytes];
+  __shared__ __align__(16) uint8_t sB[kLdsBytes];
 
   const int t = threadIdx.x;
   const int lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // scalar: what derives from it is too
-  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  // WK = 2: wavefronts wave and wave + NWAVES/2 own the same outputs and each take one 32-k block of
+  // every stage (two wavefronts per SIMD when the workgroup has a CU to itself; their sums meet in LDS
+  // after the loop).
+  const int wk = wave / (WAVES_M * WAVES_N);
+  const int wm = (wave % (WAVES_M * WAVES_N)) / WAVES_N, wn = wave % WAVES_N;
   const int g = lane >> 4, j = lane & 15;     // position inside a weight tile
   const int h = lane >> 5, i32 = lane & 31;   // position inside an MFMA operand / C tile
   // Workgroup -> tile. The hardware deals consecutive workgroups round-robin to the 8 XCDs, each
@@ -276,7 +286,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
   const uint8_t* bs_ptr[B_UNITS];
 #pragma unroll
   for (int u = 0; u < B_UNITS; ++u) {
-    int nt = nt0 + wave + NWAVES * u;
+    int ntl = wave + NWAVES * u;
+    ntl = ntl < WNT ? ntl : WNT - 1;  // a surplus unit
+    int nt = nt0 + ntl;
     nt = nt < NT ? nt : NT - 1;  // tile rows past the matrix: their columns are never stored
     bq_ptr[u] = packed + (size_t)nt * KC * kTileBytes + 16 * lane;
     bs_ptr[u] = hscale + (size_t)nt * KC * kTileScaleBytes + 8 * j;
@@ -289,7 +301,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
   // pad every weight tile (k >= K).
   auto load_a_kb = [&](int s, int kbl, uint4 (&dst)[AKB][WM][2]) {
     const int sc = s < nstages ? s : nstages - 1;
-    int blk = 2 * sc + kbl;
+    int blk = 2 * sc + (WK == 2 ? wk : kbl);
     blk = blk < KB ? blk : KB - 1;
     const int off = blk * 2048;
 #pragma unroll
@@ -317,7 +329,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
   auto frag_ptr = [&](int buf, int unit, int dd) {
     const int ntl = wave + NWAVES * unit;
     const int op_lane = 32 * (g >> 1) + 16 * (ntl & 1) + j;
-    return sB + buf * kBufBytes + ((2 * dd + (g & 1)) * BN32 + (ntl >> 1)) * 1024 + 16 * op_lane;
+    const int off = buf * kBufBytes + ((2 * dd + (g & 1)) * BN32 + (ntl >> 1)) * 1024;
+    return sB + (kSpareUnits && ntl >= WNT ? kSpareOff : off) + 16 * op_lane;
   };
 
   v16f acc[WM][WN];
@@ -385,7 +398,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
       const int slot = u & kSlotMask;
       const int rbuf = ((u / BE) & 1) * BE + u % BE;                    // buffer this stage reads
       const int wbuf = (((u + BE) / BE) & 1) * BE + (u + BE) % BE;      // buffer of stage s + BE
-      const uint8_t* bbuf = sB + rbuf * kBufBytes + 16 * lane;
+      const uint8_t* bbuf = sB + rbuf * kBufBytes + 16 * lane + (WK == 2 ? wk * (SL * BN32 * 1024) : 0);
       if (u % BE == 0) {
         __syncthreads();
 #pragma unroll
@@ -465,6 +478,51 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
     }
   }
 
+  // WK = 2: the two k-halves of an output block meet in LDS, one 32 x 32 block per wavefront and round
+  // (4 KiB each, in the stage buffers). The first half keeps column blocks 0..BH-1 and hands over the
+  // rest, the second half the other way round; every sum is (first half) + (second half).
+  constexpr int BH = WK == 2 ? (WN + 1) / 2 : WN;
+  if constexpr (WK == 2) {
+    float* xmine = reinterpret_cast<float*>(sB) + wave * 1024 + 4 * lane;
+    const float* xpeer = reinterpret_cast<const float*>(sB) + (wave ^ (NWAVES / 2)) * 1024 + 4 * lane;
+#pragma unroll
+    for (int r = 0; r < BH; ++r) {
+      const int give0 = BH + r < WN ? BH + r : WN - 1;  // block the first half hands over in this round
+      __syncthreads();  // the loop's (then the previous round's) reads of these bytes are over
+      if (wk == 0) {
+        if (BH + r < WN) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            *reinterpret_cast<float4*>(xmine + 256 * q) = make_float4(
+                acc[0][give0][4 * q], acc[0][give0][4 * q + 1], acc[0][give0][4 * q + 2], acc[0][give0][4 * q + 3]);
+        }
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          *reinterpret_cast<float4*>(xmine + 256 * q) =
+              make_float4(acc[0][r][4 * q], acc[0][r][4 * q + 1], acc[0][r][4 * q + 2], acc[0][r][4 * q + 3]);
+      }
+      __syncthreads();
+      if (wk == 0) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float4 o = *reinterpret_cast<const float4*>(xpeer + 256 * q);
+          acc[0][r][4 * q] += o.x; acc[0][r][4 * q + 1] += o.y;
+          acc[0][r][4 * q + 2] += o.z; acc[0][r][4 * q + 3] += o.w;
+        }
+      } else if (BH + r < WN) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float4 o = *reinterpret_cast<const float4*>(xpeer + 256 * q);
+          acc[0][give0][4 * q] = o.x + acc[0][give0][4 * q];
+          acc[0][give0][4 * q + 1] = o.y + acc[0][give0][4 * q + 1];
+          acc[0][give0][4 * q + 2] = o.z + acc[0][give0][4 * q + 2];
+          acc[0][give0][4 * q + 3] = o.w + acc[0][give0][4 * q + 3];
+        }
+      }
+    }
+  }
+
   // Everything the output transform reads is loaded before the first store: loads and stores
   // retire through one in-order counter, so a load issued after a store would wait for that store
   // to reach memory.
@@ -503,6 +561,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, OCC) void gemm_f16_kernel(
   for (int b = 0; b < WN; ++b) {
     constexpr int kPastEnd = 0x7FFFFFF0;
     const int n = 16 * nt0 + 32 * (wn * WN + b) + i32;
+    if (WK == 2 && (b < BH) != (wk == 0)) continue;  // the other k-half stores this block
 #pragma unroll
     for (int a = 0; a < WM; ++a) {
       const unsigned row0 = (unsigned)(32 * WM * wm + 32 * a + 4 * h);
@@ -558,7 +617,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(
 
 // One Linear (group == nullptr) or the Linears of `group`, whose column blocks add up to nb_total.
 // ksplit > 1: the stages of every tile are dealt to ksplit workgroups (partial sums in `part`).
-template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH, int OCC, int BE = 1>
+template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH, int OCC, int BE = 1, int WK = 1>
 static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                              const GemmGroup* group, const int* group_N, int count, int ksplit,
                              float* part, hipStream_t s) {
@@ -580,8 +639,8 @@ static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed,
     }
     const int NB = nb;
     const int n_major = (double)M * 2.0 <= (double)n_total * 0.5625 ? 1 : 0;
-    hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModeGrouped, BE>),
-                       dim3(((MB * NB + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N), 0, s, nullptr, ah,
+    hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModeGrouped, BE, WK>),
+                       dim3(((MB * NB + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N * WK), 0, s, nullptr, ah,
                        recip, nullptr, nullptr, nullptr, nullptr, M, 0, K, 0,
                        weight_geom(group_N[0], K).KC, MB, NB, n_major, 1, nullptr, g);
     return hipGetLastError();
@@ -594,8 +653,8 @@ static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed,
   const float* rowmul = reinterpret_cast<const float*>(packed + g.rowmul_off);
   const float* bias = reinterpret_cast<const float*>(packed + g.bias_off);
   if (ksplit > 1) {
-    hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModeSplitK, BE>),
-                       dim3(((MB * NB * ksplit + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N), 0, s, y, ah,
+    hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModeSplitK, BE, WK>),
+                       dim3(((MB * NB * ksplit + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N * WK), 0, s, y, ah,
                        recip, packed, packed + g.hscale_off, rowmul, bias, M, N, K, g.NT, g.KC, MB, NB,
                        n_major, ksplit, part, GemmGroup{});
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
@@ -609,8 +668,8 @@ static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed,
     }
     return hipGetLastError();
   }
-  hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModePlain, BE>),
-                     dim3(((MB * NB + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N), 0, s, y, ah, recip,
+  hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModePlain, BE, WK>),
+                     dim3(((MB * NB + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N * WK), 0, s, y, ah, recip,
                      packed, packed + g.hscale_off, rowmul, bias, M, N, K, g.NT, g.KC, MB, NB, n_major,
                      1, nullptr, GemmGroup{});
   return hipGetLastError();
@@ -638,8 +697,13 @@ static hipError_t launch_gemm_i8(float* y, const uint8_t* ws, const uint8_t* pac
 //   3: 256 x 128, 4 wavefronts of 64 x 128 (each B fragment feeds two products: half the LDS reads
 //      per product), loads one stage ahead only, which keeps it at 224 registers: two workgroups
 //      per CU (with two stages ahead and one workgroup per CU it never beat shape 2)
-//   4: 128 x  64 with one barrier per two stages (long K, few tiles: 12-15 % over shape 1; on the
-//      128 x 128 tile the same change measured no gain)
+//   4: 128 x  64 with one barrier per two stages (12-15 % over shape 1 at long K, 1-3 % at K = 1536; on
+//      the 128 x 128 tile the same change measured no gain)
+//   5: 128 x 160, 8 wavefronts: 4 of 32 x 160 for each 32-k half of a stage (two wavefronts per SIMD
+//      from a single workgroup per CU); gate_proj at M = 512 is 4 x 56 = 224 of these, one round on
+//      256 CUs, instead of 280 tiles of 128 x 128 that leave 24 CUs with two (28.8 -> 26.3 us)
+//   6: 128 x 128, 8 wavefronts in the same arrangement: for 129..256 tiles, where every workgroup has
+//      a CU to itself (7-19 % over shape 2)
 static hipError_t launch_f16_tile(int tile, float* y, const uint8_t* ws, const uint8_t* packed, int M,
                                   int K, int N, const GemmGroup* group, const int* group_N, int count,
                                   int ksplit, float* part, hipStream_t s) {
@@ -654,25 +718,31 @@ static hipError_t launch_f16_tile(int tile, float* y, const uint8_t* ws, const u
       return launch_f16<4, 1, 2, 4, 1, 2>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
     case 4:
       return launch_f16<4, 1, 1, 2, 2, 3, 2>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
+    case 5:
+      return launch_f16<4, 1, 1, 5, 2, 1, 1, 2>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
+    case 6:
+      return launch_f16<4, 1, 1, 4, 2, 2, 1, 2>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
   }
   return hipErrorInvalidValue;
 }
 
-static int choose_f16_tile(long tiles, int K) {
-  if (tiles < 64 && K >= 4096) return 0;
-  if (tiles < 160) return K >= 4096 ? 4 : 1;
+// tiles: 128 x 128 tiles of the problem; tiles160: 128 x 160 tiles.
+static int choose_f16_tile(long tiles, long tiles160, int K) {
+  if (tiles <= 128) return 4;
+  if (tiles <= 256) return 6;
+  if (tiles160 <= 256) return 5;
   if (tiles >= 1400 || (K >= 4096 && tiles >= 320)) return 3;
   return 2;
 }
 
 // Choice of tile shape, measured on MI355X at M = 128..8192 over the decoder and ViT shapes, by
-// the number of 128 x 128 tiles the problem has. A stage of 64 k costs a lone workgroup about the
-// same time whatever its tile size, so problems with fewer tiles than CUs take the smaller tile and
-// put two workgroups on a CU; with very few tiles and a long K the 64 x 64 tile's four-fold
-// workgroup count wins. From about one tile per CU on, 128 x 128 with three resident workgroups per
-// CU is best, but there LDS bandwidth bounds it (each B fragment feeds one product); with many
-// tiles per CU (gate_proj from M = 3072 on, down_proj from 4096 on) the 256 x 128 tile is 10-17 %
-// faster (gate_proj at M = 8192: 270 -> 227 us, 1.0 PFLOP/s).
+// the number of 128 x 128 tiles the problem has. Up to half a tile per CU the 128 x 64 tile doubles the
+// workgroups; up to one tile per CU the workgroup is alone on its CU and the eight-wavefront
+// arrangement hides some of its latencies; a problem that fits one round of 128 x 160 tiles takes
+// those. Beyond that 128 x 128 with three resident workgroups per CU is best, but there LDS bandwidth
+// bounds it (each B fragment feeds one product); with many tiles per CU (gate_proj from M = 3072 on,
+// down_proj from 4096 on) the 256 x 128 tile is 10-17 % faster (gate_proj at M = 8192: 270 -> 227 us,
+// 1.0 PFLOP/s). The 64 x 64 tile no longer wins anywhere; it stays selectable by number.
 hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                        int kernel, hipStream_t s) {
   if (kernel == kKernelGemmI8 || (kernel == kKernelAuto && M <= 32)) {
@@ -683,21 +753,23 @@ hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M
                            nullptr, s);
   }
   const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-  return launch_f16_tile(choose_f16_tile(tiles, K), y, ws, packed, M, K, N, nullptr, nullptr, 0, 1,
-                         nullptr, s);
+  const long tiles160 = (long)((M + 127) / 128) * ((N + 159) / 160);
+  return launch_f16_tile(choose_f16_tile(tiles, tiles160, K), y, ws, packed, M, K, N, nullptr, nullptr, 0,
+                         1, nullptr, s);
 }
 
 hipError_t launch_gemm_group(float* const* y, const uint8_t* ws, const uint8_t* const* packed,
                              const int* N, int count, int M, int K, hipStream_t s) {
   GemmGroup g{};
-  long tiles = 0;
+  long tiles = 0, tiles160 = 0;
   for (int i = 0; i < count; ++i) {
     g.y[i] = y[i];
     g.packed[i] = packed[i];
     g.N[i] = N[i];
     tiles += (long)((M + 127) / 128) * ((N[i] + 127) / 128);
+    tiles160 += (long)((M + 127) / 128) * ((N[i] + 159) / 160);
   }
-  return launch_f16_tile(choose_f16_tile(tiles, K), nullptr, ws, nullptr, M, K, 0, &g, N, count, 1,
+  return launch_f16_tile(choose_f16_tile(tiles, tiles160, K), nullptr, ws, nullptr, M, K, 0, &g, N, count, 1,
                          nullptr, s);
 }
 
@@ -713,6 +785,7 @@ SplitPlan splitk_plan(int M, int K, int N) {
   long parts = (640 + tiles / 2) / tiles;
   parts = parts < 2 ? 2 : parts > 10 ? 10 : parts;
   p.parts = (int)parts;
+  if (tiles <= 16) p.tile = 1;  // 128 x 64: twice the workgroups (M = 128: 19 -> 16 us)
   return p;
 }
 

@@ -275,7 +275,7 @@ def test_gemm_ragged_m(pkg, orc, m):
     assert max_abs_rel(y, ref) <= TIGHT
 
 
-@pytest.mark.parametrize("kernel", ["i8", "f16", "f16:0", "f16:1", "f16:2", "f16:3", "f16:4"])
+@pytest.mark.parametrize("kernel", ["i8", "f16"] + [f"f16:{i}" for i in range(7)])
 @pytest.mark.parametrize("m,k,n", [(9, 32, 16), (40, 96, 50), (128, 1536, 256), (300, 1280, 3840),
                                    (512, 8960, 1536), (1024, 5120, 1280)])
 def test_gemm_each_kernel_matches_oracle(pkg, orc, kernel, m, k, n):
