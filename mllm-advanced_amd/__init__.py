@@ -59,6 +59,9 @@ ABI = {
     "w4a32_op_scratch_bytes": (_sz, [_ci]),
     "w4a32_op_scratch_init": (_ci, [_vp, _ci, _vp]),
     "w4a32_op_attention": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _ci, _vp, _vp]),
+    "w4a32_op_attention_prefill_scratch_bytes": (_sz, [_ci, _ci]),
+    "w4a32_op_attention_prefill": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _ci, _vp, _sz,
+                                         _vp]),
     "w4a32_op_rope_attention_decode": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci,
                                              _vp, _ci, _vp, _vp]),
     "w4a32_op_argmax": (_ci, [_vp, _ci, _vp, _vp, _vp, _vp]),
@@ -419,6 +422,23 @@ def op_attention(q, kcache, vcache, n_heads, n_kv_heads, head_dim, pos0, scratch
     _check(lib().w4a32_op_attention(_ptr(q), _ptr(kcache), _ptr(vcache), _ptr(out), M, n_heads,
                                     n_kv_heads, head_dim, kcache.shape[1], _ptr(d_pos0), pos0,
                                     _ptr(scratch), _stream()), "w4a32_op_attention")
+    return out
+
+
+def op_attention_prefill(q, kcache, vcache, n_heads, n_kv_heads, head_dim, pos0, d_pos0=None, part=None):
+    """Causal attention of M rows with the keys of each query block dealt to several workgroups; `part`
+    is the scratch (allocated here when not given)."""
+    import torch
+
+    M = q.shape[0]
+    if part is None:
+        need = int(lib().w4a32_op_attention_prefill_scratch_bytes(M, n_heads))
+        part = torch.empty((max(need, 16),), dtype=torch.uint8, device="cuda")
+    out = torch.empty((M, n_heads * head_dim), dtype=torch.float32, device="cuda")
+    _check(lib().w4a32_op_attention_prefill(_ptr(q), _ptr(kcache), _ptr(vcache), _ptr(out), M, n_heads,
+                                            n_kv_heads, head_dim, kcache.shape[1], _ptr(d_pos0), pos0,
+                                            _ptr(part), part.numel(), _stream()),
+           "w4a32_op_attention_prefill")
     return out
 
 

@@ -127,6 +127,9 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
     const w4a32_layer_weights& lw = w->layers[l];
     float* kc = reinterpret_cast<float*>(st + g.kcache_off) + (size_t)l * g.cache_layer;
     float* vc = reinterpret_cast<float*>(st + g.vcache_off) + (size_t)l * g.cache_layer;
+    // gate and up (with what lies between them) as one scratch area for the operators that run while
+    // both are dead
+    const size_t lend = g.up_off - g.gate_off + sizeof(float) * (size_t)c->max_batch_tokens * I;
     // Prefill sizes: the operator in front of a Linear runs inside that Linear's row quantiser.
     const bool fuse_rows = M > 32 && w4::quant_rows_fusable(std::max(H, I));
     // h += mlp output of the previous layer; xn = norm(h)
@@ -152,7 +155,9 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
           reinterpret_cast<float*>(scratch + sg.part_off),
           reinterpret_cast<unsigned int*>(scratch + sg.counters_off), nullptr, nullptr, nullptr, nullptr, s)));
     } else {
-      W4_TRY(from_hip(w4::launch_attention_prefill(q, kc, vc, attn, M, Hq, Hkv, c->max_seq, d_pos, 0, s)));
+      // the gate and up buffers are dead here: they hold the per-chunk results of long query blocks
+      W4_TRY(from_hip(w4::launch_attention_prefill(q, kc, vc, attn, M, Hq, Hkv, c->max_seq, d_pos, 0, gate,
+                                                   lend, s)));
     }
     W4_TRY(w4a32_matmul(delta, attn, lw.o, ws, M, qd, H, stream));
     // h += attention output; xn = norm(h)
@@ -177,7 +182,6 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
       }
       // few output tiles, long K: split-K, with the partial sums in the gate and up buffers,
       // which are dead once the quantised rows of silu(gate) * up exist
-      const size_t lend = g.up_off - g.gate_off + sizeof(float) * (size_t)c->max_batch_tokens * I;
       W4_TRY(w4a32_matmul_quantized_splitk(delta, ws, lw.down, M, I, H, gate, lend, stream));
     } else {
       W4_TRY(from_hip(w4::launch_silu_mul(gate, up, act, (size_t)M * I, s)));
@@ -378,7 +382,26 @@ int w4a32_op_attention(const float* d_q, const float* d_kcache, const float* d_v
         reinterpret_cast<unsigned int*>(sc + sg.counters_off), nullptr, nullptr, nullptr, nullptr, S(stream)));
   }
   return from_hip(w4::launch_attention_prefill(d_q, d_kcache, d_vcache, d_out, M, n_heads, n_kv_heads,
-                                               max_seq, d_pos0, pos0, S(stream)));
+                                               max_seq, d_pos0, pos0, nullptr, 0, S(stream)));
+}
+
+size_t w4a32_op_attention_prefill_scratch_bytes(int M, int n_heads) {
+  if (M <= 0 || n_heads <= 0) return 0;
+  return w4::attention_prefill_part_bytes(M, n_heads);
+}
+
+int w4a32_op_attention_prefill(const float* d_q, const float* d_kcache, const float* d_vcache,
+                               float* d_out, int M, int n_heads, int n_kv_heads, int head_dim,
+                               int max_seq, const int* d_pos0, int pos0, void* d_part, size_t part_bytes,
+                               void* stream) {
+  if (!d_q || !d_kcache || !d_vcache || !d_out) return W4A32_EINVAL;
+  if (M <= 0 || n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0) return W4A32_EINVAL;
+  if (head_dim != 128 || n_heads % n_kv_heads != 0) return W4A32_ESHAPE;
+  if (!d_pos0 && (pos0 < 0 || pos0 + M > max_seq)) return W4A32_ESHAPE;
+  if (d_part && reinterpret_cast<uintptr_t>(d_part) % 16 != 0) return W4A32_EINVAL;
+  return from_hip(w4::launch_attention_prefill(d_q, d_kcache, d_vcache, d_out, M, n_heads, n_kv_heads,
+                                               max_seq, d_pos0, pos0, static_cast<float*>(d_part),
+                                               part_bytes, S(stream)));
 }
 
 int w4a32_op_rope_attention_decode(const float* d_q, const float* d_k, const float* d_v,

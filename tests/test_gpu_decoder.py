@@ -143,6 +143,23 @@ def test_attention_prefill_and_decode(pkg, Hq, Hkv):
         out = pkg.op_attention(q, kc, vc, Hq, Hkv, D, pos0)
         assert max_abs_rel(out.cpu().numpy(), ref(q, pos0).cpu().numpy()) < 2e-5, (M, pos0)
 
+    # the same operator with scratch lent: up to 128 (head, query block) pairs the keys of a query block go
+    # to several workgroups (12 heads: up to 320 rows; 4 heads and fewer: every case here). Positions
+    # that are no multiples of 32 leave queries with no visible key in a chunk (97: the chunk that begins
+    # at key 128).
+    for M, pos0 in [(16, 0), (33, 97), (70, 0), (130, 5), (256, 0), (300, 200), (512, 0), (512, 512),
+                    (64, 960), (100, 924)]:
+        q = torch.randn((M, Hq * D), generator=g, device="cuda")
+        want = ref(q, pos0).cpu().numpy()
+        out = pkg.op_attention_prefill(q, kc, vc, Hq, Hkv, D, pos0)
+        assert max_abs_rel(out.cpu().numpy(), want) < 2e-5, (M, pos0)
+        d_pos = torch.tensor([pos0], dtype=torch.int32, device="cuda")
+        assert torch.equal(pkg.op_attention_prefill(q, kc, vc, Hq, Hkv, D, 0, d_pos0=d_pos), out)
+        # too little scratch: the operator runs unsplit
+        tiny = torch.empty((1024,), dtype=torch.uint8, device="cuda")
+        assert torch.equal(pkg.op_attention_prefill(q, kc, vc, Hq, Hkv, D, pos0, part=tiny),
+                           pkg.op_attention(q, kc, vc, Hq, Hkv, D, pos0))
+
     scratch = pkg.op_scratch(Hq)
     for pos in [0, 1, 15, 16, 63, 64, 200, 767, 1023]:     # lengths around the split and chunk sizes
         q = torch.randn((1, Hq * D), generator=g, device="cuda")
