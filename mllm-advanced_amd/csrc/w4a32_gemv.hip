@@ -533,14 +533,9 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
 static int pick_waves(int KC) { return KC < 16 ? KC : 16; }
 
 template <typename Kern>
-static hipError_t raise_lds_limit(Kern kern, size_t lds, bool* raised) {
-  if (lds > 64 * 1024 && !*raised) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (e != hipSuccess) return e;
-    *raised = true;
-  }
-  return hipSuccess;
+static hipError_t raise_lds_limit(Kern kern, size_t lds, LdsLimitOnce* once) {
+  if (lds <= 64 * 1024) return hipSuccess;
+  return once->raise(reinterpret_cast<const void*>(kern), 160 * 1024);
 }
 
 template <int M>
@@ -551,7 +546,7 @@ static hipError_t launch_gemv_m(float* y, const uint8_t* ws, const uint8_t* pack
   const int W = pick_waves(g.KC);
   const size_t lds = (size_t)M * g.Kp + (size_t)W * M * 16 * sizeof(float) + 2 * M * sizeof(float);
   auto kern = gemv_q_kernel<M>;
-  static bool raised = false;
+  static LdsLimitOnce raised;
   if (hipError_t e = raise_lds_limit(kern, lds, &raised); e != hipSuccess) return e;
   hipLaunchKernelGGL(kern, dim3(g.NT), dim3(64 * W), lds, s, y,
                      reinterpret_cast<const int8_t*>(ws + w.aq_off),
@@ -601,7 +596,7 @@ static hipError_t launch_fused_m(const GroupArgs& ga, const float* x, int ldx, i
   const size_t lds = (size_t)M * Kp + (size_t)W * sets * M * 16 * sizeof(float) +
                      (size_t)W * M * 3 * sizeof(float);
   const dim3 grid(kPair ? ga.first[1] : ga.first[ga.count]), block(64 * W);
-  static bool raised1 = false, raisedg = false;
+  static LdsLimitOnce raised1, raisedg;
   if (ga.count == 1 || kPair) {
     auto kern = gemv_fused_kernel<M, R, false, CPW, kNorm, kPair>;
     if (hipError_t e = raise_lds_limit(kern, lds, &raised1); e != hipSuccess) return e;
@@ -835,7 +830,7 @@ static hipError_t launch_wide(float* y, const float* x, int ldx, const uint8_t* 
   const WsGeom w = ws_geom(M, K);
   const size_t lds = (size_t)M * g.Kp + (size_t)kWideWaves * M * 3 * sizeof(float);
   auto kern = gemv_wide_kernel<M, kFused, kNorm>;
-  static bool raised = false;
+  static LdsLimitOnce raised;
   if (hipError_t e = raise_lds_limit(kern, lds, &raised); e != hipSuccess) return e;
   // 4 workgroups of 4 wavefronts per CU; every wavefront then walks NT / 4096 tile rows
   const int grid = std::min((g.NT + kWideWaves - 1) / kWideWaves, 1024);

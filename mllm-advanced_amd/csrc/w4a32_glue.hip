@@ -975,13 +975,10 @@ hipError_t launch_attention_prefill(const float* q, const float* kc, const float
   if (M >= 256) {  // matrix-core kernel, 32 queries per workgroup; many key blocks: 8 wavefronts
     constexpr int W = 8;
     const size_t lds = sizeof(float) * (W - 1) * 66 * 64;
-    static bool raised = false;
-    if (!raised) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_prefill_mfma_kernel<W, false>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (e != hipSuccess) return e;
-      raised = true;
-    }
+    static LdsLimitOnce raised;  // 118 KB of dynamic LDS: above the default limit
+    if (hipError_t e = raised.raise(reinterpret_cast<const void*>(attention_prefill_mfma_kernel<W, false>), lds);
+        e != hipSuccess)
+      return e;
     hipLaunchKernelGGL((attention_prefill_mfma_kernel<W, false>), dim3(Hq, (M + 31) / 32), dim3(64 * W), lds,
                        s, q, kc, vc, out, M, Hq, Hkv, max_seq, d_pos0, pos0, scale, nullptr);
   } else if (M >= 16) {

@@ -2,6 +2,7 @@
 // validated by the caller (w4a32_capi.hip).
 #pragma once
 
+#include <atomic>
 #include <hip/hip_runtime.h>
 
 #include "w4a32_hip.h"
@@ -52,6 +53,23 @@ hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M
                        int kernel, hipStream_t s);
 // the f16 kernel with every tile's k range dealt to several workgroups (partial sums in `part`,
 // which holds parts * M * N floats), then a reduction; for few tiles and a long K
+// A kernel that needs more dynamic LDS than the default limit has the limit raised once per device
+// (the attribute belongs to the function on the current device); bit d of the mask = done on device d.
+struct LdsLimitOnce {
+  std::atomic<unsigned long long> done{0};
+  hipError_t raise(const void* kernel, size_t bytes) {
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+    const unsigned long long bit = dev < 64 ? 1ull << dev : 0;  // past 64 devices: set on every call
+    if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+    if (hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        e != hipSuccess)
+      return e;
+    done.fetch_or(bit, std::memory_order_release);
+    return hipSuccess;
+  }
+};
+
 struct SplitPlan {
   int tile, parts;
 };

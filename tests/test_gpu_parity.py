@@ -276,11 +276,12 @@ def test_gemm_ragged_m(pkg, orc, m):
 
 
 @pytest.mark.parametrize("kernel", ["i8", "f16"] + [f"f16:{i}" for i in range(7)])
-@pytest.mark.parametrize("m,k,n", [(9, 32, 16), (40, 96, 50), (128, 1536, 256), (300, 1280, 3840),
-                                   (512, 8960, 1536), (1024, 5120, 1280)])
+@pytest.mark.parametrize("m,k,n", [(9, 32, 16), (40, 96, 50), (200, 160, 330), (128, 1536, 256),
+                                   (300, 1280, 3840), (512, 8960, 1536), (1024, 5120, 1280)])
 def test_gemm_each_kernel_matches_oracle(pkg, orc, kernel, m, k, n):
-    # both prefill kernels (and each tile shape of the f16 one) on the same inputs; K = 32 and 96
-    # leave padding inside a stage
+    # both prefill kernels (and each tile shape of the f16 one) on the same inputs; K = 32, 96 and 160
+    # leave padding inside a stage (an odd number of 32-k blocks: the second k-half of the last stage
+    # is all padding); N = 330 ends inside a 160- and a 128-column tile
     w = make_weights(n, k, seed=k)
     x = make_acts(m, k, seed=m, outlier_frac=0.02)
     bias = bias_for(n, True)
