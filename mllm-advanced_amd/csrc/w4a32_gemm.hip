@@ -399,11 +399,20 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
       const int rbuf = ((u / BE) & 1) * BE + u % BE;                    // buffer this stage reads
       const int wbuf = (((u + BE) / BE) & 1) * BE + (u + BE) % BE;      // buffer of stage s + BE
       const uint8_t* bbuf = sB + rbuf * kBufBytes + 16 * lane + (WK == 2 ? wk * (SL * BN32 * 1024) : 0);
+      // B fragments are requested LA products before their use, one per product (a steady stream of LDS
+      // reads; measured the same for LA = 1..4, and the same as a whole slice at a time). A fragment's
+      // register is that of the fragment two slices before it, which must have been used: LA <= 2 WN.
+      constexpr int F = SL * WN;  // fragments of a stage; fragment f = slice f / WN, column block f % WN
+      constexpr int LA = 2;
+      static_assert(LA <= 2 * WN && LA < F, "a fragment would overwrite one that is still to be used");
+      auto fetch = [&](int f, const uint8_t* base) {
+        bf[(f / WN) & 1][f % WN] =
+            *reinterpret_cast<const h8*>(base + ((f / WN) * BN32 + wn * WN + f % WN) * 1024);
+      };
       if (u % BE == 0) {
         __syncthreads();
 #pragma unroll
-        for (int b = 0; b < WN; ++b)
-          bf[0][b] = *reinterpret_cast<const h8*>(bbuf + (wn * WN + b) * 1024);
+        for (int f = 0; f < LA; ++f) fetch(f, bbuf);
         __builtin_amdgcn_sched_barrier(0);  // requested first: their latency covers what follows
       }
       // Inputs of the dequantisation (stage s + BE, in this stage's ring slot) move to temporaries,
@@ -462,11 +471,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
             acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
                 __builtin_bit_cast(h8, areg[slot][sl >> 1][a][sl & 1]), bf[sl & 1][b], acc[a][b], 0,
                 0, 0);
-            if (sl < SL - 1 && a == 0)  // the next slice's fragment b, one read per product
-              bf[(sl + 1) & 1][b] =
-                  *reinterpret_cast<const h8*>(bbuf + ((sl + 1) * BN32 + wn * WN + b) * 1024);
-            if (sl == SL - 1 && a == 0 && (u + 1) % BE != 0)  // no barrier ahead: the next stage's first
-              bf[0][b] = *reinterpret_cast<const h8*>(bbuf + kBufBytes + (wn * WN + b) * 1024);
+            if (a == 0) {
+              const int f = sl * WN + b + LA;
+              if (f < F) {
+                fetch(f, bbuf);
+              } else if ((u + 1) % BE != 0) {  // no barrier ahead: the next stage's first fragments
+                fetch(f - F, bbuf + kBufBytes);
+              }
+            }
 #pragma unroll
             for (int st = mi * NSTEP / kMfma; st < (mi + 1) * NSTEP / kMfma; ++st) dq_step(st);
             ++mi;
