@@ -131,8 +131,8 @@ int w4a32_matmul_quantized(float* d_y, const void* d_ws, const void* d_packed, i
 #define W4A32_KERNEL_GEMM_F16 3   /* f16 MFMA on exact f16 operands, M > 8; tile shape by size */
 /* The f16 kernel with one named tile shape, W4A32_KERNEL_GEMM_F16_TILE0 + i:
  * i = 0: 64 x 64, 1: 128 x 64, 2: 128 x 128, 3: 256 x 128 (rows x columns per workgroup),
- * 4: 128 x 64 with one barrier per two stages, 5: 128 x 160 and 6: 128 x 128 with eight wavefronts
- * (each 32-k half of a stage has its own four). */
+ * 4: 128 x 64 with one barrier per two stages, 5: 128 x 160, 6: 128 x 128 with eight wavefronts (each
+ * 32-k half of a stage has its own four). */
 #define W4A32_KERNEL_GEMM_F16_TILE0 16
 #define W4A32_GEMM_F16_TILES 7
 int w4a32_matmul_quantized_ex(float* d_y, const void* d_ws, const void* d_packed, int M, int K,

@@ -711,11 +711,12 @@ static hipError_t launch_gemm_i8(float* y, const uint8_t* ws, const uint8_t* pac
 //      per CU (with two stages ahead and one workgroup per CU it never beat shape 2)
 //   4: 128 x  64 with one barrier per two stages (12-15 % over shape 1 at long K, 1-3 % at K = 1536; on
 //      the 128 x 128 tile the same change measured no gain)
-//   5: 128 x 160, 8 wavefronts: 4 of 32 x 160 for each 32-k half of a stage (two wavefronts per SIMD
-//      from a single workgroup per CU); gate_proj at M = 512 is 4 x 56 = 224 of these, one round on
-//      256 CUs, instead of 280 tiles of 128 x 128 that leave 24 CUs with two (28.8 -> 26.3 us)
-//   6: 128 x 128, 8 wavefronts in the same arrangement: for 129..256 tiles, where every workgroup has
-//      a CU to itself (7-19 % over shape 2)
+//   5: 128 x 160, 4 wavefronts of 32 x 160, two workgroups per CU: gate_proj at M = 512 is 4 x 56 = 224 of
+//      these, one on almost every CU, instead of 280 tiles of 128 x 128 that leave 24 CUs with two
+//      (28.8 -> 26.3 us); at M = 1024 it is 448, two per CU (41.1 -> 38.4 us)
+//   6: 128 x 128, 8 wavefronts: 4 of 32 x 128 for each 32-k half of a stage (two wavefronts per SIMD from
+//      a single workgroup); for 129..256 tiles, where every workgroup has a CU to itself (7-19 % over
+//      shape 2). The same arrangement on the 128 x 160 tile measured 1-3 % behind shape 5.
 static hipError_t launch_f16_tile(int tile, float* y, const uint8_t* ws, const uint8_t* packed, int M,
                                   int K, int N, const GemmGroup* group, const int* group_N, int count,
                                   int ksplit, float* part, hipStream_t s) {
@@ -731,7 +732,7 @@ static hipError_t launch_f16_tile(int tile, float* y, const uint8_t* ws, const u
     case 4:
       return launch_f16<4, 1, 1, 2, 2, 3, 2>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
     case 5:
-      return launch_f16<4, 1, 1, 5, 2, 1, 1, 2>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
+      return launch_f16<4, 1, 1, 5, 2, 2>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
     case 6:
       return launch_f16<4, 1, 1, 4, 2, 2, 1, 2>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
   }
@@ -742,7 +743,9 @@ static hipError_t launch_f16_tile(int tile, float* y, const uint8_t* ws, const u
 static int choose_f16_tile(long tiles, long tiles160, int K) {
   if (tiles <= 128) return 4;
   if (tiles <= 256) return 6;
-  if (tiles160 <= 256) return 5;
+  // 128 x 160 tiles, two workgroups per CU: when they come to one or two per CU with few CUs left over
+  const long slots = 256 * ((tiles160 + 255) / 256);
+  if (tiles160 <= 512 && tiles160 * 100 >= slots * 85) return 5;
   if (tiles >= 1400 || (K >= 4096 && tiles >= 320)) return 3;
   return 2;
 }
@@ -750,8 +753,8 @@ static int choose_f16_tile(long tiles, long tiles160, int K) {
 // Choice of tile shape, measured on MI355X at M = 128..8192 over the decoder and ViT shapes, by
 // the number of 128 x 128 tiles the problem has. Up to half a tile per CU the 128 x 64 tile doubles the
 // workgroups; up to one tile per CU the workgroup is alone on its CU and the eight-wavefront
-// arrangement hides some of its latencies; a problem that fits one round of 128 x 160 tiles takes
-// those. Beyond that 128 x 128 with three resident workgroups per CU is best, but there LDS bandwidth
+// arrangement hides some of its latencies; a problem whose 128 x 160 tiles come to (nearly) one or two per
+// CU takes those. Beyond that 128 x 128 with three resident workgroups per CU is best, but there LDS bandwidth
 // bounds it (each B fragment feeds one product); with many tiles per CU (gate_proj from M = 3072 on,
 // down_proj from 4096 on) the 256 x 128 tile is 10-17 % faster (gate_proj at M = 8192: 270 -> 227 us,
 // 1.0 PFLOP/s). The 64 x 64 tile no longer wins anywhere; it stays selectable by number.
