@@ -23,7 +23,7 @@ def test_backend_library_is_built_and_loads():
 
 def test_container_structs_have_the_on_disk_sizes():
     # head 268 bytes, descriptor 416 bytes: the header static_asserts them; check the text is there
-    text = open(os.path.join(HOST, "mllm", "Engine", "ParameterReader.hpp")).read()
+    text = open(os.path.join(HOST, "mllm", "EngineSlice.hpp")).read()
     assert "sizeof(ParameterPackHead) == 268" in text and "sizeof(ParameterDescriptor) == 416" in text
     assert "0x519ACE0519ACE000" in text
 
