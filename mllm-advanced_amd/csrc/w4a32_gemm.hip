@@ -206,9 +206,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
   constexpr int NSTEP = 4 * NDW;               // in four steps each
   constexpr int kLdsBufs = 2 * BE;             // two sets (read / being written) of BE stage buffers
   constexpr int kSpareOff = kLdsBufs * kBufBytes;
-  constexpr int kLdsBytes = kSpareOff + (kSpareUnits ? 1024 : 0);
+  constexpr int kStageBytes = kSpareOff + (kSpareUnits ? 1024 : 0);
+  constexpr int kMeetBytes = WK == 2 ? NWAVES * 4096 : 0;  // the k-halves' sums meet in the same memory
+  constexpr int kLdsBytes = kStageBytes > kMeetBytes ? kStageBytes : kMeetBytes;
   static_assert(kLdsBytes <= 65536, "static LDS");
-  static_assert(WK == 1 || kSpareOff >= NWAVES * 4096, "the k-halves meet through the stage buffers");
 
   __shared__ __align__(16) uint8_t sB[kLdsBytes];
 
