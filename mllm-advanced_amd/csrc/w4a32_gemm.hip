@@ -790,18 +790,22 @@ hipError_t launch_gemm_group(float* const* y, const uint8_t* ws, const uint8_t* 
 }
 
 // Split-K: tile shape and number of parts for a problem (parts == 1: not worth splitting).
-// Measured on MI355X (down_proj, K = 8960, N = 1536): M = 128: 44 -> 19 us, 256: 48 -> 21,
-// 512: 51 -> 30, 2048: 95 -> 80; at K = 1536 and K = 5120 the second kernel and the partial sums'
-// traffic cost what the shorter loops gain, so only long K qualifies.
+// Measured on MI355X (down_proj, K = 8960, N = 1536): M = 128: 44 -> 16 us, 256: 44 -> 21,
+// 512: 47 -> 29, 1024: 50 -> 45, 2048: 85 -> 82; at K = 1536 and K = 5120 the second kernel and the
+// partial sums' traffic cost what the shorter loops gain, so only long K qualifies. Parts: about one or
+// two workgroups per CU in all (10 parts up to 24 tiles, 5 up to 96, then 4); more parts only add
+// partial sums for the second kernel to read.
 SplitPlan splitk_plan(int M, int K, int N) {
   SplitPlan p{2, 1};
   const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
   const int nstages = (K + kF16BK - 1) / kF16BK;
   if (M <= 32 || nstages < 96 || tiles > 256) return p;
-  long parts = (640 + tiles / 2) / tiles;
-  parts = parts < 2 ? 2 : parts > 10 ? 10 : parts;
-  p.parts = (int)parts;
-  if (tiles <= 16) p.tile = 1;  // 128 x 64: twice the workgroups (M = 128: 19 -> 16 us)
+  p.parts = tiles <= 24 ? 10 : tiles <= 96 ? 5 : 4;
+  if (tiles <= 16) {
+    p.tile = 1;  // 128 x 64: twice the workgroups (M = 128: 19 -> 16 us)
+  } else if (tiles * p.parts <= 256) {
+    p.tile = 6;  // every workgroup alone on its CU: the eight-wavefront shape (M = 512: 30.1 -> 29.1 us)
+  }
   return p;
 }
 

@@ -301,7 +301,8 @@ def test_gemm_each_kernel_matches_oracle(pkg, orc, kernel, m, k, n):
     assert err <= GEMM_TOL and err <= TIGHT, (kernel, err)
 
 
-@pytest.mark.parametrize("m,k,n", [(512, 8960, 1536), (100, 8960, 50), (300, 6144, 272), (64, 256, 64)])
+@pytest.mark.parametrize("m,k,n", [(512, 8960, 1536), (100, 8960, 50), (300, 6144, 272), (1024, 8960, 1536),
+                                   (1100, 6144, 1536), (64, 256, 64)])
 def test_splitk_matches_oracle_and_plain(pkg, orc, m, k, n):
     # few tiles and a long K: the k range of a tile is dealt to several workgroups and the parts are
     # added by a second kernel; the last shape is one the library does not split (falls through)
