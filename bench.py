@@ -352,16 +352,16 @@ def main():
                     tot_flop += flop
                     tot_ms += times[0]
                     tot_kms += times[1]
-                # The layer's Linears as a prefill issues them: rows quantised once per input, q,k,v and
-                # gate,up each as one grouped launch, down with its k range split over workgroups
-                # (partial sums in lent scratch).
+                # The layer's Linears as a prefill issues them: rows quantised once per input, q,k,v as one
+                # grouped launch, gate,up as one launch that stores silu(gate) * up only, down with its k
+                # range split over workgroups (partial sums in lent scratch).
                 lay = layers[0]
                 xh = torch.randn((M, 1536), generator=xgen, device="cuda")
                 xi = torch.randn((M, 8960), generator=xgen, device="cuda")
                 ws_h = torch.empty(pkg.workspace_bytes(M, 1536), dtype=torch.uint8, device="cuda")
                 ws_i = torch.empty(pkg.workspace_bytes(M, 8960), dtype=torch.uint8, device="cuda")
                 yq, yk, yv = (torch.empty((M, n), device="cuda") for n in (1536, 256, 256))
-                yg, yu = (torch.empty((M, 8960), device="cuda") for _ in range(2))
+                yg = torch.empty((M, 8960), device="cuda")
                 yo = torch.empty((M, 1536), device="cuda")
                 scratch = torch.empty(max(16, int(L.w4a32_splitk_scratch_bytes(M, 8960, 1536))),
                                       dtype=torch.uint8, device="cuda")
@@ -373,8 +373,7 @@ def main():
                     pkg.quant_lhs(xh, ws_h)
                     pkg.matmul_quantized(ws_h, lay[3].packed, M, 1536, 1536, out=yo)
                     pkg.quant_lhs(xh, ws_h)
-                    pkg.matmul_quantized_grouped(ws_h, [lay[4].packed, lay[5].packed], [8960, 8960], M,
-                                                 1536, outs=[yg, yu])
+                    pkg.matmul_quantized_silu_pair(ws_h, lay[4].packed, lay[5].packed, M, 1536, 8960, out=yg)
                     pkg.quant_lhs(xi, ws_i)
                     pkg.matmul_quantized_splitk(ws_i, lay[6].packed, M, 8960, 1536, scratch=scratch, out=yo)
                 for _ in range(3):

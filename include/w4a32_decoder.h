@@ -30,7 +30,10 @@ int w4a32_op_embedding(const int64_t* d_ids, const float* d_table, int M, int D,
 int w4a32_op_rmsnorm(const float* d_h, const float* d_delta, const float* d_weight, int M, int D,
                      float eps, float* d_h_out, float* d_y, void* stream);
 
-/* out = a + b; out = silu(gate) * up (QWenMLP::forward, modeling_ds_qwen2.hpp:47-54). n % 4 == 0. */
+/* out = a + b; out = silu(gate) * up (QWenMLP::forward, modeling_ds_qwen2.hpp:47-54). n % 4 == 0.
+ * silu(g) * u is evaluated as g * rcp(1 + exp2(-g * log2 e)) * u with the hardware's exponential and
+ * reciprocal (about 1 ulp each, 3e-7 relative against the correctly rounded expression), the same
+ * expression in every kernel of this library that applies it. */
 int w4a32_op_add(const float* d_a, const float* d_b, float* d_out, size_t n, void* stream);
 int w4a32_op_silu_mul(const float* d_gate, const float* d_up, float* d_out, size_t n, void* stream);
 

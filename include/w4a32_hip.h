@@ -170,6 +170,15 @@ int w4a32_matmul_grouped(float* const* d_y, const float* d_x, const void* const*
 int w4a32_matmul_quantized_grouped(float* const* d_y, const void* d_ws, const void* const* d_packed,
                                    const int* N, int count, int M, int K, void* stream);
 
+/* d_act[M][N] = silu(x W_gate^T + b_gate) * (x W_up^T + b_up) on rows already quantised into d_ws, M > 32:
+ * the MLP's gate_proj, up_proj, SiLU and multiply (modeling_ds_qwen2.hpp:47-54) in one launch of the
+ * prefill kernel. A wavefront computes both Linears for the same outputs and stores only their product,
+ * so neither Linear's [M][N] result is written or read back. Each factor is the value
+ * w4a32_matmul_quantized gives (same products and summation order), combined with w4a32_op_silu_mul's
+ * expression. W4A32_ESHAPE for M <= 32. */
+int w4a32_matmul_quantized_silu_pair(float* d_act, const void* d_ws, const void* d_gate, const void* d_up,
+                                     int M, int K, int N, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -59,6 +59,7 @@ ABI = {
     "w4a32_op_scratch_bytes": (_sz, [_ci]),
     "w4a32_op_scratch_init": (_ci, [_vp, _ci, _vp]),
     "w4a32_op_attention": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _ci, _vp, _vp]),
+    "w4a32_matmul_quantized_silu_pair": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a32_op_attention_prefill_scratch_bytes": (_sz, [_ci, _ci]),
     "w4a32_op_attention_prefill": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _ci, _vp, _sz,
                                          _vp]),
@@ -286,6 +287,16 @@ def matmul_quantized_grouped(ws, packed_list, Ns, M, K, outs=None):
     _check(lib().w4a32_matmul_quantized_grouped(yarr, _ptr(ws), parr, narr, n, M, K, _stream()),
            "w4a32_matmul_quantized_grouped")
     return ys
+
+
+def matmul_quantized_silu_pair(ws, gate, up, M, K, N, out=None):
+    """silu(gate Linear) * (up Linear) on rows already quantised into ws, one launch (M > 32)."""
+    import torch
+
+    y = out if out is not None else torch.empty((M, N), dtype=torch.float32, device="cuda")
+    _check(lib().w4a32_matmul_quantized_silu_pair(_ptr(y), _ptr(ws), _ptr(gate), _ptr(up), M, K, N, _stream()),
+           "w4a32_matmul_quantized_silu_pair")
+    return y
 
 
 def matmul_quantized_splitk(ws, packed, M, K, N, scratch=None, out=None):

@@ -255,4 +255,17 @@ int w4a32_matmul_quantized_grouped(float* const* d_y, const void* d_ws, const vo
   return W4A32_OK;
 }
 
+int w4a32_matmul_quantized_silu_pair(float* d_act, const void* d_ws, const void* d_gate, const void* d_up,
+                                     int M, int K, int N, void* stream) {
+  if (!d_act || !d_ws || !d_gate || !d_up || M <= 0) return W4A32_EINVAL;
+  if (int e = shape_ok(N, K)) return e;
+  if (M <= 32) return W4A32_ESHAPE;  // the f16 product kernel's sizes only
+  if (!aligned(d_ws, 256) || !aligned(d_gate, 16) || !aligned(d_up, 16) || !aligned(d_act, 4)) {
+    return W4A32_EINVAL;
+  }
+  return from_hip(w4::launch_gemm_pair(d_act, static_cast<const uint8_t*>(d_ws),
+                                       static_cast<const uint8_t*>(d_gate), static_cast<const uint8_t*>(d_up),
+                                       M, K, N, static_cast<hipStream_t>(stream)));
+}
+
 }  // extern "C"

@@ -166,8 +166,9 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
       const void* ps[2] = {lw.gate, lw.up};
       const int ns[2] = {I, I};
       if (fuse_rows) {
+        // gate, up, SiLU and the multiply in one launch: only silu(gate) * up is stored
         W4_TRY(w4a32_quant_lhs_norm(h, delta, lw.ffn_norm, c->rms_eps, h, M, H, ws, stream));
-        W4_TRY(w4a32_matmul_quantized_grouped(ys, ws, ps, ns, 2, M, H, stream));
+        W4_TRY(w4a32_matmul_quantized_silu_pair(act, ws, lw.gate, lw.up, M, H, I, stream));
       } else {
         W4_TRY(from_hip(w4::launch_rmsnorm(h, delta, lw.ffn_norm, M, H, c->rms_eps, h, xn, s)));
         W4_TRY(w4a32_matmul_grouped(ys, xn, ps, ns, 2, ws, M, H, stream));
@@ -175,7 +176,7 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
     }
     if (M > 32) {
       if (fuse_rows) {
-        W4_TRY(w4a32_quant_lhs_silu_mul(gate, up, M, I, ws, stream));
+        W4_TRY(w4a32_quant_lhs(act, M, I, I, ws, stream));
       } else {
         W4_TRY(from_hip(w4::launch_silu_mul(gate, up, act, (size_t)M * I, s)));
         W4_TRY(w4a32_quant_lhs(act, M, I, I, ws, stream));

@@ -162,11 +162,16 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 // blocks are numbered through (Linear i owns blocks nb_first[i] .. nb_first[i+1]-1); a workgroup
 // looks its Linear up and takes N, the blob and the output from the table.
 //
+// PAIR: two Linears of equal N on the same rows (the MLP's gate and up) whose outputs are only wanted as
+// silu(y0) * y1: the left half of a workgroup's column fragments comes from Linear 0, the right half from
+// Linear 1, same columns, so that a wavefront holds both factors of an output in the same lane and
+// register index; it stores the product (N columns) and neither factor reaches memory.
+//
 // SPLITK: `ksplit` workgroups share a tile, each takes a contiguous range of the stages and stores
 // its raw f32 sums to part[ks][M][N]; splitk_reduce_kernel adds the parts in a fixed order and
 // applies the output transform. For problems with few tiles and a long K (down_proj at M <= 512:
 // 48 tiles of 128 x 128 for 256 CUs, 140 stages each).
-constexpr int kModePlain = 0, kModeGrouped = 1, kModeSplitK = 2;
+constexpr int kModePlain = 0, kModeGrouped = 1, kModeSplitK = 2, kModePair = 3;
 constexpr int kMaxGemmGroup = W4A32_MAX_GROUP;
 struct GemmGroup {
   float* y[kMaxGemmGroup];
@@ -182,7 +187,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
     const float* __restrict__ rowmul_arg, const float* __restrict__ bias_arg, int M, int N_arg, int K,
     int NT_arg, int KC, int MB, int NB, int n_major, int ksplit, float* __restrict__ part,
     const GemmGroup grp) {
-  constexpr bool GROUPED = MODE == kModeGrouped, SPLITK = MODE == kModeSplitK;
+  constexpr bool GROUPED = MODE == kModeGrouped, SPLITK = MODE == kModeSplitK, PAIR = MODE == kModePair;
+  static_assert(!PAIR || (WAVES_N == 1 && WN % 2 == 0 && WK == 1), "a wavefront must own both halves");
   constexpr int D = DEPTH;
   // BE = stages per barrier (1 or 2). The loop is unrolled U stages at a time so that ring slots and
   // LDS buffers are compile-time constants.
@@ -259,8 +265,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
     rowmul = reinterpret_cast<const float*>(packed + wgm.rowmul_off);
     bias = reinterpret_cast<const float*>(packed + wgm.bias_off);
   }
+  if constexpr (PAIR) {
+    N = grp.N[0];
+    NT = weight_geom(N, K).NT;
+    y = grp.y[0];
+  }
   const int m0 = mb * BM + 32 * WM * wm;
-  const int nt0 = nb * WNT;
+  // first 16-row weight tile row of this workgroup's columns (PAIR: in both Linears, half the units each)
+  const int nt0 = nb * (PAIR ? WNT / 2 : WNT);
   // this workgroup's stages: [s_begin, nstages)
   int s_begin = 0, nstages = (K + kF16BK - 1) / kF16BK;
   if constexpr (SPLITK) {
@@ -289,10 +301,18 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
   for (int u = 0; u < B_UNITS; ++u) {
     int ntl = wave + NWAVES * u;
     ntl = ntl < WNT ? ntl : WNT - 1;  // a surplus unit
+    const uint8_t* pk = packed;
+    const uint8_t* hs = hscale;
+    if constexpr (PAIR) {
+      const int side = ntl >= WNT / 2 ? 1 : 0;  // wavefront-uniform
+      ntl -= side * (WNT / 2);
+      pk = grp.packed[side];
+      hs = pk + weight_geom(N, K).hscale_off;
+    }
     int nt = nt0 + ntl;
     nt = nt < NT ? nt : NT - 1;  // tile rows past the matrix: their columns are never stored
-    bq_ptr[u] = packed + (size_t)nt * KC * kTileBytes + 16 * lane;
-    bs_ptr[u] = hscale + (size_t)nt * KC * kTileScaleBytes + 8 * j;
+    bq_ptr[u] = pk + (size_t)nt * KC * kTileBytes + 16 * lane;
+    bs_ptr[u] = hs + (size_t)nt * KC * kTileScaleBytes + 8 * j;
   }
 
   // The steady-state loop must stay ONE basic block (the compiler can then wait for exactly
@@ -540,6 +560,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
   // retire through one in-order counter, so a load issued after a store would wait for that store
   // to reach memory.
   float rc[WM][16], rm[WN], bs[WN];
+  constexpr int WNH = PAIR ? WN / 2 : WN;  // column blocks a wavefront stores
 #pragma unroll
   for (int a = 0; a < WM; ++a) {
 #pragma unroll
@@ -550,9 +571,17 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
   }
 #pragma unroll
   for (int b = 0; b < WN; ++b) {
-    const int n = 16 * nt0 + 32 * (wn * WN + b) + i32;
-    rm[b] = load_global<float>(rowmul + (n < N ? n : N - 1));
-    bs[b] = load_global<float>(bias + (n < N ? n : N - 1));
+    const int n = 16 * nt0 + 32 * (wn * WN + b % WNH) + i32;
+    const float* rmp = rowmul;
+    const float* bsp = bias;
+    if constexpr (PAIR) {
+      const WeightGeom wgm = weight_geom(N, K);
+      const uint8_t* pk = grp.packed[b / WNH];
+      rmp = reinterpret_cast<const float*>(pk + wgm.rowmul_off);
+      bsp = reinterpret_cast<const float*>(pk + wgm.bias_off);
+    }
+    rm[b] = load_global<float>(rmp + (n < N ? n : N - 1));
+    bs[b] = load_global<float>(bsp + (n < N ? n : N - 1));
   }
 
   __builtin_amdgcn_sched_barrier(0);
@@ -571,7 +600,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
       out_base, 0, (int)((unsigned)rows_valid * (unsigned)N * 4u), 0x00020000);
   const unsigned row_bytes = (unsigned)N * 4u;
 #pragma unroll
-  for (int b = 0; b < WN; ++b) {
+  for (int b = 0; b < WNH; ++b) {
     constexpr int kPastEnd = 0x7FFFFFF0;
     const int n = 16 * nt0 + 32 * (wn * WN + b) + i32;
     if (WK == 2 && (b < BH) != (wk == 0)) continue;  // the other k-half stores this block
@@ -585,6 +614,11 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
         if constexpr (!SPLITK) {
           val = __fmaf_rn(val * rm[b], rc[a][v], bs[b]);
           val = fminf(fmaxf(val, -3.402823466e+38f), 3.402823466e+38f);
+        }
+        if constexpr (PAIR) {
+          float up = __fmaf_rn(acc[a][b + WNH][v] * rm[b + WNH], rc[a][v], bs[b + WNH]);
+          up = fminf(fmaxf(up, -3.402823466e+38f), 3.402823466e+38f);
+          val = silu_mul(val, up);
         }
         const unsigned dm = 8 * (v >> 2) + (v & 3);  // row offset from row0
         const int off = n < N ? (int)(off0 + dm * row_bytes) : kPastEnd;
@@ -688,6 +722,29 @@ static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed,
   return hipGetLastError();
 }
 
+// silu(x W0^T) * (x W1^T) for two Linears of equal N, stored to one [M][N] output.
+template <int WAVES_M, int WN, int DEPTH, int OCC, int WM = 1>
+static hipError_t launch_f16_pair(float* act, const uint8_t* ws, const uint8_t* gate, const uint8_t* up, int M,
+                                  int K, int N, hipStream_t s) {
+  constexpr int BM = 32 * WM * WAVES_M, WNT = 2 * WN;
+  const WsGeom w = ws_geom(M, K);
+  const WeightGeom wg = weight_geom(N, K);
+  const int MB = (M + BM - 1) / BM;
+  const int NB = (wg.NT + WNT / 2 - 1) / (WNT / 2);
+  GemmGroup g{};
+  g.y[0] = act;
+  g.packed[0] = gate;
+  g.packed[1] = up;
+  g.N[0] = g.N[1] = N;
+  const int n_major = (double)M * 2.0 <= (double)N * 2.0 * 0.5625 ? 1 : 0;
+  hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, 1, WM, WN, DEPTH, OCC, kModePair, 1, 1>),
+                     dim3(((MB * NB + 7) / 8) * 8), dim3(64 * WAVES_M), 0, s, nullptr,
+                     reinterpret_cast<const _Float16*>(ws + w.ah_off),
+                     reinterpret_cast<const float*>(ws + w.scale_off), nullptr, nullptr, nullptr, nullptr, M, 0,
+                     K, 0, wg.KC, MB, NB, n_major, 1, nullptr, g);
+  return hipGetLastError();
+}
+
 static hipError_t launch_gemm_i8(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K,
                                  int N, hipStream_t s) {
   const WeightGeom g = weight_geom(N, K);
@@ -787,6 +844,18 @@ hipError_t launch_gemm_group(float* const* y, const uint8_t* ws, const uint8_t* 
   }
   return launch_f16_tile(choose_f16_tile(tiles, tiles160, K), nullptr, ws, nullptr, M, K, 0, &g, N, count, 1,
                          nullptr, s);
+}
+
+// The MLP's gate and up Linears with silu(gate) * up as the only output. Tile shape as for the two Linears
+// side by side (2N columns), among the shapes whose wavefronts own whole rows of a column block pair.
+hipError_t launch_gemm_pair(float* act, const uint8_t* ws, const uint8_t* gate, const uint8_t* up, int M,
+                            int K, int N, hipStream_t s) {
+  const long tiles = (long)((M + 127) / 128) * ((2 * N + 127) / 128);
+  if (tiles <= 128) return launch_f16_pair<4, 2, 2, 4>(act, ws, gate, up, M, K, N, s);
+  if (tiles >= 1000 || (K >= 4096 && tiles >= 320)) {  // 256 x 128 (M = 1024: 71 -> 69 us, 2048: 132 -> 127)
+    return launch_f16_pair<4, 4, 1, 2, 2>(act, ws, gate, up, M, K, N, s);
+  }
+  return launch_f16_pair<4, 4, 2, 3>(act, ws, gate, up, M, K, N, s);
 }
 
 // Split-K: tile shape and number of parts for a problem (parts == 1: not worth splitting).

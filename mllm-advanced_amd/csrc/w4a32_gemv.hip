@@ -524,7 +524,7 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
         res[st] = fminf(fmaxf(v, -3.402823466e+38f), 3.402823466e+38f);
       }
       float v = res[0];
-      if (kPair) v = res[0] / (1.0f + expf(-res[0])) * res[kSets - 1];  // silu(gate) * up
+      if (kPair) v = silu_mul(res[0], res[kSets - 1]);
       *(W4_GLOBAL float*)(y + (size_t)m * N + n) = v;
     }
   }

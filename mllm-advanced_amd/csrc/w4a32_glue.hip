@@ -140,10 +140,10 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__
     const float4 a = reinterpret_cast<const float4*>(g)[i];
     const float4 b = reinterpret_cast<const float4*>(u)[i];
     float4 o;
-    o.x = a.x / (1.0f + expf(-a.x)) * b.x;
-    o.y = a.y / (1.0f + expf(-a.y)) * b.y;
-    o.z = a.z / (1.0f + expf(-a.z)) * b.z;
-    o.w = a.w / (1.0f + expf(-a.w)) * b.w;
+    o.x = silu_mul(a.x, b.x);
+    o.y = silu_mul(a.y, b.y);
+    o.z = silu_mul(a.z, b.z);
+    o.w = silu_mul(a.w, b.w);
     reinterpret_cast<float4*>(out)[i] = o;
   }
 }

@@ -74,6 +74,8 @@ struct SplitPlan {
   int tile, parts;
 };
 SplitPlan splitk_plan(int M, int K, int N);
+hipError_t launch_gemm_pair(float* act, const uint8_t* ws, const uint8_t* gate, const uint8_t* up, int M,
+                            int K, int N, hipStream_t s);
 hipError_t launch_gemm_splitk(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                               float* part, hipStream_t s);
 // several Linears on the same quantised rows in one launch of the f16 kernel (M > 32)
@@ -124,6 +126,16 @@ __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 #define W4_GLOBAL __attribute__((address_space(1)))
+// silu(g) * u = g / (1 + e^-g) * u, the one expression every kernel that applies the MLP's activation
+// uses (the standalone operator, the row quantiser that applies it on the way, the decode pair kernel and
+// the prefill pair kernel's epilogue), so that they agree bit for bit. Hardware exponential and
+// reciprocal (about 1 ulp each): where the activation runs in a product kernel's epilogue, on a few
+// wavefronts per CU, the correctly rounded library routines cost as much as the products of a tile.
+__device__ __forceinline__ float silu_mul(float g, float u) {
+  const float e = __builtin_amdgcn_exp2f(g * -1.44269504088896340736f);
+  return g * __builtin_amdgcn_rcpf(1.0f + e) * u;
+}
+
 template <typename T>
 __device__ __forceinline__ T load_global(const void* p) {
   return *(const W4_GLOBAL T*)p;

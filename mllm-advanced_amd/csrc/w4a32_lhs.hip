@@ -119,14 +119,14 @@ __global__ __launch_bounds__(kLhsThreads) void quant_rows_kernel(
       if constexpr (SRC == kSrcSiluMul) {
         const float4 u0 = *reinterpret_cast<const float4*>(b + row + i);
         const float4 u1 = *reinterpret_cast<const float4*>(b + row + i + 4);
-        x0.x = x0.x / (1.0f + expf(-x0.x)) * u0.x;
-        x0.y = x0.y / (1.0f + expf(-x0.y)) * u0.y;
-        x0.z = x0.z / (1.0f + expf(-x0.z)) * u0.z;
-        x0.w = x0.w / (1.0f + expf(-x0.w)) * u0.w;
-        x1.x = x1.x / (1.0f + expf(-x1.x)) * u1.x;
-        x1.y = x1.y / (1.0f + expf(-x1.y)) * u1.y;
-        x1.z = x1.z / (1.0f + expf(-x1.z)) * u1.z;
-        x1.w = x1.w / (1.0f + expf(-x1.w)) * u1.w;
+        x0.x = silu_mul(x0.x, u0.x);
+        x0.y = silu_mul(x0.y, u0.y);
+        x0.z = silu_mul(x0.z, u0.z);
+        x0.w = silu_mul(x0.w, u0.w);
+        x1.x = silu_mul(x1.x, u1.x);
+        x1.y = silu_mul(x1.y, u1.y);
+        x1.z = silu_mul(x1.z, u1.z);
+        x1.w = silu_mul(x1.w, u1.w);
       }
       v[r][0] = x0.x; v[r][1] = x0.y; v[r][2] = x0.z; v[r][3] = x0.w;
       v[r][4] = x1.x; v[r][5] = x1.y; v[r][6] = x1.z; v[r][7] = x1.w;

@@ -328,6 +328,31 @@ def test_splitk_matches_oracle_and_plain(pkg, orc, m, k, n):
     assert np.array_equal(host(pkg.matmul_quantized_splitk(ws, packed, m, k, n, scratch=tiny)), plain)
 
 
+@pytest.mark.parametrize("m,k,n", [(33, 64, 48), (130, 160, 100), (256, 1536, 8960), (512, 1536, 8960),
+                                   (1100, 1280, 5120), (300, 4096, 2560)])
+def test_silu_pair_matches_the_three_operators(pkg, orc, m, k, n):
+    # gate Linear, up Linear, silu(gate) * up in one launch: against the separate operators of the library
+    # (same products, same f32 expression) and against the oracle's two Linears; N = 48 and 100 end inside
+    # a tile's half, K = 160 leaves padding in the last stage; the shapes cover the three tile choices
+    wg, wu = make_weights(n, k, seed=n), make_weights(n, k, seed=n + 1)
+    x = make_acts(m, k, seed=m, outlier_frac=0.02)
+    bg, bu = bias_for(n, True, seed=3), bias_for(n, True, seed=4)
+    (u4g, scg), (u4u, scu) = orc.quant_rhs(wg), orc.quant_rhs(wu)
+    pg = pkg.repack_native(dev(u4g), dev(scg.view(np.int16)), dev(bg), n, k)
+    pu = pkg.repack_native(dev(u4u), dev(scu.view(np.int16)), dev(bu), n, k)
+    ws = pkg.quant_lhs(dev(x))
+    got = host(pkg.matmul_quantized_silu_pair(ws, pg, pu, m, k, n))
+    yg = pkg.matmul_quantized(ws, pg, m, k, n, kernel=pkg.KERNEL_GEMM_F16_TILE0 + 2)
+    yu = pkg.matmul_quantized(ws, pu, m, k, n, kernel=pkg.KERNEL_GEMM_F16_TILE0 + 2)
+    sep = host(pkg.op_silu_mul(yg, yu))
+    assert np.array_equal(got, sep)
+    rows = np.unique(np.concatenate([np.arange(0, m, 53), [m - 1]]))
+    rg = orc.linear(x[rows], u4g, scg, bias=bg, threads=8).astype(np.float64)
+    ru = orc.linear(x[rows], u4u, scu, bias=bu, threads=8).astype(np.float64)
+    ref = (rg / (1.0 + np.exp(-rg)) * ru).astype(np.float32)
+    assert max_abs_rel(got[rows], ref) <= TIGHT
+
+
 def test_f16_kernel_with_wide_scale_range(pkg, orc):
     # rows whose block scales differ by many octaves, and rows that are tiny or huge overall:
     # the per-row power-of-two normalisation must keep the f16 operands exact
