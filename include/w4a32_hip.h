@@ -125,7 +125,7 @@ int w4a32_matmul_quantized(float* d_y, const void* d_ws, const void* d_packed, i
 /* Same product with the kernel named by the caller (tests and benchmarks compare them).
  * The reference picks its micro-kernel the same way, by a tile id argument
  * (KaiLinear_f32_qai8dxp_qsi4c32p_mxk_nxk::Tiles, kai_linear.hpp:76-118). */
-#define W4A32_KERNEL_AUTO 0       /* M <= 8: GEMV, M <= 32: int8 MFMA, else f16 MFMA */
+#define W4A32_KERNEL_AUTO 0       /* M <= 8: GEMV, else f16 MFMA */
 #define W4A32_KERNEL_GEMV 1       /* v_dot4 decode kernel, M <= 8 */
 #define W4A32_KERNEL_GEMM_I8 2    /* int8 MFMA, exact int32 block sums, any M */
 #define W4A32_KERNEL_GEMM_F16 3   /* f16 MFMA on exact f16 operands, M > 8; tile shape by size */
@@ -165,17 +165,17 @@ int w4a32_matmul_grouped(float* const* d_y, const float* d_x, const void* const*
                          const int* N, int count, void* d_ws, int M, int K, void* stream);
 
 /* The grouped product on rows that are already quantised into d_ws (w4a32_quant_lhs or one of the
- * fused quantisers of w4a32_decoder.h): at M > 32 one launch of the prefill kernel over all the
+ * fused quantisers of w4a32_decoder.h): at M > 8 one launch of the prefill kernel over all the
  * Linears, else one product per Linear. */
 int w4a32_matmul_quantized_grouped(float* const* d_y, const void* d_ws, const void* const* d_packed,
                                    const int* N, int count, int M, int K, void* stream);
 
-/* d_act[M][N] = silu(x W_gate^T + b_gate) * (x W_up^T + b_up) on rows already quantised into d_ws, M > 32:
+/* d_act[M][N] = silu(x W_gate^T + b_gate) * (x W_up^T + b_up) on rows already quantised into d_ws, M > 8:
  * the MLP's gate_proj, up_proj, SiLU and multiply (modeling_ds_qwen2.hpp:47-54) in one launch of the
  * prefill kernel. A wavefront computes both Linears for the same outputs and stores only their product,
  * so neither Linear's [M][N] result is written or read back. Each factor is the value
  * w4a32_matmul_quantized gives (same products and summation order), combined with w4a32_op_silu_mul's
- * expression. W4A32_ESHAPE for M <= 32. */
+ * expression. W4A32_ESHAPE for M <= 8. */
 int w4a32_matmul_quantized_silu_pair(float* d_act, const void* d_ws, const void* d_gate, const void* d_up,
                                      int M, int K, int N, void* stream);
 

@@ -276,7 +276,7 @@ def matmul_quantized(ws, packed, M, K, N, out=None, kernel=KERNEL_AUTO):
 
 
 def matmul_quantized_grouped(ws, packed_list, Ns, M, K, outs=None):
-    """Several Linears on rows already quantised into ws (one launch at M > 32)."""
+    """Several Linears on rows already quantised into ws (one launch at M > 8)."""
     import torch
 
     n = len(Ns)
@@ -290,7 +290,7 @@ def matmul_quantized_grouped(ws, packed_list, Ns, M, K, outs=None):
 
 
 def matmul_quantized_silu_pair(ws, gate, up, M, K, N, out=None):
-    """silu(gate Linear) * (up Linear) on rows already quantised into ws, one launch (M > 32)."""
+    """silu(gate Linear) * (up Linear) on rows already quantised into ws, one launch (M > 8)."""
     import torch
 
     y = out if out is not None else torch.empty((M, N), dtype=torch.float32, device="cuda")

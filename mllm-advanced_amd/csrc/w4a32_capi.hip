@@ -172,7 +172,7 @@ int w4a32_matmul_quantized_ex(float* d_y, const void* d_ws, const void* d_packed
 }
 
 size_t w4a32_splitk_scratch_bytes(int M, int K, int N) {
-  if (M <= 32 || shape_ok(N, K)) return 0;
+  if (M <= w4::kGemvMaxM || shape_ok(N, K)) return 0;
   const w4::SplitPlan p = w4::splitk_plan(M, K, N);
   return p.parts > 1 ? (size_t)p.parts * M * N * sizeof(float) : 0;
 }
@@ -228,7 +228,7 @@ int w4a32_matmul_grouped(float* const* d_y, const float* d_x, const void* const*
     return from_hip(w4::launch_gemv_group(d_y, d_x, K, pk, N, count, M, K, s));
   }
   // other sizes: quantise the rows once, then one launch of the f16 kernel over all the Linears
-  // (M > 32) or one product per Linear
+  // (M > 8) or one product per Linear
   if (int e = w4a32_quant_lhs(d_x, M, K, K, d_ws, stream)) return e;
   return w4a32_matmul_quantized_grouped(d_y, d_ws, d_packed, N, count, M, K, stream);
 }
@@ -243,7 +243,7 @@ int w4a32_matmul_quantized_grouped(float* const* d_y, const void* d_ws, const vo
     if (!aligned(d_packed[i], 16) || !aligned(d_y[i], 4)) return W4A32_EINVAL;
   }
   if (!aligned(d_ws, 256)) return W4A32_EINVAL;
-  if (M > 32 && count > 1) {
+  if (M > w4::kGemvMaxM && count > 1) {
     const uint8_t* pk[W4A32_MAX_GROUP];
     for (int i = 0; i < count; ++i) pk[i] = static_cast<const uint8_t*>(d_packed[i]);
     return from_hip(w4::launch_gemm_group(d_y, static_cast<const uint8_t*>(d_ws), pk, N, count, M, K,
@@ -259,7 +259,7 @@ int w4a32_matmul_quantized_silu_pair(float* d_act, const void* d_ws, const void*
                                      int M, int K, int N, void* stream) {
   if (!d_act || !d_ws || !d_gate || !d_up || M <= 0) return W4A32_EINVAL;
   if (int e = shape_ok(N, K)) return e;
-  if (M <= 32) return W4A32_ESHAPE;  // the f16 product kernel's sizes only
+  if (M <= w4::kGemvMaxM) return W4A32_ESHAPE;  // the f16 product kernel's sizes only
   if (!aligned(d_ws, 256) || !aligned(d_gate, 16) || !aligned(d_up, 16) || !aligned(d_act, 4)) {
     return W4A32_EINVAL;
   }

@@ -131,7 +131,7 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
     // both are dead
     const size_t lend = g.up_off - g.gate_off + sizeof(float) * (size_t)c->max_batch_tokens * I;
     // Prefill sizes: the operator in front of a Linear runs inside that Linear's row quantiser.
-    const bool fuse_rows = M > 32 && w4::quant_rows_fusable(std::max(H, I));
+    const bool fuse_rows = M > w4::kGemvMaxM && w4::quant_rows_fusable(std::max(H, I));
     // h += mlp output of the previous layer; xn = norm(h)
     {
       float* ys[3] = {q, k, v};
@@ -174,7 +174,7 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
         W4_TRY(w4a32_matmul_grouped(ys, xn, ps, ns, 2, ws, M, H, stream));
       }
     }
-    if (M > 32) {
+    if (M > w4::kGemvMaxM) {
       if (fuse_rows) {
         W4_TRY(w4a32_quant_lhs(act, M, I, I, ws, stream));
       } else {

@@ -2,7 +2,7 @@
 //
 // Two kernels:
 //
-//  * gemm_f16_kernel (M > 32): v_mfma_f32_32x32x16_f16 on EXACT f16 operands. The activation
+//  * gemm_f16_kernel (M > 8): v_mfma_f32_32x32x16_f16 on EXACT f16 operands. The activation
 //    operand is a_q - zp (an integer in [-255, 255]); the weight operand is q * scale / 2^E_n
 //    (4 + 8 significant bits), dequantised ONCE per workgroup from the 4-bit tiles into LDS,
 //    already in MFMA fragment order. Every product is exact in f32; only the order of the f32
@@ -10,7 +10,8 @@
 //    is what lets the matrix cores run ahead of the VALU: with int8 MFMA every 32-k block would
 //    need a convert + scale FMA per accumulator register, and that is VALU-bound.
 //
-//  * gemm_i8_kernel (9 <= M <= 32, and a cross-check for the other): integer path.
+//  * gemm_i8_kernel (selectable by number, a cross-check for the other): integer path. It served
+//    9 <= M <= 32 until the f16 kernel's small tiles made that one 2-3 x faster there too.
 //
 // Integer path: v_mfma_i32_16x16x32_i8. One MFMA spans exactly one scale block (32 k), so the
 // block sums are exact int32, as in the reference's scalar model
@@ -818,7 +819,7 @@ static int choose_f16_tile(long tiles, long tiles160, int K) {
 // 1.0 PFLOP/s). The 64 x 64 tile no longer wins anywhere; it stays selectable by number.
 hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                        int kernel, hipStream_t s) {
-  if (kernel == kKernelGemmI8 || (kernel == kKernelAuto && M <= 32)) {
+  if (kernel == kKernelGemmI8) {
     return launch_gemm_i8(y, ws, packed, M, K, N, s);
   }
   if (kernel >= kKernelGemmF16Tile && kernel < kKernelGemmF16Tile + kGemmF16Tiles) {
@@ -868,7 +869,7 @@ SplitPlan splitk_plan(int M, int K, int N) {
   SplitPlan p{2, 1};
   const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
   const int nstages = (K + kF16BK - 1) / kF16BK;
-  if (M <= 32 || nstages < 96 || tiles > 256) return p;
+  if (M <= kGemvMaxM || nstages < 96 || tiles > 256) return p;
   p.parts = tiles <= 24 ? 10 : tiles <= 96 ? 5 : 4;
   if (tiles <= 16) {
     p.tile = 1;  // 128 x 64: twice the workgroups (M = 128: 19 -> 16 us)

@@ -78,7 +78,7 @@ hipError_t launch_gemm_pair(float* act, const uint8_t* ws, const uint8_t* gate, 
                             int K, int N, hipStream_t s);
 hipError_t launch_gemm_splitk(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                               float* part, hipStream_t s);
-// several Linears on the same quantised rows in one launch of the f16 kernel (M > 32)
+// several Linears on the same quantised rows in one launch of the f16 kernel (M > 8)
 hipError_t launch_gemm_group(float* const* y, const uint8_t* ws, const uint8_t* const* packed,
                              const int* N, int count, int M, int K, hipStream_t s);
 

@@ -301,7 +301,8 @@ def test_gemm_each_kernel_matches_oracle(pkg, orc, kernel, m, k, n):
     assert err <= GEMM_TOL and err <= TIGHT, (kernel, err)
 
 
-@pytest.mark.parametrize("m,k,n", [(512, 8960, 1536), (100, 8960, 50), (300, 6144, 272), (1024, 8960, 1536),
+@pytest.mark.parametrize("m,k,n", [(512, 8960, 1536), (100, 8960, 50), (16, 8960, 1536), (300, 6144, 272),
+                                   (1024, 8960, 1536),
                                    (1100, 6144, 1536), (64, 256, 64)])
 def test_splitk_matches_oracle_and_plain(pkg, orc, m, k, n):
     # few tiles and a long K: the k range of a tile is dealt to several workgroups and the parts are
@@ -328,7 +329,7 @@ def test_splitk_matches_oracle_and_plain(pkg, orc, m, k, n):
     assert np.array_equal(host(pkg.matmul_quantized_splitk(ws, packed, m, k, n, scratch=tiny)), plain)
 
 
-@pytest.mark.parametrize("m,k,n", [(33, 64, 48), (130, 160, 100), (256, 1536, 8960), (512, 1536, 8960),
+@pytest.mark.parametrize("m,k,n", [(9, 64, 48), (33, 64, 48), (130, 160, 100), (256, 1536, 8960), (512, 1536, 8960),
                                    (1100, 1280, 5120), (300, 4096, 2560)])
 def test_silu_pair_matches_the_three_operators(pkg, orc, m, k, n):
     # gate Linear, up Linear, silu(gate) * up in one launch: against the separate operators of the library
