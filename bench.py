@@ -313,7 +313,7 @@ def main():
     if not args.no_gemm:
         prefill = {}
         with torch.cuda.stream(stream):
-            for M in (512, 2048):
+            for M in (128, 512, 2048):
                 per, tot_flop, tot_ms, tot_kms = {}, 0.0, 0.0, 0.0
                 for idx, (name, K, N, b) in enumerate(LAYER_LINEARS):
                     lin = layers[0][idx]
