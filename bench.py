@@ -20,6 +20,7 @@ bounded sample.
 import argparse
 import importlib
 import json
+import numpy as np
 import os
 import sys
 import time
@@ -547,6 +548,27 @@ def main():
                          f"({layer_bytes} algorithmic bytes per pass), scalar C restatement of the "
                          f"reference path; the reference runs decode (M=1) as a single task",
                "host_cpus": os.cpu_count()}
+        # the same restatement with its output columns dealt to threads (the reference itself splits rows
+        # only, so it gains nothing at M=1): 4 threads = the reference's default pool, 16 = this box's share
+        threaded = {}
+        for nthr in (4, 16):
+            reps_t, t0 = 0, time.perf_counter()
+            while time.perf_counter() - t0 < 3.0:
+                for (l, u4, sc, bias) in host:
+                    orc.linear(xs[l.K], u4, sc, bias=bias, threads=nthr)
+                reps_t += 1
+            threaded[f"threads_{nthr}"] = round(layer_bytes * reps_t / (time.perf_counter() - t0) / 1e9, 3)
+        # prefill: gate_proj at M=128 (the reference deals rows to its 4 workers)
+        (l, u4, sc, bias) = host[4]
+        xp = np.random.default_rng(1).standard_normal((128, l.K)).astype(np.float32)
+        t0 = time.perf_counter()
+        orc.linear(xp, u4, sc, bias=bias, threads=4)
+        dtp = time.perf_counter() - t0
+        extra["cpu_baseline_more"] = {"decode_GBps_by_threads": threaded,
+                                      "prefill_gate_proj_M128_4_threads_TFLOPs":
+                                          round(2.0 * 128 * l.N * l.K / dtp / 1e12, 5),
+                                      "note": "scalar C restatement; columns (decode) or rows x columns "
+                                              "(prefill) dealt to OpenMP threads"}
 
     out = {
         "metric": "W4 GEMV HBM GB/s (M=1)", "value": round(value, 1), "unit": "GB/s",
