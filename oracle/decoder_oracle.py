@@ -75,13 +75,16 @@ def silu_mul(g, u):
 class Linear:
     """One W4A32 Linear: quantised once by the oracle's quantiser, applied by the oracle's matmul."""
 
+    threads = 1   # of the C matmul (rows x columns dealt to threads: same results); tests at full shapes raise it
+
     def __init__(self, w, bias=None):
         self.n, self.k = w.shape
         self.u4, self.scales = orc.quant_rhs(np.ascontiguousarray(w, dtype=F))
         self.bias = None if bias is None else np.ascontiguousarray(bias, dtype=F)
 
     def __call__(self, x):
-        return orc.linear(np.ascontiguousarray(x, dtype=F), self.u4, self.scales, bias=self.bias)
+        return orc.linear(np.ascontiguousarray(x, dtype=F), self.u4, self.scales, bias=self.bias,
+                          threads=Linear.threads)
 
 
 class Decoder:
