@@ -88,6 +88,14 @@ HipBackend::~HipBackend() {
   }
 }
 
+Tensor& HipBackend::scratch(size_t bytes) {
+  if (scratch_.isNil() || scratch_.bytes() < bytes) {
+    synchronize();  // nothing in flight may still read the old buffer when it is freed
+    scratch_ = Tensor::empty({static_cast<int32_t>(bytes)}, kInt8, kHIP).alloc();
+  }
+  return scratch_;
+}
+
 void HipBackend::synchronize() const {
   MLLM_CHECK_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream_)));
 }

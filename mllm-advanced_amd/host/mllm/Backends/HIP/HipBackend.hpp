@@ -52,8 +52,14 @@ class HipBackend final : public BackendBase {
   [[nodiscard]] void* stream() const { return stream_; }  // hipStream_t
   void synchronize() const;
 
+  // Device memory that an op may use while its kernels run (partial sums of a product whose k range is
+  // dealt to several workgroups): one buffer for the backend, grown on demand, contents undefined. All ops
+  // run in order on the backend's one stream, so the next borrower cannot overlap the previous one.
+  Tensor& scratch(size_t bytes);
+
  private:
   void* stream_ = nullptr;
+  Tensor scratch_;
 };
 
 std::shared_ptr<HipBackend> createHipBackend();

@@ -143,8 +143,19 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
   if (workspace_.isNil() || workspace_.bytes() < need) {
     workspace_ = Tensor::empty({static_cast<int32_t>(need)}, kInt8, kHIP).alloc();
   }
+  auto& hb = currentHipBackend();
+  if (const size_t lend = w4a32_splitk_scratch_bytes(M, K, N)) {
+    // few output tiles and a long K (down_proj at prefill sizes): the library deals each tile's k range to
+    // several workgroups when it is lent room for their partial sums
+    Tensor& scratch = hb.scratch(lend);
+    check(w4a32_quant_lhs(x.ptr<float>(), M, K, K, workspace_.ptr<void>(), hb.stream()), "w4a32_quant_lhs");
+    check(w4a32_matmul_quantized_splitk(y.ptr<float>(), workspace_.ptr<void>(), weight_.ptr<void>(), M, K, N,
+                                        scratch.ptr<void>(), scratch.bytes(), hb.stream()),
+          "w4a32_matmul_quantized_splitk");
+    return;
+  }
   check(w4a32_matmul(y.ptr<float>(), x.ptr<float>(), weight_.ptr<void>(), workspace_.ptr<void>(), M, K,
-                     N, currentHipBackend().stream()),
+                     N, hb.stream()),
         "w4a32_matmul");
   // Stays asynchronous on the backend's stream: a host consumer goes through D2H, which waits.
 }
