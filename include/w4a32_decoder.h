@@ -90,9 +90,9 @@ int w4a32_op_attention(const float* d_q, const float* d_kcache, const float* d_v
 /* The same operator for M > 1 rows with scratch lent by the caller: with at least
  * w4a32_op_attention_prefill_scratch_bytes(M, n_heads) bytes at d_part (16-byte aligned; contents need
  * not be kept or cleared) and at most 128 (head, block of 32 queries) pairs, the keys of a query block are
- * dealt to up to 8 workgroups and a second launch combines their results (short prompts, or few rows that
- * continue a long context, would otherwise use a fraction of the CUs); else it runs as w4a32_op_attention
- * does. */
+ * dealt to up to 8 workgroups and the last of them to finish combines their results (short prompts, or few
+ * rows that continue a long context, would otherwise use a fraction of the CUs; the arrival counters at the
+ * head of d_part are cleared by a small launch first); else it runs as w4a32_op_attention does. */
 size_t w4a32_op_attention_prefill_scratch_bytes(int M, int n_heads);
 int w4a32_op_attention_prefill(const float* d_q, const float* d_kcache, const float* d_vcache,
                                float* d_out, int M, int n_heads, int n_kv_heads, int head_dim,

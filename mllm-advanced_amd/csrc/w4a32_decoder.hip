@@ -41,11 +41,15 @@ ScratchGeom scratch_geom(int n_heads) {
 
 // Everything a decoder instance keeps on the device, in one caller-owned allocation.
 struct StateGeom {
-  size_t pos_off, scratch_off, sin_off, cos_off, kcache_off, vcache_off;
+  size_t pos_off, scratch_off, pfcnt_off, sin_off, cos_off, kcache_off, vcache_off;
   size_t h_off, xn_off, q_off, k_off, v_off, attn_off, delta_off, gate_off, up_off, act_off;
   size_t logits_off, ws_off, total;
   size_t cache_layer;  // floats per layer in each cache
 };
+
+size_t pf_counters(const w4a32_decoder_config* c) {
+  return (size_t)c->n_heads * ((c->max_batch_tokens + 31) / 32);
+}
 
 bool config_ok(const w4a32_decoder_config* c) {
   if (!c) return false;
@@ -70,6 +74,8 @@ StateGeom state_geom(const w4a32_decoder_config* c) {
   };
   g.pos_off = take(sizeof(int));
   g.scratch_off = take(scratch_geom(c->n_heads).total);
+  // arrival counters of the prefill attention, one per (head, block of 32 queries)
+  g.pfcnt_off = take(sizeof(unsigned int) * pf_counters(c));
   g.sin_off = take(sizeof(float) * c->max_seq * (c->head_dim / 2));
   g.cos_off = take(sizeof(float) * c->max_seq * (c->head_dim / 2));
   g.cache_layer = kvd * c->max_seq;
@@ -157,7 +163,8 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
     } else {
       // the gate and up buffers are dead here: they hold the per-chunk results of long query blocks
       W4_TRY(from_hip(w4::launch_attention_prefill(q, kc, vc, attn, M, Hq, Hkv, c->max_seq, d_pos, 0, gate,
-                                                   lend, s)));
+                                                   lend, reinterpret_cast<unsigned int*>(st + g.pfcnt_off),
+                                                   s)));
     }
     W4_TRY(w4a32_matmul(delta, attn, lw.o, ws, M, qd, H, stream));
     // h += attention output; xn = norm(h)
@@ -383,7 +390,7 @@ int w4a32_op_attention(const float* d_q, const float* d_kcache, const float* d_v
         reinterpret_cast<unsigned int*>(sc + sg.counters_off), nullptr, nullptr, nullptr, nullptr, S(stream)));
   }
   return from_hip(w4::launch_attention_prefill(d_q, d_kcache, d_vcache, d_out, M, n_heads, n_kv_heads,
-                                               max_seq, d_pos0, pos0, nullptr, 0, S(stream)));
+                                               max_seq, d_pos0, pos0, nullptr, 0, nullptr, S(stream)));
 }
 
 size_t w4a32_op_attention_prefill_scratch_bytes(int M, int n_heads) {
@@ -402,7 +409,7 @@ int w4a32_op_attention_prefill(const float* d_q, const float* d_kcache, const fl
   if (d_part && reinterpret_cast<uintptr_t>(d_part) % 16 != 0) return W4A32_EINVAL;
   return from_hip(w4::launch_attention_prefill(d_q, d_kcache, d_vcache, d_out, M, n_heads, n_kv_heads,
                                                max_seq, d_pos0, pos0, static_cast<float*>(d_part),
-                                               part_bytes, S(stream)));
+                                               part_bytes, nullptr, S(stream)));
 }
 
 int w4a32_op_rope_attention_decode(const float* d_q, const float* d_k, const float* d_v,
@@ -477,6 +484,8 @@ int w4a32_decoder_init(const w4a32_decoder_config* cfg, void* d_state, void* str
   W4_TRY(from_hip(w4::launch_set_int(reinterpret_cast<int*>(st + g.pos_off), 0, s)));
   W4_TRY(from_hip(w4::launch_zero_u32(reinterpret_cast<unsigned int*>(st + g.scratch_off),
                                       cfg->n_heads + 1, s)));
+  W4_TRY(from_hip(w4::launch_zero_u32(reinterpret_cast<unsigned int*>(st + g.pfcnt_off),
+                                      (int)pf_counters(cfg), s)));
   return from_hip(w4::launch_rope_table(reinterpret_cast<float*>(st + g.sin_off),
                                         reinterpret_cast<float*>(st + g.cos_off), cfg->max_seq,
                                         cfg->head_dim, cfg->rope_theta, s));

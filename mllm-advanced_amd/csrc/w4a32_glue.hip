@@ -64,7 +64,6 @@ __device__ __forceinline__ int load_shared_across_wgs(const int* p) {
 }
 // All of this wavefront's stores above have reached the coherence point.
 __device__ __forceinline__ void stores_done() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); }
-
 }  // namespace
 
 // ---------------------------------------------------------------------------------------------
@@ -310,9 +309,10 @@ typedef float v16f32 __attribute__((ext_vector_type(16)));
 // workgroup each (blockIdx.z). A 32 x 32 block pair costs a SIMD 8192 clocks of f32 MFMA, and the last
 // query block of a 512-token prompt has 16 of them: on one CU that alone is 33k clocks, while a fair share
 // of the whole launch is 13k per SIMD. A query block with more than one chunk leaves (O, max, sum) per
-// chunk in `part` and attention_prefill_merge_kernel combines them; with one chunk it writes the output.
+// chunk in `part` and the last of its workgroups to finish combines them; with one chunk it writes the
+// output directly.
 constexpr int kPfMaxChunks = 8;
-constexpr int kPfPartStride = kHeadDim + 4;  // 128 dims, max, sum; rows stay 16-byte aligned
+constexpr int kPfItemFloats = 66 * 64;       // one chunk's hand-over: 64 O^T registers, max, sum x 64 lanes
 
 // Key blocks per chunk for a launch of M rows from position pos0 on: at least 4 (one per wavefront), at
 // most kPfMaxChunks chunks per query block and about kPfTargetChunks in all (every chunk has a whole pass
@@ -332,7 +332,7 @@ template <int kPfWaves, bool kSplit>
 __global__ __launch_bounds__(64 * kPfWaves) void attention_prefill_mfma_kernel(
     const float* __restrict__ q, const float* __restrict__ kc, const float* __restrict__ vc,
     float* __restrict__ out, int M, int Hq, int Hkv, int max_seq, const int* __restrict__ d_pos0,
-    int pos0, float scale, float* __restrict__ part) {
+    int pos0, float scale, float* __restrict__ part, unsigned int* counters) {
   extern __shared__ __align__(16) float s_merge[];  // [kPfWaves - 1][66][64]: O^T registers, max, sum
   const int h = blockIdx.x, qb = blockIdx.y;
   const int hk = h / (Hq / Hkv);
@@ -467,14 +467,48 @@ __global__ __launch_bounds__(64 * kPfWaves) void attention_prefill_mfma_kernel(
   }
   // lane = query; register v of block c = dim 4*(8*(v/4) + 4*hh + v%4) + c: four blocks -> one float4
   if (kSplit && nchunks > 1) {
-    float* dst = part + ((((size_t)h * gridDim.y + qb) * kPfMaxChunks + blockIdx.z) * 32 + j) * kPfPartStride;
+    // This chunk's (O^T registers, max, sum) go to scratch as [register][lane] (every store of the wavefront
+    // is 256 contiguous bytes), written through to the device's coherence point; the last workgroup of the
+    // query block to get here (arrival counter, left at 0) reads all chunks back and combines them.
+    float* mine = part + (((size_t)h * gridDim.y + qb) * kPfMaxChunks) * kPfItemFloats + lane;
+    float* dst = mine + (size_t)blockIdx.z * kPfItemFloats;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int row = 8 * (v >> 2) + 4 * hh + (v & 3);
-      *reinterpret_cast<float4*>(dst + 4 * row) = make_float4(o[0][v], o[1][v], o[2][v], o[3][v]);
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) store_shared_across_wgs(dst + (16 * c + v) * 64, o[c][v]);
+    store_shared_across_wgs(dst + 64 * 64, total_max);
+    store_shared_across_wgs(dst + 65 * 64, total_sum);
+    stores_done();
+    unsigned int* cnt = counters + (size_t)h * gridDim.y + qb;
+    unsigned int prev = 0;
+    if (lane == 0) prev = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    prev = __shfl(prev, 0, 64);
+    if (prev != (unsigned)nchunks - 1) return;
+    float cmax[kPfMaxChunks], csum[kPfMaxChunks];
+    float all_max = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < kPfMaxChunks; ++c) {
+      const float* ps = mine + (size_t)(c < nchunks ? c : 0) * kPfItemFloats;
+      cmax[c] = load_shared_across_wgs(ps + 64 * 64);
+      csum[c] = load_shared_across_wgs(ps + 65 * 64);
+      if (c >= nchunks) cmax[c] = -INFINITY;
+      all_max = fmaxf(all_max, cmax[c]);
     }
-    if (hh == 0) *reinterpret_cast<float2*>(dst + kHeadDim) = make_float2(total_max, total_sum);
-    return;
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o[c][v] = 0.0f;
+    total_sum = 0.0f;
+    for (int ch = 0; ch < nchunks; ++ch) {
+      const float wt = cmax[ch] == -INFINITY ? 0.0f : __expf(cmax[ch] - all_max);
+      total_sum += csum[ch] * wt;
+      const float* ps = mine + (size_t)ch * kPfItemFloats;
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[c][v] += load_shared_across_wgs(ps + (16 * c + v) * 64) * wt;
+    }
+    if (lane == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   if (32 * qb + j < M) {
     const float inv = 1.0f / total_sum;  // every query sees at least its own key
@@ -486,55 +520,6 @@ __global__ __launch_bounds__(64 * kPfWaves) void attention_prefill_mfma_kernel(
           make_float4(o[0][v] * inv, o[1][v] * inv, o[2][v] * inv, o[3][v] * inv);
     }
   }
-}
-
-// Combines the chunks of every query block that attention_prefill_mfma_kernel<.., true> cut in several:
-// thread = (query, 16 dims), the usual max / rescale rule over the chunks in their order.
-__global__ __launch_bounds__(256) void attention_prefill_merge_kernel(
-    const float* __restrict__ part, float* __restrict__ out, int M, int Hq, int max_seq,
-    const int* __restrict__ d_pos0, int pos0) {
-  const int h = blockIdx.x, qb = blockIdx.y;
-  if (d_pos0) pos0 = *d_pos0;
-  const int last_key = min(pos0 + min(32 * qb + 31, M - 1), max_seq - 1);
-  const int nkb = last_key / 32 + 1;
-  const int cb = prefill_chunk_blocks(pos0, M, max_seq, Hq);
-  const int nchunks = (nkb + cb - 1) / cb;
-  const int j = threadIdx.x >> 3, dg = threadIdx.x & 7;
-  if (nchunks <= 1 || 32 * qb + j >= M) return;
-  const float* src = part + ((((size_t)h * gridDim.y + qb) * kPfMaxChunks) * 32 + j) * kPfPartStride;
-  constexpr size_t kChunkStride = (size_t)32 * kPfPartStride;
-  float cmax[kPfMaxChunks], csum[kPfMaxChunks];
-  float total_max = -INFINITY;
-#pragma unroll
-  for (int c = 0; c < kPfMaxChunks; ++c) {
-    const float2 ms = *reinterpret_cast<const float2*>(src + (c < nchunks ? c : 0) * kChunkStride + kHeadDim);
-    cmax[c] = c < nchunks ? ms.x : -INFINITY;
-    csum[c] = ms.y;
-    total_max = fmaxf(total_max, cmax[c]);
-  }
-  float acc[16];
-#pragma unroll
-  for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
-  float total_sum = 0.0f;
-#pragma unroll
-  for (int c = 0; c < kPfMaxChunks; ++c) {
-    if (c < nchunks) {
-      const float wt = cmax[c] == -INFINITY ? 0.0f : __expf(cmax[c] - total_max);
-      total_sum += csum[c] * wt;
-      const float4* o4 = reinterpret_cast<const float4*>(src + c * kChunkStride + 16 * dg);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float4 o = o4[i];
-        acc[4 * i] += o.x * wt; acc[4 * i + 1] += o.y * wt;
-        acc[4 * i + 2] += o.z * wt; acc[4 * i + 3] += o.w * wt;
-      }
-    }
-  }
-  const float inv = 1.0f / total_sum;  // every query sees at least its own key
-  float4* dst = reinterpret_cast<float4*>(out + ((size_t)(32 * qb + j) * Hq + h) * kHeadDim + 16 * dg);
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-    dst[i] = make_float4(acc[4 * i] * inv, acc[4 * i + 1] * inv, acc[4 * i + 2] * inv, acc[4 * i + 3] * inv);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -947,29 +932,40 @@ hipError_t launch_rope_kv(float* q, const float* k, const float* v, const float*
   return hipGetLastError();
 }
 
+// Scratch of the chunked launch: arrival counters (one per head and query block, 256-byte aligned) in front
+// of the chunks' hand-over areas.
+static size_t pf_counter_bytes(int M, int Hq) {
+  return (sizeof(unsigned int) * (size_t)Hq * ((M + 31) / 32) + 255) / 256 * 256;
+}
 size_t attention_prefill_part_bytes(int M, int Hq) {
-  return sizeof(float) * (size_t)Hq * ((M + 31) / 32) * kPfMaxChunks * 32 * kPfPartStride;
+  return pf_counter_bytes(M, Hq) +
+         sizeof(float) * (size_t)Hq * ((M + 31) / 32) * kPfMaxChunks * kPfItemFloats;
 }
 
 // part: optional scratch of attention_prefill_part_bytes(M, Hq) bytes; with it, and when the query blocks
-// alone would leave half of the CUs idle, the key range of a query block is dealt to several workgroups.
-// Measured (12 heads; unsplit -> chunked): 256 rows at position 0: 19.2 -> 16.3 us, at 768: 46 -> 41;
-// 128 rows at 3000: 218 -> 65; 64 at 2000: 135 -> 39; 32 at 500: 38 -> 17. From 384 rows on the unsplit
-// kernel's 8 wavefronts with several key blocks each do better when the prompt continues a long context
-// (512 rows at 512: 49 against 62 us), so those sizes stay unsplit (512 rows at 0: 29.5 against 27).
+// alone would leave half of the CUs idle, the key range of a query block is dealt to several workgroups
+// and the last of them to finish combines their results.
+// counters: optional Hq * ceil(M / 32) words that are 0 and are left 0; without them the head of `part`
+// serves and is cleared by a launch of its own first.
+// Measured (12 heads; unsplit -> chunked, counters given): 256 rows at position 0: 19 -> 16 us, at 768:
+// 46 -> 40; 128 rows at 3000: 218 -> 64; 64 at 2000: 134 -> 39; 32 at 500: 38 -> 17. From 384 rows on the
+// unsplit kernel's 8 wavefronts with several key blocks each do better when the prompt continues a long
+// context (512 rows at 512: 49 against 63 us), so those sizes stay unsplit (512 rows at 0: 29.4 against 26).
 hipError_t launch_attention_prefill(const float* q, const float* kc, const float* vc, float* out,
                                     int M, int Hq, int Hkv, int max_seq, const int* d_pos0, int pos0,
-                                    float* part, size_t part_bytes, hipStream_t s) {
+                                    float* part, size_t part_bytes, unsigned int* counters, hipStream_t s) {
   const float scale = 1.0f / sqrtf((float)kHeadDim);
   if (M >= 16 && Hq * ((M + 31) / 32) <= 128 && part && part_bytes >= attention_prefill_part_bytes(M, Hq)) {
     constexpr int W = 4;
     const size_t lds = sizeof(float) * (W - 1) * 66 * 64;
     const dim3 grid(Hq, (M + 31) / 32, kPfMaxChunks);
+    if (!counters) {
+      counters = reinterpret_cast<unsigned int*>(part);
+      if (hipError_t e = launch_zero_u32(counters, Hq * ((M + 31) / 32), s); e != hipSuccess) return e;
+    }
+    float* areas = part + pf_counter_bytes(M, Hq) / sizeof(float);
     hipLaunchKernelGGL((attention_prefill_mfma_kernel<W, true>), grid, dim3(64 * W), lds, s, q, kc, vc, out,
-                       M, Hq, Hkv, max_seq, d_pos0, pos0, scale, part);
-    if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
-    hipLaunchKernelGGL(attention_prefill_merge_kernel, dim3(Hq, (M + 31) / 32), dim3(256), 0, s, part, out,
-                       M, Hq, max_seq, d_pos0, pos0);
+                       M, Hq, Hkv, max_seq, d_pos0, pos0, scale, areas, counters);
     return hipGetLastError();
   }
   if (M >= 256) {  // matrix-core kernel, 32 queries per workgroup; many key blocks: 8 wavefronts
@@ -980,12 +976,12 @@ hipError_t launch_attention_prefill(const float* q, const float* kc, const float
         e != hipSuccess)
       return e;
     hipLaunchKernelGGL((attention_prefill_mfma_kernel<W, false>), dim3(Hq, (M + 31) / 32), dim3(64 * W), lds,
-                       s, q, kc, vc, out, M, Hq, Hkv, max_seq, d_pos0, pos0, scale, nullptr);
+                       s, q, kc, vc, out, M, Hq, Hkv, max_seq, d_pos0, pos0, scale, nullptr, nullptr);
   } else if (M >= 16) {
     constexpr int W = 4;
     const size_t lds = sizeof(float) * (W - 1) * 66 * 64;
     hipLaunchKernelGGL((attention_prefill_mfma_kernel<W, false>), dim3(Hq, (M + 31) / 32), dim3(64 * W), lds,
-                       s, q, kc, vc, out, M, Hq, Hkv, max_seq, d_pos0, pos0, scale, nullptr);
+                       s, q, kc, vc, out, M, Hq, Hkv, max_seq, d_pos0, pos0, scale, nullptr, nullptr);
   } else {
     hipLaunchKernelGGL(attention_prefill_kernel, dim3(Hq, M), dim3(64), 0, s, q, kc, vc, out, Hq, Hkv,
                        max_seq, d_pos0, pos0, scale);

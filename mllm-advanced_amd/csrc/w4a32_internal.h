@@ -96,7 +96,7 @@ hipError_t launch_rope_kv(float* q, const float* k, const float* v, const float*
 size_t attention_prefill_part_bytes(int M, int Hq);
 hipError_t launch_attention_prefill(const float* q, const float* kc, const float* vc, float* out,
                                     int M, int Hq, int Hkv, int max_seq, const int* d_pos0, int pos0,
-                                    float* part, size_t part_bytes, hipStream_t s);
+                                    float* part, size_t part_bytes, unsigned int* counters, hipStream_t s);
 hipError_t launch_attention_decode(const float* q, float* kc, float* vc, float* out, int Hq, int Hkv,
                                    int max_seq, const int* d_pos0, int pos0, int nsplit, float* part,
                                    unsigned int* counters, const float* k_new, const float* v_new,
