@@ -98,6 +98,17 @@ __global__ __launch_bounds__(kLhsThreads) void quant_rows_kernel(
 
   float v[R][8];
   float ss = 0.0f;
+  // the norm weights do not depend on the row: requested with it, not behind the sum of squares
+  float4 g0[SRC == kSrcNorm ? R : 1], g1[SRC == kSrcNorm ? R : 1];
+  if constexpr (SRC == kSrcNorm) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int i = 8 * t + 8 * kLhsThreads * r;
+      const int ic = i < K ? i : 0;
+      g0[r] = *reinterpret_cast<const float4*>(norm_w + ic);
+      g1[r] = *reinterpret_cast<const float4*>(norm_w + ic + 4);
+    }
+  }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int i = 8 * t + 8 * kLhsThreads * r;
@@ -149,10 +160,8 @@ __global__ __launch_bounds__(kLhsThreads) void quant_rows_kernel(
     for (int r = 0; r < R; ++r) {
       const int i = 8 * t + 8 * kLhsThreads * r;
       if (i < K) {
-        const float4 g0 = *reinterpret_cast<const float4*>(norm_w + i);
-        const float4 g1 = *reinterpret_cast<const float4*>(norm_w + i + 4);
-        v[r][0] *= g0.x * rstd; v[r][1] *= g0.y * rstd; v[r][2] *= g0.z * rstd; v[r][3] *= g0.w * rstd;
-        v[r][4] *= g1.x * rstd; v[r][5] *= g1.y * rstd; v[r][6] *= g1.z * rstd; v[r][7] *= g1.w * rstd;
+        v[r][0] *= g0[r].x * rstd; v[r][1] *= g0[r].y * rstd; v[r][2] *= g0[r].z * rstd; v[r][3] *= g0[r].w * rstd;
+        v[r][4] *= g1[r].x * rstd; v[r][5] *= g1[r].y * rstd; v[r][6] *= g1[r].z * rstd; v[r][7] *= g1[r].w * rstd;
       }
     }
   }
