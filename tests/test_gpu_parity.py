@@ -428,5 +428,22 @@ def test_bad_arguments_return_error_codes(pkg):
     assert L.w4a32_matmul_quantized_ex(*args, 4, 64, 16, pkg.KERNEL_GEMM_F16, None) == -2
     assert L.w4a32_matmul_quantized_ex(*args, 16, 64, 16, pkg.KERNEL_GEMV, None) == -2
     assert L.w4a32_matmul_quantized_ex(*args, 4, 64, 16, 99, None) == -1
+    # one past the last named tile shape of the f16 kernel
+    assert L.w4a32_matmul_quantized_ex(*args, 16, 64, 16, pkg.KERNEL_GEMM_F16_TILE0 + pkg.GEMM_F16_TILES,
+                                       None) == -1
+    # the pair launch: decode row counts have no f16 activation copy; null and misaligned operands
+    act = torch.zeros((16, 16), device="cuda")
+    assert L.w4a32_matmul_quantized_silu_pair(act.data_ptr(), ws.data_ptr(), pk.data_ptr(), pk.data_ptr(),
+                                              8, 64, 16, None) == -2
+    assert L.w4a32_matmul_quantized_silu_pair(act.data_ptr(), ws.data_ptr(), None, pk.data_ptr(),
+                                              16, 64, 16, None) == -1
+    assert L.w4a32_matmul_quantized_silu_pair(act.data_ptr(), ws.data_ptr(), pk.data_ptr() + 4, pk.data_ptr(),
+                                              16, 64, 16, None) == -1
+    assert L.w4a32_matmul_quantized_silu_pair(act.data_ptr(), ws.data_ptr(), pk.data_ptr(), pk.data_ptr(),
+                                              16, 48, 16, None) == -2
+    # split-K: shapes the library does not split ask for no scratch
+    assert L.w4a32_splitk_scratch_bytes(8, 8960, 1536) == 0
+    assert L.w4a32_splitk_scratch_bytes(512, 1536, 1536) == 0
+    assert L.w4a32_splitk_scratch_bytes(512, 8960, 1536) == 5 * 512 * 1536 * 4
     with pytest.raises(pkg.W4A32Error):
         pkg._check(-2, "probe")
