@@ -29,9 +29,16 @@
  *                         RNE zero point, error bound, clamp)
  *   orc_matmul            pinned (exactly-representable inputs == numpy matmul,
  *                         K=32 brute force, row linearity, bias closed form)
- *   the adding of bias    pinned only by its closed form "+bias[n] after the
- *                         lhs scale": the reference test passes no bias, so
- *                         where the real kernel adds it is parity unpinned.
+ *   orc_linear_w4a32      the whole op (row quantiser, block dots, scales, bias,
+ *                         clamp) pinned bit for bit against a routine written
+ *                         elsewhere: PyTorch's aten::_dyn_quant_matmul_4bit
+ *                         (block 32, bf16 scales), whose portable C++ path is the
+ *                         Arm kernels' authors' own reference for this scheme -
+ *                         random rows with outliers, the quantiser's corner rows
+ *                         and the reference test's srand() inputs.
+ *   the adding of bias    "+bias[n] after the lhs scale": closed form, and equal
+ *                         to PyTorch's routine above. The reference test passes no
+ *                         bias, so the Arm kernel itself is not observed adding it.
  */
 #ifndef W4A32_ORACLE_H
 #define W4A32_ORACLE_H

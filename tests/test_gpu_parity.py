@@ -354,6 +354,26 @@ def test_silu_pair_matches_the_three_operators(pkg, orc, m, k, n):
     assert max_abs_rel(got[rows], ref) <= TIGHT
 
 
+@pytest.mark.skipif(not hasattr(torch.ops.aten, "_dyn_quant_matmul_4bit"),
+                    reason="this torch build has no aten::_dyn_quant_matmul_4bit")
+@pytest.mark.parametrize("m,k,n", [(1, 1536, 256), (8, 8960, 64), (64, 1536, 320), (300, 1280, 160)])
+def test_hip_path_matches_torch_dyn_quant_matmul(pkg, orc, m, k, n):
+    # the HIP op against PyTorch's own CPU routine for the same scheme (block 32, bf16 scales, dynamic
+    # per-row int8 activations), without the oracle in between; weights quantised by the HIP quantiser
+    w = make_weights(n, k, seed=n)
+    x = make_acts(m, k, seed=m, outlier_frac=0.05)
+    bias = bias_for(n, True)
+    u4d, scd = pkg.quant_rhs_native(dev(w))
+    packed = pkg.repack_native(u4d, scd, dev(bias), n, k)
+    y = host(pkg.matmul(dev(x), packed, n))
+    u4, sc = host(u4d), host(scd).view(np.uint16)
+    tw = torch.from_numpy(u4)
+    ts = torch.from_numpy(sc.view(np.int16)).view(torch.bfloat16)
+    tp = torch.ops.aten._dyn_quant_pack_4bit_weight(tw, ts, torch.from_numpy(bias), 32, k, n)
+    want = torch.ops.aten._dyn_quant_matmul_4bit(torch.from_numpy(x), tp, 32, k, n).numpy()
+    assert max_abs_rel(y, want) <= TIGHT
+
+
 def test_f16_kernel_with_wide_scale_range(pkg, orc):
     # rows whose block scales differ by many octaves, and rows that are tiny or huge overall:
     # the per-row power-of-two normalisation must keep the f16 operands exact

@@ -325,3 +325,70 @@ def test_reference_test_case_is_close_to_dense_matmul(orc):
     rms = float(np.sqrt(np.mean((y - dense) ** 2)))
     assert rms < 0.06 * float(np.sqrt(np.mean(dense ** 2))) + 0.5
     assert np.corrcoef(y.ravel(), dense.ravel())[0, 1] > 0.995
+
+
+# --------------------------------------------------------------------------- an independent library routine
+
+def torch_dyn_quant_linear(x, u4, sc_bits, bias):
+    """PyTorch's own W4 dynamic-quantised Linear (aten::_dyn_quant_pack_4bit_weight +
+    aten::_dyn_quant_matmul_4bit, block 32, bf16 scales): on this x86 build its portable C++ path,
+    written by the authors of the Arm kernels as the reference for the same qai8dxp x qsi4c32p
+    scheme. Same input format as the oracle's: u4 [N][K/2] with the even k in the low nibble,
+    bf16 scales [N][K/32], optional f32 bias."""
+    n, k = u4.shape[0], u4.shape[1] * 2
+    tw = torch.from_numpy(np.ascontiguousarray(u4))
+    ts = torch.from_numpy(np.ascontiguousarray(sc_bits).view(np.int16)).view(torch.bfloat16)
+    tb = None if bias is None else torch.from_numpy(np.ascontiguousarray(bias))
+    packed = torch.ops.aten._dyn_quant_pack_4bit_weight(tw, ts, tb, 32, k, n)
+    return torch.ops.aten._dyn_quant_matmul_4bit(torch.from_numpy(np.ascontiguousarray(x)), packed, 32, k,
+                                                 n).numpy()
+
+
+needs_torch_dynq = pytest.mark.skipif(not hasattr(torch.ops.aten, "_dyn_quant_matmul_4bit"),
+                                      reason="this torch build has no aten::_dyn_quant_matmul_4bit")
+
+
+@needs_torch_dynq
+@pytest.mark.parametrize("m,k,n,has_bias", [(1, 32, 4, False), (1, 64, 8, True), (3, 128, 16, True),
+                                            (8, 1536, 256, True), (4, 1536, 64, False), (2, 8960, 48, False),
+                                            (5, 1280, 40, True)])
+def test_oracle_equals_torch_dyn_quant_matmul(orc, m, k, n, has_bias):
+    # Row quantiser, zero point, integer block dots, bf16 scales, lhs scale, bias and clamp of the whole op
+    # against a routine this repository did not write: bit for bit, on random rows with outliers.
+    w = make_weights(n, k, seed=k + n)
+    x = make_acts(m, k, seed=m + k, outlier_frac=0.25)
+    bias = (np.random.default_rng(n).standard_normal(n) * 0.02).astype(np.float32) if has_bias else None
+    u4, sc = orc.quant_rhs(w)
+    got = orc.linear(x, u4, sc, bias=bias)
+    want = torch_dyn_quant_linear(x, u4, sc, bias)
+    assert np.array_equal(got, want)
+
+
+@needs_torch_dynq
+def test_oracle_equals_torch_dyn_quant_matmul_on_corner_rows(orc):
+    # the rows that pin the quantiser's special cases: all zero, constant, one-sided, symmetric (zero point
+    # -0.5 -> ties to even), exact .5 ties of x * scale, a lone huge outlier, denormal-small values
+    k, n = 128, 12
+    rng = np.random.default_rng(3)
+    rows = [np.zeros(k), np.full(k, 0.75), np.abs(rng.standard_normal(k)), -np.abs(rng.standard_normal(k)),
+            np.where(np.arange(k) % 2 == 0, 1.5, -1.5), np.linspace(-1.0, 1.0, k) * 127.5 / 255.0,
+            np.concatenate([[1000.0], rng.standard_normal(k - 1) * 1e-3]), rng.standard_normal(k) * 1e-30,
+            np.concatenate([[0.0, 255.0], np.arange(k - 2) + 0.5])]
+    x = np.stack(rows).astype(np.float32)
+    w = make_weights(n, k, seed=11)
+    w[0, :32] = 0.0                       # a zero block: scale -0.0, nibbles 8
+    w[1, 32:64] = 0.3                     # a constant block: every q = -8
+    u4, sc = orc.quant_rhs(w)
+    bias = np.linspace(-1.0, 1.0, n).astype(np.float32)
+    assert np.array_equal(orc.linear(x, u4, sc, bias=bias), torch_dyn_quant_linear(x, u4, sc, bias))
+    assert np.array_equal(orc.linear(x, u4, sc), torch_dyn_quant_linear(x, u4, sc, None))
+
+
+@needs_torch_dynq
+def test_reference_test_protocol_equals_torch_dyn_quant_matmul(orc):
+    # the reference's own test case (KaiLinearTest.hpp:391-427: M=1, K=N=1024, uniform[-1,1] from
+    # srand(4568) / srand(4572), no bias), which it compares with the Arm kernel to 1e-4
+    lhs = orc.fill_uniform_random(1, 1024, 4568)
+    rhs = orc.fill_uniform_random(1024, 1024, 4572)
+    u4, sc = orc.quant_rhs(rhs)
+    assert np.array_equal(orc.linear(lhs, u4, sc), torch_dyn_quant_linear(lhs, u4, sc, None))
