@@ -392,3 +392,31 @@ def test_reference_test_protocol_equals_torch_dyn_quant_matmul(orc):
     rhs = orc.fill_uniform_random(1024, 1024, 4572)
     u4, sc = orc.quant_rhs(rhs)
     assert np.array_equal(orc.linear(lhs, u4, sc), torch_dyn_quant_linear(lhs, u4, sc, None))
+
+
+@needs_torch_dynq
+def test_oracle_equals_torch_dyn_quant_matmul_on_many_small_cases(orc):
+    # 120 seeded cases: shapes with K = 32..416 (every multiple of 32), N = 1..24, M = 1..6; rows drawn from
+    # normal, uniform, heavy-tailed and sparse distributions at scales 1e-6..1e4; weights likewise
+    rng = np.random.default_rng(2026)
+    for case in range(120):
+        k = 32 * int(rng.integers(1, 14))
+        n, m = int(rng.integers(1, 25)), int(rng.integers(1, 7))
+        kind = case % 4
+        if kind == 0:
+            x = rng.standard_normal((m, k))
+        elif kind == 1:
+            x = rng.uniform(-1.0, 1.0, (m, k))
+        elif kind == 2:
+            x = rng.standard_cauchy((m, k))
+        else:
+            x = rng.standard_normal((m, k)) * (rng.uniform(0, 1, (m, k)) < 0.1)
+        x = (x * 10.0 ** rng.uniform(-6, 4, (m, 1))).astype(np.float32)
+        w = (rng.standard_normal((n, k)) * 10.0 ** rng.uniform(-4, 1, (n, 1))).astype(np.float32)
+        if case % 5 == 0:
+            w[:, :32] = 0.0
+        bias = rng.standard_normal(n).astype(np.float32) if case % 2 else None
+        u4, sc = orc.quant_rhs(w)
+        got = orc.linear(x, u4, sc, bias=bias)
+        want = torch_dyn_quant_linear(x, u4, sc, bias)
+        assert np.array_equal(got, want), (case, m, k, n, kind)
