@@ -351,6 +351,43 @@ def test_decoder_step_replays_from_a_graph(pkg):
         assert dec.position == 19
 
 
+def test_decoder_prefill_replays_from_a_graph(pkg):
+    """The prefill launches nothing that a capture cannot hold (no allocation, no memset; the position and the
+    arrival counters of the chunked attention live in the state and are left as they were found): captured
+    once for a prompt length, replayed with eager work in between, it gives the eager result every time."""
+    rng = np.random.default_rng(8)
+    H, Hq, Hkv, I, V, L = 256, 4, 2, 3072, 640, 2
+    weights = tiny_model(rng, H, Hq, Hkv, I, V, L)
+    n = 70                                        # three query blocks: the attention splits their keys
+    # (the decoder lends its gate and up buffers, 2 * n * I floats, which must hold the chunks' hand-over)
+    assert pkg.lib().w4a32_op_attention_prefill_scratch_bytes(n, Hq) <= 2 * n * I * 4
+    prompts = [dev(rng.integers(0, V, size=n).astype(np.int64)) for _ in range(3)]
+
+    eager = to_device_model(pkg, weights, Hq, Hkv, max_seq=128, max_batch_tokens=n)
+    want = []
+    for p in prompts:
+        eager.prefill(p)
+        want.append((int(eager.token), eager.logits.clone()))
+
+    dec = to_device_model(pkg, weights, Hq, Hkv, max_seq=128, max_batch_tokens=n)
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        buf = prompts[0].clone()                  # the captured launch reads its tokens from here
+        dec.prefill(buf)                          # warm-up outside the capture
+        s.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            dec.prefill(buf)
+        for rep in range(2):
+            for p, (tok, logits) in zip(prompts, want):
+                buf.copy_(p)
+                graph.replay()
+                s.synchronize()
+                assert int(dec.token) == tok and dec.position == n
+                assert torch.equal(dec.logits, logits), rep
+                _ = (dec.logits * 2).sum().item()  # unrelated eager work between replays
+
+
 @pytest.mark.parametrize("K,Ns,pair", [(1536, [1536, 256, 256], False), (1536, [8960, 8960], True),
                                          (1536, [151936], False), (8960, [1536], False), (256, [640], False)])
 def test_decode_linear_fusions_match_separate_operators(pkg, orc, K, Ns, pair):
