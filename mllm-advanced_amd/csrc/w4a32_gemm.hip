@@ -21,6 +21,8 @@
 // is 8 consecutive int8 of an activation row.
 #include "w4a32_internal.h"
 
+#include <type_traits>
+
 namespace w4 {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -277,8 +279,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
   // this workgroup's stages: [s_begin, nstages)
   int s_begin = 0, nstages = (K + kF16BK - 1) / kF16BK;
   if constexpr (SPLITK) {
-    s_begin = (int)((long)ks * nstages / ksplit);
-    nstages = (int)((long)(ks + 1) * nstages / ksplit);
+    // whole pairs of stages (one 128-k weight chunk): a range starts on an even stage, which makes the
+    // half of the chunk that a stage of the unrolled loop reads a compile-time constant
+    const int npairs = (nstages + 1) >> 1;
+    const int s_end = 2 * (int)((long)(ks + 1) * npairs / ksplit);
+    s_begin = 2 * (int)((long)ks * npairs / ksplit);
+    nstages = s_end < nstages ? s_end : nstages;
   }
 
   uint4 areg[D][AKB][WM][2];  // [ring slot][k-block][32-row tile][slice of the block]
@@ -316,31 +322,54 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
     bs_ptr[u] = hs + (size_t)nt * KC * kTileScaleBytes + 8 * j;
   }
 
-  // The steady-state loop must stay ONE basic block (the compiler can then wait for exactly
-  // the load it needs instead of draining all of them), so nothing below branches: stage
-  // numbers and k-blocks are clamped to valid addresses, and what must not contribute is
-  // multiplied by a zero scale (padded stages) or meets the zero nibbles and zero scales that
-  // pad every weight tile (k >= K).
+  // The loops must stay ONE basic block each (the compiler can then wait for exactly the load it
+  // needs instead of draining all of them), so nothing below branches. The steady-state loop runs
+  // while every stage it loads exists: its pointers advance by constants and no address is computed.
+  // The prologue and the last iterations load through the clamped forms below: stage numbers and
+  // k-blocks are clamped to valid addresses, and what must not contribute is multiplied by a zero
+  // scale (padded stages) or meets the zero nibbles and zero scales that pad every weight tile
+  // (k >= K). a_pos, bq_pos and bs_pos are the bytes by which the per-lane pointers have advanced.
+  int a_pos = 0, bq_pos = 0, bs_pos = 0;
   auto load_a_kb = [&](int s, int kbl, uint4 (&dst)[AKB][WM][2]) {
     const int sc = s < nstages ? s : nstages - 1;
     int blk = 2 * sc + (WK == 2 ? wk : kbl);
     blk = blk < KB ? blk : KB - 1;
-    const int off = blk * 2048;
+    const int off = blk * 2048 - a_pos;
 #pragma unroll
     for (int a = 0; a < WM; ++a) {
       dst[kbl][a][0] = *reinterpret_cast<const uint4*>(a_ptr[a] + off);
       dst[kbl][a][1] = *reinterpret_cast<const uint4*>(a_ptr[a] + off + 16);
     }
   };
+  // steady state: a_ptr stands at k-block 2 * (the stage to load) (+ wk)
+  auto load_a_kb_next = [&](int kbl, uint4 (&dst)[AKB][WM][2]) {
+#pragma unroll
+    for (int a = 0; a < WM; ++a) {
+      dst[kbl][a][0] = *reinterpret_cast<const uint4*>(a_ptr[a] + kbl * 2048);
+      dst[kbl][a][1] = *reinterpret_cast<const uint4*>(a_ptr[a] + kbl * 2048 + 16);
+    }
+  };
 
   auto load_b = [&](int s, uint2 (&q)[B_UNITS], uint32_t (&sc)[B_UNITS]) {
     const int st = s < nstages ? s : nstages - 1;
     const int kc = st >> 1, half = st & 1;
-    const int offq = kc * kTileBytes + 8 * half;
-    const int offs = kc * kTileScaleBytes + 4 * half;
+    const int offq = kc * kTileBytes + 8 * half - bq_pos;
+    const int offs = kc * kTileScaleBytes + 4 * half - bs_pos;
 #pragma unroll
     for (int u = 0; u < B_UNITS; ++u) {
       const u32x2 t2 = load_global<u32x2>(bq_ptr[u] + offq);  // (a table pointer is a generic one)
+      q[u] = make_uint2(t2.x, t2.y);
+      sc[u] = load_global<uint32_t>(bs_ptr[u] + offs);
+    }
+  };
+  // steady state: the pointers stand at the chunk of the iteration's first stage, `rel` (a constant
+  // after unrolling) is the stage to load counted from there
+  auto load_b_rel = [&](int rel, uint2 (&q)[B_UNITS], uint32_t (&sc)[B_UNITS]) {
+    const int offq = (rel >> 1) * kTileBytes + 8 * (rel & 1);
+    const int offs = (rel >> 1) * kTileScaleBytes + 4 * (rel & 1);
+#pragma unroll
+    for (int u = 0; u < B_UNITS; ++u) {
+      const u32x2 t2 = load_global<u32x2>(bq_ptr[u] + offq);
       q[u] = make_uint2(t2.x, t2.y);
       sc[u] = load_global<uint32_t>(bs_ptr[u] + offs);
     }
@@ -410,8 +439,18 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
   // With BE = 2 the barrier comes every second stage (four LDS buffers): the stage behind it finds its
   // first fragments requested under the previous stage's last products, and a lone workgroup on a CU
   // pays the barrier and that LDS round trip half as often.
+  //
+  // Dequantisation of a packed dword (eight two's complement nibbles n): (dword & 0x000F000F) ^ 0x64086408
+  // is the f16 pair 1024 + (n ^ 8) of nibbles 0 and 4 in one three-input bit operation, likewise
+  // 0x00F000F0 / 0x64806480 for 1024 + 16 (n ^ 8) of nibbles 1 and 5, and the same on the dword >> 8;
+  // minus 1032 (1152) that is n exactly, times the scale (scale / 16) the weight: 13 instructions for
+  // eight weights. The two constants sit in vector registers (an instruction reads one scalar operand).
+  uint32_t k_lo = 0x64086408u, k_hi = 0x64806480u;
+  asm volatile("" : "+v"(k_lo), "+v"(k_hi));
   h8 bf[2][WN];
-  for (int s_base = s_begin; s_base < nstages; s_base += U) {
+  // TAIL = false: every load of the U stages is in range and goes through the advancing pointers.
+  auto run_stages = [&](auto tail_tag, const int s_base) __attribute__((always_inline)) {
+    constexpr bool TAIL = decltype(tail_tag)::value;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int s = s_base + u;
@@ -437,30 +476,35 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
         for (int f = 0; f < LA; ++f) fetch(f, bbuf);
         __builtin_amdgcn_sched_barrier(0);  // requested first: their latency covers what follows
       }
-      // Inputs of the dequantisation (stage s + BE, in this stage's ring slot) move to temporaries,
-      // which frees the slot for its next load. A stage past the end (loaded from clamped addresses)
-      // gets scale 0.
+      // Inputs of the dequantisation (stage s + BE, in this stage's ring slot); the slot then takes its
+      // next load. A stage past the end (loaded from clamped addresses) gets scale 0.
       uint32_t dx[NDW];
       h2 dsc[NDW], dsc16[NDW];
       {
-        const uint32_t keep = s + BE < nstages ? 0xFFFFFFFFu : 0u;
+        const uint32_t keep = !TAIL || s + BE < nstages ? 0xFFFFFFFFu : 0u;
         const h2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
 #pragma unroll
         for (int q = 0; q < B_UNITS; ++q) {
-          const h2 s2 = __builtin_bit_cast(h2, sreg[slot][q] & keep);
+          const h2 s2 = __builtin_bit_cast(h2, TAIL ? sreg[slot][q] & keep : sreg[slot][q]);
           const h2 s2_16 = s2 * sixteenth;
           dsc[2 * q] = h2{s2[0], s2[0]};
           dsc16[2 * q] = h2{s2_16[0], s2_16[0]};
           dsc[2 * q + 1] = h2{s2[1], s2[1]};
           dsc16[2 * q + 1] = h2{s2_16[1], s2_16[1]};
-          dx[2 * q] = breg[slot][q].x ^ 0x88888888u;  // two's complement nibbles -> offset-8 nibbles
-          dx[2 * q + 1] = breg[slot][q].y ^ 0x88888888u;
+          dx[2 * q] = breg[slot][q].x;
+          dx[2 * q + 1] = breg[slot][q].y;
         }
       }
-      load_b(s + BE + D, breg[slot], sreg[slot]);
+      if constexpr (TAIL) {
+        load_b(s + BE + D, breg[slot], sreg[slot]);
+      } else {
+        load_b_rel(u + BE + D, breg[slot], sreg[slot]);
+      }
       __builtin_amdgcn_sched_barrier(0);
-      // dequant8() cut into four steps per dword d (unit d / 2, scale block d % 2)
-      h2 dp[NDW];
+      // Four steps per dword d (unit d / 2, scale block d % 2). A step never multiplies what it has just
+      // subtracted: a product that reads half of a register the instruction before it wrote costs a
+      // wait state.
+      h2 dlo[NDW], dhi[NDW];
       uint32_t dxh[NDW];
       uint4 dout[NDW];
       auto dq_step = [&](int idx) {
@@ -468,18 +512,18 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
         const h2 b1 = {(_Float16)1032.0f, (_Float16)1032.0f};
         const h2 b16 = {(_Float16)1152.0f, (_Float16)1152.0f};
         if (ph == 0) {
-          const h2 p0 = __builtin_bit_cast(h2, and_or(dx[d], 0x000F000Fu, 0x64006400u));
-          dp[d] = __builtin_bit_cast(h2, and_or(dx[d], 0x00F000F0u, 0x64006400u));
-          dout[d].x = __builtin_bit_cast(uint32_t, (p0 - b1) * dsc[d]);
+          dlo[d] = __builtin_bit_cast(h2, (dx[d] & 0x000F000Fu) ^ k_lo) - b1;
+          dhi[d] = __builtin_bit_cast(h2, (dx[d] & 0x00F000F0u) ^ k_hi) - b16;
         } else if (ph == 1) {
-          dout[d].y = __builtin_bit_cast(uint32_t, (dp[d] - b16) * dsc16[d]);
+          dout[d].x = __builtin_bit_cast(uint32_t, dlo[d] * dsc[d]);
+          dout[d].y = __builtin_bit_cast(uint32_t, dhi[d] * dsc16[d]);
           dxh[d] = dx[d] >> 8;
         } else if (ph == 2) {
-          const h2 p2 = __builtin_bit_cast(h2, and_or(dxh[d], 0x000F000Fu, 0x64006400u));
-          dp[d] = __builtin_bit_cast(h2, and_or(dxh[d], 0x00F000F0u, 0x64006400u));
-          dout[d].z = __builtin_bit_cast(uint32_t, (p2 - b1) * dsc[d]);
+          dlo[d] = __builtin_bit_cast(h2, (dxh[d] & 0x000F000Fu) ^ k_lo) - b1;
+          dhi[d] = __builtin_bit_cast(h2, (dxh[d] & 0x00F000F0u) ^ k_hi) - b16;
         } else {
-          dout[d].w = __builtin_bit_cast(uint32_t, (dp[d] - b16) * dsc16[d]);
+          dout[d].z = __builtin_bit_cast(uint32_t, dlo[d] * dsc[d]);
+          dout[d].w = __builtin_bit_cast(uint32_t, dhi[d] * dsc16[d]);
           *reinterpret_cast<uint4*>(frag_ptr(wbuf, d >> 1, d & 1)) = dout[d];
         }
       };
@@ -507,10 +551,47 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
             __builtin_amdgcn_sched_barrier(0);
           }
         }
-        if (sl & 1) load_a_kb(s + D, sl >> 1, areg[slot]);  // that k-block's registers are free now
+        if (sl & 1) {  // that k-block's registers are free now
+          if constexpr (TAIL) {
+            load_a_kb(s + D, sl >> 1, areg[slot]);
+          } else {
+            load_a_kb_next(sl >> 1, areg[slot]);
+          }
+        }
+      }
+      if constexpr (!TAIL) {
+#pragma unroll
+        for (int a = 0; a < WM; ++a) a_ptr[a] += 4096;
       }
     }
+    if constexpr (!TAIL) {
+#pragma unroll
+      for (int q = 0; q < B_UNITS; ++q) {
+        bq_ptr[q] += (U / 2) * kTileBytes;
+        bs_ptr[q] += (U / 2) * kTileScaleBytes;
+      }
+    }
+  };
+
+  int s_base = s_begin;
+  if (s_base + U + BE + D <= nstages) {
+    // a_ptr to the first stage the loop loads, the weight pointers to the chunk of its first stage
+    // (s_begin is even, and so is U: stage s_base + u lies u stages into that chunk)
+#pragma unroll
+    for (int a = 0; a < WM; ++a) a_ptr[a] += (size_t)(s_begin + D) * 4096 + (WK == 2 ? wk * 2048 : 0);
+#pragma unroll
+    for (int q = 0; q < B_UNITS; ++q) {
+      bq_ptr[q] += (size_t)(s_begin >> 1) * kTileBytes;
+      bs_ptr[q] += (size_t)(s_begin >> 1) * kTileScaleBytes;
+    }
+    // the last stage loaded is s_base + U - 1 + BE + D; BE >= 1 also keeps the activations' last
+    // k-block (absent when K / 32 is odd) out of this loop
+    for (; s_base + U + BE + D <= nstages; s_base += U) run_stages(std::false_type{}, s_base);
+    a_pos = (s_base + D) * 4096 + (WK == 2 ? wk * 2048 : 0);
+    bq_pos = (s_base >> 1) * kTileBytes;
+    bs_pos = (s_base >> 1) * kTileScaleBytes;
   }
+  for (; s_base < nstages; s_base += U) run_stages(std::true_type{}, s_base);
 
   // WK = 2: the two k-halves of an output block meet in LDS, one 32 x 32 block per wavefront and round
   // (4 KiB each, in the stage buffers). The first half keeps column blocks 0..BH-1 and hands over the
@@ -798,25 +879,28 @@ static hipError_t launch_f16_tile(int tile, float* y, const uint8_t* ws, const u
   return hipErrorInvalidValue;
 }
 
-// tiles: 128 x 128 tiles of the problem; tiles160: 128 x 160 tiles.
-static int choose_f16_tile(long tiles, long tiles160, int K) {
+// tiles: 128 x 128 tiles of the problem; tiles160: 128 x 160 tiles; tiles256: 256 x 128 tiles.
+static int choose_f16_tile(long tiles, long tiles160, long tiles256, int K) {
   if (tiles <= 128) return 4;
   if (tiles <= 256) return 6;
   // 128 x 160 tiles, two workgroups per CU: when they come to one or two per CU with few CUs left over
   const long slots = 256 * ((tiles160 + 255) / 256);
   if (tiles160 <= 512 && tiles160 * 100 >= slots * 85) return 5;
-  if (tiles >= 1400 || (K >= 4096 && tiles >= 320)) return 3;
+  // 256 x 128 tiles, two workgroups per CU: from three quarters of a full round on, for up to one per CU,
+  // and on a long K
+  if (tiles256 >= 384 || (tiles256 >= 160 && tiles256 <= 256) || (K >= 4096 && tiles >= 320)) return 3;
   return 2;
 }
 
 // Choice of tile shape, measured on MI355X at M = 128..8192 over the decoder and ViT shapes, by
-// the number of 128 x 128 tiles the problem has. Up to half a tile per CU the 128 x 64 tile doubles the
+// the number of tiles the problem has. Up to half a 128 x 128 tile per CU the 128 x 64 tile doubles the
 // workgroups; up to one tile per CU the workgroup is alone on its CU and the eight-wavefront
 // arrangement hides some of its latencies; a problem whose 128 x 160 tiles come to (nearly) one or two per
-// CU takes those. Beyond that 128 x 128 with three resident workgroups per CU is best, but there LDS bandwidth
-// bounds it (each B fragment feeds one product); with many tiles per CU (gate_proj from M = 3072 on,
-// down_proj from 4096 on) the 256 x 128 tile is 10-17 % faster (gate_proj at M = 8192: 270 -> 227 us,
-// 1.0 PFLOP/s). The 64 x 64 tile no longer wins anywhere; it stays selectable by number.
+// CU takes those. The 256 x 128 tile reads each B fragment for two products, where LDS bandwidth bounds
+// the 128-row tiles, and wins wherever its coarser tiles still fill the chip: gate_proj from M = 1536 on
+// (M = 1792: 60 -> 50 us, 990 TFLOP/s; M = 8192: 253 -> 208 us, 1.08 PFLOP/s), q/o from M = 4096 on,
+// down_proj from M = 3456 on; in between 128 x 128 with three resident workgroups per CU. The 64 x 64 tile
+// no longer wins anywhere; it stays selectable by number.
 hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                        int kernel, hipStream_t s) {
   if (kernel == kKernelGemmI8) {
@@ -828,22 +912,24 @@ hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M
   }
   const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
   const long tiles160 = (long)((M + 127) / 128) * ((N + 159) / 160);
-  return launch_f16_tile(choose_f16_tile(tiles, tiles160, K), y, ws, packed, M, K, N, nullptr, nullptr, 0,
+  const long tiles256 = (long)((M + 255) / 256) * ((N + 127) / 128);
+  return launch_f16_tile(choose_f16_tile(tiles, tiles160, tiles256, K), y, ws, packed, M, K, N, nullptr, nullptr, 0,
                          1, nullptr, s);
 }
 
 hipError_t launch_gemm_group(float* const* y, const uint8_t* ws, const uint8_t* const* packed,
                              const int* N, int count, int M, int K, hipStream_t s) {
   GemmGroup g{};
-  long tiles = 0, tiles160 = 0;
+  long tiles = 0, tiles160 = 0, tiles256 = 0;
   for (int i = 0; i < count; ++i) {
     g.y[i] = y[i];
     g.packed[i] = packed[i];
     g.N[i] = N[i];
     tiles += (long)((M + 127) / 128) * ((N[i] + 127) / 128);
     tiles160 += (long)((M + 127) / 128) * ((N[i] + 159) / 160);
+    tiles256 += (long)((M + 255) / 256) * ((N[i] + 127) / 128);
   }
-  return launch_f16_tile(choose_f16_tile(tiles, tiles160, K), nullptr, ws, nullptr, M, K, 0, &g, N, count, 1,
+  return launch_f16_tile(choose_f16_tile(tiles, tiles160, tiles256, K), nullptr, ws, nullptr, M, K, 0, &g, N, count, 1,
                          nullptr, s);
 }
 
@@ -853,7 +939,8 @@ hipError_t launch_gemm_pair(float* act, const uint8_t* ws, const uint8_t* gate, 
                             int K, int N, hipStream_t s) {
   const long tiles = (long)((M + 127) / 128) * ((2 * N + 127) / 128);
   if (tiles <= 128) return launch_f16_pair<4, 2, 2, 4>(act, ws, gate, up, M, K, N, s);
-  if (tiles >= 1000 || (K >= 4096 && tiles >= 320)) {  // 256 x 128 (M = 1024: 71 -> 69 us, 2048: 132 -> 127)
+  const long tiles256 = (long)((M + 255) / 256) * ((2 * N + 127) / 128);
+  if (tiles256 >= 384 || (K >= 4096 && tiles >= 320)) {  // 256 x 128, as for a single Linear
     return launch_f16_pair<4, 4, 1, 2, 2>(act, ws, gate, up, M, K, N, s);
   }
   return launch_f16_pair<4, 4, 2, 3>(act, ws, gate, up, M, K, N, s);
