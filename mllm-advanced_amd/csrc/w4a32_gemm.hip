@@ -448,9 +448,13 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
   uint32_t k_lo = 0x64086408u, k_hi = 0x64806480u;
   asm volatile("" : "+v"(k_lo), "+v"(k_hi));
   h8 bf[2][WN];
-  // TAIL = false: every load of the U stages is in range and goes through the advancing pointers.
-  auto run_stages = [&](auto tail_tag, const int s_base) __attribute__((always_inline)) {
-    constexpr bool TAIL = decltype(tail_tag)::value;
+  // Three forms of U stages. kSteady: every load is in range and goes through the advancing pointers.
+  // kClamped: any stage may lie past the end. kLast: the U stages are exactly the last ones, so what lies
+  // past the end is known at compile time and neither loaded nor dequantised.
+  constexpr int kSteady = 0, kClamped = 1, kLast = 2;
+  auto run_stages = [&](auto form_tag, const int s_base) __attribute__((always_inline)) {
+    constexpr int FORM = decltype(form_tag)::value;
+    constexpr bool TAIL = FORM != kSteady;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int s = s_base + u;
@@ -481,11 +485,11 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
       uint32_t dx[NDW];
       h2 dsc[NDW], dsc16[NDW];
       {
-        const uint32_t keep = !TAIL || s + BE < nstages ? 0xFFFFFFFFu : 0u;
+        const uint32_t keep = FORM != kClamped || s + BE < nstages ? 0xFFFFFFFFu : 0u;
         const h2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
 #pragma unroll
         for (int q = 0; q < B_UNITS; ++q) {
-          const h2 s2 = __builtin_bit_cast(h2, TAIL ? sreg[slot][q] & keep : sreg[slot][q]);
+          const h2 s2 = __builtin_bit_cast(h2, FORM == kClamped ? sreg[slot][q] & keep : sreg[slot][q]);
           const h2 s2_16 = s2 * sixteenth;
           dsc[2 * q] = h2{s2[0], s2[0]};
           dsc16[2 * q] = h2{s2_16[0], s2_16[0]};
@@ -495,10 +499,11 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
           dx[2 * q + 1] = breg[slot][q].y;
         }
       }
-      if constexpr (TAIL) {
-        load_b(s + BE + D, breg[slot], sreg[slot]);
-      } else {
+      const bool dequantise = FORM != kLast || u + BE < U;  // (after unrolling: a constant)
+      if constexpr (FORM == kSteady) {
         load_b_rel(u + BE + D, breg[slot], sreg[slot]);
+      } else {
+        if (FORM != kLast || u + BE + D < U) load_b(s + BE + D, breg[slot], sreg[slot]);
       }
       __builtin_amdgcn_sched_barrier(0);
       // Four steps per dword d (unit d / 2, scale block d % 2). A step never multiplies what it has just
@@ -546,25 +551,27 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
               }
             }
 #pragma unroll
-            for (int st = mi * NSTEP / kMfma; st < (mi + 1) * NSTEP / kMfma; ++st) dq_step(st);
+            for (int st = mi * NSTEP / kMfma; st < (mi + 1) * NSTEP / kMfma; ++st) {
+              if (dequantise) dq_step(st);
+            }
             ++mi;
             __builtin_amdgcn_sched_barrier(0);
           }
         }
         if (sl & 1) {  // that k-block's registers are free now
           if constexpr (TAIL) {
-            load_a_kb(s + D, sl >> 1, areg[slot]);
+            if (FORM != kLast || u + D < U) load_a_kb(s + D, sl >> 1, areg[slot]);
           } else {
             load_a_kb_next(sl >> 1, areg[slot]);
           }
         }
       }
-      if constexpr (!TAIL) {
+      if constexpr (FORM == kSteady) {
 #pragma unroll
         for (int a = 0; a < WM; ++a) a_ptr[a] += 4096;
       }
     }
-    if constexpr (!TAIL) {
+    if constexpr (FORM == kSteady) {
 #pragma unroll
       for (int q = 0; q < B_UNITS; ++q) {
         bq_ptr[q] += (U / 2) * kTileBytes;
@@ -586,12 +593,18 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
     }
     // the last stage loaded is s_base + U - 1 + BE + D; BE >= 1 also keeps the activations' last
     // k-block (absent when K / 32 is odd) out of this loop
-    for (; s_base + U + BE + D <= nstages; s_base += U) run_stages(std::false_type{}, s_base);
+    for (; s_base + U + BE + D <= nstages; s_base += U) {
+      run_stages(std::integral_constant<int, kSteady>{}, s_base);
+    }
     a_pos = (s_base + D) * 4096 + (WK == 2 ? wk * 2048 : 0);
     bq_pos = (s_base >> 1) * kTileBytes;
     bs_pos = (s_base >> 1) * kTileScaleBytes;
   }
-  for (; s_base < nstages; s_base += U) run_stages(std::true_type{}, s_base);
+  const bool whole = (nstages - s_begin) % U == 0;  // the stages come in whole iterations
+  for (; s_base + (whole ? U : 0) < nstages; s_base += U) {
+    run_stages(std::integral_constant<int, kClamped>{}, s_base);
+  }
+  if (whole) run_stages(std::integral_constant<int, kLast>{}, s_base);
 
   // WK = 2: the two k-halves of an output block meet in LDS, one 32 x 32 block per wavefront and round
   // (4 KiB each, in the stage buffers). The first half keeps column blocks 0..BH-1 and hands over the
