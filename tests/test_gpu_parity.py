@@ -277,7 +277,10 @@ def test_gemm_ragged_m(pkg, orc, m):
 
 @pytest.mark.parametrize("kernel", ["i8", "f16"] + [f"f16:{i}" for i in range(7)])
 @pytest.mark.parametrize("m,k,n", [(9, 32, 16), (40, 96, 50), (200, 160, 330), (128, 1536, 256),
-                                   (300, 1280, 3840), (512, 8960, 1536), (1024, 5120, 1280)])
+                                   (300, 1280, 3840), (512, 8960, 1536), (1024, 5120, 1280),
+                                   # a last 64-k stage that is half empty, behind whole and behind
+                                   # ragged unrolled iterations of the main loop
+                                   (70, 1760, 80), (150, 1632, 200)])
 def test_gemm_each_kernel_matches_oracle(pkg, orc, kernel, m, k, n):
     # both prefill kernels (and each tile shape of the f16 one) on the same inputs; K = 32, 96 and 160
     # leave padding inside a stage (an odd number of 32-k blocks: the second k-half of the last stage
@@ -303,10 +306,11 @@ def test_gemm_each_kernel_matches_oracle(pkg, orc, kernel, m, k, n):
 
 @pytest.mark.parametrize("m,k,n", [(512, 8960, 1536), (100, 8960, 50), (16, 8960, 1536), (300, 6144, 272),
                                    (1024, 8960, 1536),
-                                   (1100, 6144, 1536), (64, 256, 64)])
+                                   (1100, 6144, 1536), (64, 256, 64), (64, 6208, 96)])
 def test_splitk_matches_oracle_and_plain(pkg, orc, m, k, n):
     # few tiles and a long K: the k range of a tile is dealt to several workgroups and the parts are
-    # added by a second kernel; the last shape is one the library does not split (falls through)
+    # added by a second kernel; K = 256 is one the library does not split (falls through); K = 6208 is an
+    # odd number of stages (the ranges are whole pairs of stages, the last one ends on the odd stage)
     w = make_weights(n, k, seed=n)
     x = make_acts(m, k, seed=m, outlier_frac=0.02)
     bias = bias_for(n, True)
