@@ -64,7 +64,7 @@ def parse():
     ap.add_argument("--no-decoder", action="store_true", help="skip the whole-decoder tokens/s leg")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="a 256 MiB copy, then the decode kernel on gate_proj and lm_head and the "
-                         "prefill kernel on gate_proj (the run profiled under rocprofv3 --pmc)")
+                         "prefill kernel on gate_proj and down_proj (the run profiled under rocprofv3 --pmc)")
     return ap.parse_args()
 
 
@@ -196,6 +196,16 @@ def main():
             for _ in range(3):
                 L.w4a32_matmul(y.data_ptr(), x.data_ptr(), gate.packed.data_ptr(), ws.data_ptr(), M,
                                gate.K, gate.N, sptr)
+            # down_proj (K = 8960) at M = 512 through the 128 x 64 tile shape, plain kernel: 96 workgroups,
+            # each alone on its CU, 140 stages each (the launch whose instruction counters are profiled)
+            down = layers[0][6]
+            xd = torch.randn((M, down.K), generator=xgen, device="cuda")
+            wsd = torch.empty(pkg.workspace_bytes(M, down.K), dtype=torch.uint8, device="cuda")
+            yd = torch.empty((M, down.N), device="cuda")
+            L.w4a32_quant_lhs(xd.data_ptr(), M, down.K, down.K, wsd.data_ptr(), sptr)
+            for _ in range(3):
+                L.w4a32_matmul_quantized_ex(yd.data_ptr(), wsd.data_ptr(), down.packed.data_ptr(), M, down.K,
+                                            down.N, pkg.KERNEL_GEMM_F16_TILE0 + 4, sptr)
         torch.cuda.synchronize()
         print(json.dumps({"traffic_probe": {
             "copy_bytes_read": 256 << 20, "copy_bytes_written": 256 << 20,
