@@ -438,6 +438,46 @@ def test_golden_fixture(pkg):
     assert max_abs_rel(y, g["y"]) <= TIGHT
 
 
+def test_f16_kernel_forms_agree_with_the_integer_kernel_on_random_shapes(pkg):
+    # The f16 kernel's main loop exists in three forms (advancing pointers while every load is in range,
+    # clamped addresses, a last iteration that skips what lies past the end) and which stages run in which
+    # depends on K, the tile shape and the split. gemm_i8_kernel shares none of that code and was checked
+    # against the oracle above: 40 seeded shapes x (7 tile shapes, split-K, grouped, gate/up pair) against it.
+    import random
+    rnd = random.Random(1)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0)
+    L = pkg.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    ks = [32, 96, 160, 224, 288, 352, 480, 544, 736, 1056, 1568, 1632, 1760, 2080, 3104, 6176, 6208, 6240]
+    for _ in range(40):
+        k, m = rnd.choice(ks), rnd.choice([9, 31, 33, 100, 129, 300, 513])
+        n = rnd.choice([16, 40, 100, 160, 330, 700])
+        w1, w2 = (torch.randn((n, k), generator=gen, device="cuda") * 0.05 for _ in range(2))
+        p1, p2 = pkg.quant_pack_rhs(w1), pkg.quant_pack_rhs(w2)
+        ws = pkg.quant_lhs(torch.randn((m, k), generator=gen, device="cuda"))
+        r1 = pkg.matmul_quantized(ws, p1, m, k, n, kernel=pkg.KERNEL_GEMM_I8)
+        r2 = pkg.matmul_quantized(ws, p2, m, k, n, kernel=pkg.KERNEL_GEMM_I8)
+        den = float(r1.abs().max())
+
+        def close(y, r, what, tol=2e-6):
+            err = float((y - r).abs().max()) / den
+            assert err <= tol, (what, m, k, n, err)   # (a NaN fails the comparison too)
+
+        y = torch.empty_like(r1)
+        for t in range(pkg.GEMM_F16_TILES):
+            y.fill_(float("nan"))
+            assert L.w4a32_matmul_quantized_ex(y.data_ptr(), ws.data_ptr(), p1.data_ptr(), m, k, n,
+                                               pkg.KERNEL_GEMM_F16_TILE0 + t, stream) == 0
+            close(y, r1, f"tile {t}")
+        close(pkg.matmul_quantized_splitk(ws, p1, m, k, n), r1, "split-K")
+        for o, r in zip(pkg.matmul_quantized_grouped(ws, [p1, p2], [n, n], m, k), (r1, r2)):
+            close(o, r, "grouped")
+        act = pkg.matmul_quantized_silu_pair(ws, p1, p2, m, k, n)
+        want = torch.nn.functional.silu(r1) * r2
+        assert float((act - want).abs().max()) <= 1e-4 * float(want.abs().max()), ("pair", m, k, n)
+
+
 def test_bad_arguments_return_error_codes(pkg):
     L = pkg.lib()
     x = torch.zeros((1, 48), device="cuda")
