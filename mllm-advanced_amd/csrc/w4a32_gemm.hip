@@ -291,8 +291,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
   uint2 breg[D][B_UNITS];
   uint32_t sreg[D][B_UNITS];
 
-  // Per-lane base pointers; everything that changes from stage to stage is a wavefront-uniform
-  // offset (scalar registers), so issuing a load costs no vector address arithmetic.
+  // Per-lane pointers. In the steady-state loop they advance by constants and a stage's loads use
+  // immediate offsets; elsewhere what changes from stage to stage is a wavefront-uniform offset.
   const int KB = K >> 5;  // 32-k blocks per row
   const uint8_t* a_ptr[WM];
 #pragma unroll
