@@ -50,6 +50,23 @@ int w4a32_quant_lhs_norm(const float* d_h, const float* d_delta, const float* d_
 int w4a32_quant_lhs_silu_mul(const float* d_gate, const float* d_up, int M, int K, void* d_ws,
                              void* stream);
 
+/* A Linear that runs split over K (w4a32_splitk_scratch_bytes(M, K, N) != 0, include/w4a32_hip.h) followed by
+ * the residual add and the next RMSNorm + row quantiser, without the kernel that adds the parts up:
+ *   w4a32_matmul_quantized_splitk_parts leaves *parts_out partial products [parts][M][N] in d_scratch (at
+ *     least w4a32_splitk_scratch_bytes bytes), each already carrying the row and column factors of the
+ *     Linear's output transform; W4A32_ESHAPE when the library does not split this problem;
+ *   w4a32_quant_lhs_norm_parts is w4a32_quant_lhs_norm with delta = ((part 0 + part 1) + ...) + bias of
+ *     that Linear (d_packed, N_linear = this call's K, K_linear), clamped to the finite f32 range like
+ *     every Linear output.
+ * Same operators as above (the MLP's down_proj, the decoder layer's residual add and the next layer's
+ * input_layer_norm_: modeling_ds_qwen2.hpp:47-54, :175-183); the sum differs from w4a32_matmul_quantized_splitk's
+ * in f32 rounding only (the factors are applied before the parts are added instead of after). */
+int w4a32_matmul_quantized_splitk_parts(const void* d_ws, const void* d_packed, int M, int K, int N,
+                                        void* d_scratch, size_t scratch_bytes, int* parts_out, void* stream);
+int w4a32_quant_lhs_norm_parts(const float* d_h, const void* d_parts, int parts, const void* d_packed,
+                               int K_linear, const float* d_weight, float eps, float* d_h_out, int M, int K,
+                               void* d_ws, void* stream);
+
 /* sin/cos tables [max_pos][head_dim/2]: theta = pos / base^(2d/head_dim).
  * precompute_normal_hf_sin_cos, mllm/Backends/Arm/Kernels/rope.cpp:20-37. */
 int w4a32_op_rope_table(float* d_sin, float* d_cos, int max_pos, int head_dim, float base,

@@ -46,6 +46,8 @@ ABI = {
     "w4a32_unpack_kai": (_ci, [_vp, _ci, _ci, _ci, _ci, _ci, _vp, _vp, _vp, _vp]),
     "w4a32_splitk_scratch_bytes": (_sz, [_ci, _ci, _ci]),
     "w4a32_matmul_quantized_splitk": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp, _sz, _vp]),
+    "w4a32_matmul_quantized_splitk_parts": (_ci, [_vp, _vp, _ci, _ci, _ci, _vp, _sz, _vp, _vp]),
+    "w4a32_quant_lhs_norm_parts": (_ci, [_vp, _vp, _ci, _vp, _ci, _vp, ctypes.c_float, _vp, _ci, _ci, _vp, _vp]),
     "w4a32_matmul": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a32_matmul_grouped": (_ci, [_vp, _vp, _vp, _vp, _ci, _vp, _ci, _ci, _vp]),
     # include/w4a32_decoder.h
@@ -312,6 +314,31 @@ def matmul_quantized_splitk(ws, packed, M, K, N, scratch=None, out=None):
                                                scratch.numel() * scratch.element_size() if scratch is not None else 0,
                                                _stream()), "w4a32_matmul_quantized_splitk")
     return y
+
+
+def matmul_quantized_splitk_parts(ws, packed, M, K, N):
+    """The split-K product without the kernel that adds its parts up: returns (scratch, parts)."""
+    need = int(lib().w4a32_splitk_scratch_bytes(M, K, N))
+    scratch = _dev_empty(max(need, 16))
+    parts = ctypes.c_int(0)
+    _check(lib().w4a32_matmul_quantized_splitk_parts(_ptr(ws), _ptr(packed), M, K, N, _ptr(scratch), need,
+                                                     ctypes.byref(parts), _stream()),
+           "w4a32_matmul_quantized_splitk_parts")
+    return scratch, parts.value
+
+
+def quant_lhs_norm_parts(h, scratch, parts, packed, K_linear, weight, eps, ws=None):
+    """quant_lhs_norm() with delta = the sum of a split-K Linear's parts + its bias: returns (ws, h + delta)."""
+    import torch
+
+    M, K = h.shape
+    if ws is None:
+        ws = _dev_empty(workspace_bytes(M, K))
+    h_out = torch.empty_like(h)
+    _check(lib().w4a32_quant_lhs_norm_parts(_ptr(h), _ptr(scratch), parts, _ptr(packed), K_linear, _ptr(weight),
+                                            eps, _ptr(h_out), M, K, _ptr(ws), _stream()),
+           "w4a32_quant_lhs_norm_parts")
+    return ws, h_out
 
 
 def matmul(x, packed, N, ws=None, out=None):

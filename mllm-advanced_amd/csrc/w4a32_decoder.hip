@@ -129,23 +129,38 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
   const float* cos_t = reinterpret_cast<const float*>(st + g.cos_off);
   void* ws = st + g.ws_off;
 
+  // gate and up (with what lies between them) as one scratch area for the operators that run while
+  // both are dead
+  const size_t lend = g.up_off - g.gate_off + sizeof(float) * (size_t)c->max_batch_tokens * I;
+  // Prefill sizes: the operator in front of a Linear runs inside that Linear's row quantiser.
+  const bool fuse_rows = M > w4::kGemvMaxM && w4::quant_rows_fusable(std::max(H, I));
+  // When down_proj runs split over K, its parts are not added up by a kernel of their own: the next layer's
+  // first quantiser (residual add + RMSNorm) reads them instead of `delta`. The parts lie in the gate/up
+  // area, which nothing else uses between down_proj and that quantiser.
+  const int down_parts = fuse_rows ? w4::splitk_plan(M, I, H).parts : 1;
+  const size_t parts_bytes = down_parts > 1 ? w4a32_splitk_scratch_bytes(M, I, H) : 0;
+  const bool defer_sum = down_parts > 1 && parts_bytes <= lend;
+  bool delta_in_parts = false;  // the previous layer's down_proj left parts, not delta
+
   for (int l = 0; l < c->n_layers; ++l) {
     const w4a32_layer_weights& lw = w->layers[l];
     float* kc = reinterpret_cast<float*>(st + g.kcache_off) + (size_t)l * g.cache_layer;
     float* vc = reinterpret_cast<float*>(st + g.vcache_off) + (size_t)l * g.cache_layer;
-    // gate and up (with what lies between them) as one scratch area for the operators that run while
-    // both are dead
-    const size_t lend = g.up_off - g.gate_off + sizeof(float) * (size_t)c->max_batch_tokens * I;
-    // Prefill sizes: the operator in front of a Linear runs inside that Linear's row quantiser.
-    const bool fuse_rows = M > w4::kGemvMaxM && w4::quant_rows_fusable(std::max(H, I));
     // h += mlp output of the previous layer; xn = norm(h)
     {
       float* ys[3] = {q, k, v};
       const void* ps[3] = {lw.q, lw.k, lw.v};
       const int ns[3] = {qd, kvd, kvd};
       if (fuse_rows) {
-        W4_TRY(w4a32_quant_lhs_norm(h, l == 0 ? nullptr : delta, lw.attn_norm, c->rms_eps, h, M, H, ws,
-                                    stream));
+        if (delta_in_parts) {
+          const uint8_t* down_prev = static_cast<const uint8_t*>(w->layers[l - 1].down);
+          W4_TRY(from_hip(w4::launch_quant_lhs_norm_parts(h, gate, down_parts, w4::linear_bias(down_prev, H, I),
+                                                          lw.attn_norm, c->rms_eps, h, M, H,
+                                                          static_cast<uint8_t*>(ws), s)));
+        } else {
+          W4_TRY(w4a32_quant_lhs_norm(h, l == 0 ? nullptr : delta, lw.attn_norm, c->rms_eps, h, M, H, ws,
+                                      stream));
+        }
         W4_TRY(w4a32_matmul_quantized_grouped(ys, ws, ps, ns, 3, M, H, stream));
       } else {
         W4_TRY(from_hip(w4::launch_rmsnorm(h, l == 0 ? nullptr : delta, lw.attn_norm, M, H, c->rms_eps,
@@ -190,7 +205,13 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
       }
       // few output tiles, long K: split-K, with the partial sums in the gate and up buffers,
       // which are dead once the quantised rows of silu(gate) * up exist
-      W4_TRY(w4a32_matmul_quantized_splitk(delta, ws, lw.down, M, I, H, gate, lend, stream));
+      delta_in_parts = defer_sum && l + 1 < c->n_layers;
+      if (delta_in_parts) {
+        W4_TRY(from_hip(w4::launch_gemm_splitk(nullptr, static_cast<const uint8_t*>(ws),
+                                               static_cast<const uint8_t*>(lw.down), M, I, H, gate, s)));
+      } else {
+        W4_TRY(w4a32_matmul_quantized_splitk(delta, ws, lw.down, M, I, H, gate, lend, stream));
+      }
     } else {
       W4_TRY(from_hip(w4::launch_silu_mul(gate, up, act, (size_t)M * I, s)));
       W4_TRY(w4a32_matmul(delta, act, lw.down, ws, M, I, H, stream));
@@ -318,6 +339,40 @@ int w4a32_op_silu_mul(const float* d_gate, const float* d_up, float* d_out, size
   if (!d_gate || !d_up || !d_out || n == 0) return W4A32_EINVAL;
   if (n % 4 != 0) return W4A32_ESHAPE;
   return from_hip(w4::launch_silu_mul(d_gate, d_up, d_out, n, S(stream)));
+}
+
+int w4a32_matmul_quantized_splitk_parts(const void* d_ws, const void* d_packed, int M, int K, int N,
+                                        void* d_scratch, size_t scratch_bytes, int* parts_out, void* stream) {
+  if (!d_ws || !d_packed || !d_scratch || !parts_out) return W4A32_EINVAL;
+  const size_t need = w4a32_splitk_scratch_bytes(M, K, N);
+  if (need == 0) return W4A32_ESHAPE;
+  if (scratch_bytes < need) return W4A32_EINVAL;
+  if ((reinterpret_cast<uintptr_t>(d_ws) & 255) != 0 || (reinterpret_cast<uintptr_t>(d_packed) & 15) != 0 ||
+      (reinterpret_cast<uintptr_t>(d_scratch) & 15) != 0) {
+    return W4A32_EINVAL;
+  }
+  *parts_out = w4::splitk_plan(M, K, N).parts;
+  return from_hip(w4::launch_gemm_splitk(nullptr, static_cast<const uint8_t*>(d_ws),
+                                         static_cast<const uint8_t*>(d_packed), M, K, N,
+                                         static_cast<float*>(d_scratch), S(stream)));
+}
+
+int w4a32_quant_lhs_norm_parts(const float* d_h, const void* d_parts, int parts, const void* d_packed,
+                               int K_linear, const float* d_weight, float eps, float* d_h_out, int M, int K,
+                               void* d_ws, void* stream) {
+  if (!d_h || !d_parts || !d_packed || !d_weight || !d_h_out || !d_ws || M <= 0 || K <= 0 || parts < 1) {
+    return W4A32_EINVAL;
+  }
+  if (K % 32 != 0 || K_linear <= 0 || K_linear % 32 != 0 || M <= w4::kGemvMaxM || !w4::quant_rows_fusable(K)) {
+    return W4A32_ESHAPE;
+  }
+  if ((reinterpret_cast<uintptr_t>(d_ws) & 255) != 0 || (reinterpret_cast<uintptr_t>(d_parts) & 15) != 0) {
+    return W4A32_EINVAL;
+  }
+  return from_hip(w4::launch_quant_lhs_norm_parts(
+      d_h, static_cast<const float*>(d_parts), parts,
+      w4::linear_bias(static_cast<const uint8_t*>(d_packed), K, K_linear), d_weight, eps, d_h_out, M, K,
+      static_cast<uint8_t*>(d_ws), S(stream)));
 }
 
 int w4a32_quant_lhs_norm(const float* d_h, const float* d_delta, const float* d_weight, float eps,

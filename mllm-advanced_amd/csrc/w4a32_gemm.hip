@@ -679,6 +679,13 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
     bs[b] = load_global<float>(bsp + (n < N ? n : N - 1));
   }
 
+  // SPLITK without an output (y == nullptr): the parts are stored with the row and column factors applied
+  // (the reader adds them up and adds the bias); with an output they are raw sums (factors 1).
+  const bool scaled_parts = SPLITK && y_arg == nullptr;
+  float part_rm[WN];
+#pragma unroll
+  for (int b = 0; b < WN; ++b) part_rm[b] = scaled_parts ? rm[b] : 1.0f;
+
   __builtin_amdgcn_sched_barrier(0);
 
   // C layout of a 32x32 tile: lane (h, i32) holds column i32; register v holds row
@@ -709,6 +716,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
         if constexpr (!SPLITK) {
           val = __fmaf_rn(val * rm[b], rc[a][v], bs[b]);
           val = fminf(fmaxf(val, -3.402823466e+38f), 3.402823466e+38f);
+        } else {
+          val = val * part_rm[b] * (scaled_parts ? rc[a][v] : 1.0f);
         }
         if constexpr (PAIR) {
           float up = __fmaf_rn(acc[a][b + WNH][v] * rm[b + WNH], rc[a][v], bs[b + WNH]);
@@ -800,6 +809,7 @@ static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed,
                        recip, packed, packed + g.hscale_off, rowmul, bias, M, N, K, g.NT, g.KC, MB, NB,
                        n_major, ksplit, part, GemmGroup{});
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+    if (!y) return hipSuccess;  // the caller's next kernel adds the (scaled) parts up
     const size_t total = (size_t)M * N;
     if (N % 4 == 0) {
       hipLaunchKernelGGL(splitk_reduce_kernel<4>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256),
@@ -979,10 +989,16 @@ SplitPlan splitk_plan(int M, int K, int N) {
   return p;
 }
 
+// y == nullptr: no reduction; part[i][M][N], i < parts, then holds sums that already carry the row and column
+// factors, for a reader that computes (((part[0] + part[1]) + ...) + bias) itself.
 hipError_t launch_gemm_splitk(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                               float* part, hipStream_t s) {
   const SplitPlan p = splitk_plan(M, K, N);
   return launch_f16_tile(p.tile, y, ws, packed, M, K, N, nullptr, nullptr, 0, p.parts, part, s);
+}
+
+const float* linear_bias(const uint8_t* packed, int N, int K) {
+  return reinterpret_cast<const float*>(packed + weight_geom(N, K).bias_off);
 }
 
 }  // namespace w4

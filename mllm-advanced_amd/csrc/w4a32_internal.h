@@ -29,6 +29,11 @@ hipError_t launch_quant_lhs(const float* x, int M, int K, int ldx, uint8_t* ws, 
 bool quant_rows_fusable(int K);
 hipError_t launch_quant_lhs_norm(const float* h, const float* delta, const float* norm_w, float eps,
                                  float* h_out, int M, int K, uint8_t* ws, hipStream_t s);
+// ... with delta = ((parts[0] + parts[1]) + ...) + bias, parts = [nparts][M][K] as launch_gemm_splitk leaves
+// them when it is given no output
+hipError_t launch_quant_lhs_norm_parts(const float* h, const float* parts, int nparts, const float* bias,
+                                       const float* norm_w, float eps, float* h_out, int M, int K,
+                                       uint8_t* ws, hipStream_t s);
 hipError_t launch_quant_lhs_silu_mul(const float* gate, const float* up, int M, int K, uint8_t* ws,
                                      hipStream_t s);
 
@@ -76,6 +81,7 @@ struct SplitPlan {
 SplitPlan splitk_plan(int M, int K, int N);
 hipError_t launch_gemm_pair(float* act, const uint8_t* ws, const uint8_t* gate, const uint8_t* up, int M,
                             int K, int N, hipStream_t s);
+const float* linear_bias(const uint8_t* packed, int N, int K);  // the bias row inside a packed blob
 hipError_t launch_gemm_splitk(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                               float* part, hipStream_t s);
 // several Linears on the same quantised rows in one launch of the f16 kernel (M > 8)

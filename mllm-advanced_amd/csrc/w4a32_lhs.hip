@@ -90,7 +90,8 @@ template <int SRC, int R>
 __global__ __launch_bounds__(kLhsThreads) void quant_rows_kernel(
     const float* __restrict__ a, const float* __restrict__ b, const float* __restrict__ norm_w,
     float eps, float* h_out, int K, int lda, float* __restrict__ recip_out,
-    int32_t* __restrict__ negzp_out, int8_t* __restrict__ aq, _Float16* __restrict__ ah) {
+    int32_t* __restrict__ negzp_out, int8_t* __restrict__ aq, _Float16* __restrict__ ah, int nparts,
+    size_t part_stride, const float* __restrict__ part_bias) {
   const int m = blockIdx.x;
   const int t = threadIdx.x;
   const size_t row = (size_t)m * lda;
@@ -117,8 +118,25 @@ __global__ __launch_bounds__(kLhsThreads) void quant_rows_kernel(
       float4 x1 = *reinterpret_cast<const float4*>(a + row + i + 4);
       if constexpr (SRC == kSrcNorm) {
         if (b) {
-          const float4 d0 = *reinterpret_cast<const float4*>(b + row + i);
-          const float4 d1 = *reinterpret_cast<const float4*>(b + row + i + 4);
+          float4 d0 = *reinterpret_cast<const float4*>(b + row + i);
+          float4 d1 = *reinterpret_cast<const float4*>(b + row + i + 4);
+          if (nparts > 0) {
+            // b = the parts of a split-K product, [nparts][M][K] with the row and column factors applied:
+            // delta = ((part 0 + part 1) + ...) + bias, clamped like every Linear output
+            for (int p = 1; p < nparts; ++p) {
+              const float4 e0 = *reinterpret_cast<const float4*>(b + p * part_stride + row + i);
+              const float4 e1 = *reinterpret_cast<const float4*>(b + p * part_stride + row + i + 4);
+              d0.x += e0.x; d0.y += e0.y; d0.z += e0.z; d0.w += e0.w;
+              d1.x += e1.x; d1.y += e1.y; d1.z += e1.z; d1.w += e1.w;
+            }
+            const float4 b0 = *reinterpret_cast<const float4*>(part_bias + i);
+            const float4 b1 = *reinterpret_cast<const float4*>(part_bias + i + 4);
+            constexpr float kMax = 3.402823466e+38f;
+            d0.x = fminf(fmaxf(d0.x + b0.x, -kMax), kMax); d0.y = fminf(fmaxf(d0.y + b0.y, -kMax), kMax);
+            d0.z = fminf(fmaxf(d0.z + b0.z, -kMax), kMax); d0.w = fminf(fmaxf(d0.w + b0.w, -kMax), kMax);
+            d1.x = fminf(fmaxf(d1.x + b1.x, -kMax), kMax); d1.y = fminf(fmaxf(d1.y + b1.y, -kMax), kMax);
+            d1.z = fminf(fmaxf(d1.z + b1.z, -kMax), kMax); d1.w = fminf(fmaxf(d1.w + b1.w, -kMax), kMax);
+          }
           x0.x += d0.x; x0.y += d0.y; x0.z += d0.z; x0.w += d0.w;
           x1.x += d1.x; x1.y += d1.y; x1.z += d1.z; x1.w += d1.w;
           *reinterpret_cast<float4*>(h_out + row + i) = x0;
@@ -222,7 +240,8 @@ constexpr int kQuantRowsMaxK = 8 * 8 * kLhsThreads;
 
 template <int SRC>
 static hipError_t launch_quant_rows(const float* a, const float* b, const float* norm_w, float eps,
-                                    float* h_out, int M, int K, int lda, uint8_t* ws, hipStream_t s) {
+                                    float* h_out, int M, int K, int lda, uint8_t* ws, hipStream_t s,
+                                    int nparts = 0, const float* part_bias = nullptr) {
   const WsGeom g = ws_geom(M, K);
   float* recip = reinterpret_cast<float*>(ws + g.scale_off);
   int32_t* negzp = reinterpret_cast<int32_t*>(ws + g.off_off);
@@ -231,7 +250,7 @@ static hipError_t launch_quant_rows(const float* a, const float* b, const float*
   const int groups = (K + 8 * kLhsThreads - 1) / (8 * kLhsThreads);
 #define W4_LAUNCH_ROWS(R)                                                                          \
   hipLaunchKernelGGL((quant_rows_kernel<SRC, R>), dim3(M), dim3(kLhsThreads), 0, s, a, b, norm_w, eps, \
-                     h_out, K, lda, recip, negzp, aq, ah)
+                     h_out, K, lda, recip, negzp, aq, ah, nparts, (size_t)M * K, part_bias)
   if (groups <= 1) W4_LAUNCH_ROWS(1);
   else if (groups <= 2) W4_LAUNCH_ROWS(2);
   else if (groups <= 5) W4_LAUNCH_ROWS(5);
@@ -246,6 +265,14 @@ bool quant_rows_fusable(int K) { return K <= kQuantRowsMaxK; }
 hipError_t launch_quant_lhs_norm(const float* h, const float* delta, const float* norm_w, float eps,
                                  float* h_out, int M, int K, uint8_t* ws, hipStream_t s) {
   return launch_quant_rows<kSrcNorm>(h, delta, norm_w, eps, h_out, M, K, K, ws, s);
+}
+
+// The same with delta = the sum of a split-K product's `nparts` scaled parts ([nparts][M][K]) + bias.
+hipError_t launch_quant_lhs_norm_parts(const float* h, const float* parts, int nparts, const float* bias,
+                                       const float* norm_w, float eps, float* h_out, int M, int K,
+                                       uint8_t* ws, hipStream_t s) {
+  if (nparts < 1 || !parts || !bias) return hipErrorInvalidValue;
+  return launch_quant_rows<kSrcNorm>(h, parts, norm_w, eps, h_out, M, K, K, ws, s, nparts, bias);
 }
 
 hipError_t launch_quant_lhs_silu_mul(const float* gate, const float* up, int M, int K, uint8_t* ws,

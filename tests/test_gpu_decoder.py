@@ -74,6 +74,37 @@ def test_fused_row_quantisers_match_separate_operators(pkg, M, K):
         assert torch.equal(x1, x0)          # elementwise: the same arithmetic, bit for bit
 
 
+@pytest.mark.parametrize("M,K,N,bias", [(512, 8960, 1536, False), (100, 6144, 288, True), (16, 8960, 1536, True),
+                                          (1100, 6208, 1536, False)])
+def test_split_k_parts_summed_by_the_norm_quantiser(pkg, M, K, N, bias):
+    # down_proj split over K whose parts are added up by the next residual add + RMSNorm + quantiser,
+    # against the same three steps with the reduction kernel in between
+    g = torch.Generator(device="cuda").manual_seed(M + N)
+    packed = pkg.quant_pack_rhs(torch.randn((N, K), generator=g, device="cuda") * 0.05,
+                                torch.randn((N,), generator=g, device="cuda") if bias else None)
+    ws_in = pkg.quant_lhs(torch.randn((M, K), generator=g, device="cuda"))
+    h = torch.randn((M, N), generator=g, device="cuda") * 2
+    w = 1 + 0.1 * torch.randn((N,), generator=g, device="cuda")
+    delta = pkg.matmul_quantized_splitk(ws_in, packed, M, K, N)
+    ws0, h0 = pkg.quant_lhs_norm(h, w, 1e-6, delta=delta)
+    scratch, parts = pkg.matmul_quantized_splitk_parts(ws_in, packed, M, K, N)
+    assert parts > 1
+    ws1, h1 = pkg.quant_lhs_norm_parts(h, scratch, parts, packed, K, w, 1e-6)
+    # the factors of the output transform are applied before the parts are added instead of after
+    assert float((h1 - h0).abs().max()) <= 2e-6 * float(delta.abs().max())
+    aq0, recip0, nzp0 = pkg.export_lhs(ws0, M, N)
+    aq1, recip1, nzp1 = pkg.export_lhs(ws1, M, N)
+    assert torch.allclose(recip1, recip0, rtol=1e-5, atol=0)
+    assert int((nzp1 - nzp0).abs().max()) <= 1
+    diff = (aq1.int() - aq0.int()).abs()
+    assert int(diff.max()) <= 1 and float((diff > 0).float().mean()) < 5e-3
+    # a problem the library does not split has no parts to hand over
+    small = pkg.quant_pack_rhs(torch.randn((64, 256), generator=g, device="cuda"))
+    with pytest.raises(RuntimeError):
+        pkg.matmul_quantized_splitk_parts(pkg.quant_lhs(torch.randn((64, 256), generator=g, device="cuda")),
+                                          small, 64, 256, 64)
+
+
 def test_fused_row_quantisers_reject_what_they_do_not_take(pkg):
     h = torch.zeros((8, 64), device="cuda")
     w = torch.ones((64,), device="cuda")
