@@ -600,7 +600,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
     bq_pos = (s_base >> 1) * kTileBytes;
     bs_pos = (s_base >> 1) * kTileScaleBytes;
   }
-  const bool whole = (nstages - s_begin) % U == 0;  // the stages come in whole iterations
+  // the stages come in whole iterations (a range without stages runs nothing)
+  const bool whole = nstages > s_begin && (nstages - s_begin) % U == 0;
   for (; s_base + (whole ? U : 0) < nstages; s_base += U) {
     run_stages(std::integral_constant<int, kClamped>{}, s_base);
   }
