@@ -665,7 +665,10 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
     if (has_new) {
 #pragma unroll
       for (int it = 0; it < 4; ++it) {
-        const bool is_new = blk + 4 * it + kq == pos0;
+        // pos0 is this wavefront's last key: what lies behind it was loaded from the row of pos0 too
+        // (clamped), which the cache does not hold yet. Those lanes get weight 0, but 0 x whatever
+        // the memory held (Inf, NaN) must not reach the sums: they take the new row as well.
+        const bool is_new = blk + 4 * it + kq >= pos0;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           kk[it][i] = is_new ? knew[i] : kk[it][i];

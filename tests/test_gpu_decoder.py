@@ -298,6 +298,37 @@ def test_decoder_runner_matches_oracle(pkg):
         assert dec.position == 12 + step
 
 
+def test_decoder_ignores_what_its_state_memory_held(pkg):
+    # The state is caller-owned memory that init does not clear: rows of the KV cache behind the position,
+    # scratch areas and activations hold whatever was there. Bytes 0xFF (NaN as f32) against zeros: prefill
+    # and decode steps must give the same logits bit for bit. (The decode attention loads the row of the new
+    # token's position before anybody has written it.)
+    import ctypes
+
+    rng = np.random.default_rng(7)
+    H, Hq, Hkv, I, V, L = 256, 2, 1, 384, 640, 2
+    weights = tiny_model(rng, H, Hq, Hkv, I, V, L)
+    prompt = dev(rng.integers(0, V, size=21).astype(np.int64))
+    runs = []
+    for fill in (0, 255):
+        dec = to_device_model(pkg, weights, Hq, Hkv, max_seq=64, max_batch_tokens=32, rope_theta=1e6)
+        dec.state.fill_(fill)
+        assert pkg.lib().w4a32_decoder_init(ctypes.byref(dec.cfg), dec.state.data_ptr(), None) == 0
+        out = []
+        dec.step()                                  # a first token at position 0, nothing cached yet
+        out.append(dec.logits.clone())
+        dec.prefill(prompt)                         # (from position 0 again)
+        out.append(dec.logits.clone())
+        for _ in range(20):                         # positions 21..40: every place inside a block of 16 keys
+            dec.step()
+            out.append(dec.logits.clone())
+        torch.cuda.synchronize()
+        runs.append(out)
+    for a, b in zip(*runs):
+        assert not bool(torch.isnan(b).any())
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("prompt_len", [300, 520])
 def test_decoder_runner_at_the_model_s_widths(pkg, prompt_len):
     # hidden 1536, 12 / 2 heads, MLP 8960 (two layers, small vocabulary): the prefill runs the kernels the
