@@ -587,6 +587,17 @@ def main():
                     orc.linear(xs[l.K], u4, sc, bias=bias, threads=nthr)
                 reps_t += 1
             threaded[f"threads_{nthr}"] = round(layer_bytes * reps_t / (time.perf_counter() - t0) / 1e9, 3)
+        # the same product with its block dots on AVX-512 VNNI (bit-identical results), where the host has it
+        vnni = None
+        if orc.has_vnni():
+            vnni = {}
+            for nthr in (1, 4, 16):
+                reps_t, t0 = 0, time.perf_counter()
+                while time.perf_counter() - t0 < 2.0:
+                    for (l, u4, sc, bias) in host:
+                        orc.linear_vnni(xs[l.K], u4, sc, bias=bias, threads=nthr)
+                    reps_t += 1
+                vnni[f"threads_{nthr}"] = round(layer_bytes * reps_t / (time.perf_counter() - t0) / 1e9, 3)
         # prefill: gate_proj at M=128 (the reference deals rows to its 4 workers)
         (l, u4, sc, bias) = host[4]
         xp = np.random.default_rng(1).standard_normal((128, l.K)).astype(np.float32)
@@ -594,6 +605,7 @@ def main():
         orc.linear(xp, u4, sc, bias=bias, threads=4)
         dtp = time.perf_counter() - t0
         extra["cpu_baseline_more"] = {"decode_GBps_by_threads": threaded,
+                                      "decode_GBps_avx512_vnni_by_threads": vnni,
                                       "prefill_gate_proj_M128_4_threads_TFLOPs":
                                           round(2.0 * 128 * l.N * l.K / dtp / 1e12, 5),
                                       "note": "scalar C restatement; columns (decode) or rows x columns "

@@ -90,6 +90,19 @@ void orc_dequant_qs4c32(size_t n, size_t k, size_t bl, const uint8_t* rhs_u4,
 void orc_linear_w4a32(size_t m, size_t n, size_t k, const float* x, const uint8_t* rhs_u4,
                       const uint16_t* scales_bf16, const float* bias, float* y, int num_threads);
 
+/*
+ * w4a32_oracle_vnni.c: orc_matmul_qa8dx_qs4c32 / orc_linear_w4a32 with the block dots on AVX-512
+ * VNNI (bl = 32, k % 32 == 0), bit-identical results; for the benchmark's CPU-baseline leg.
+ * Return 0, or -1 when the CPU lacks AVX-512 VNNI (orc_has_avx512_vnni() == 0) or k does not fit.
+ */
+int orc_has_avx512_vnni(void);
+int orc_matmul_qa8dx_qs4c32_vnni(size_t m, size_t n, size_t k, const int8_t* lhs_qa8dx,
+                                 const uint8_t* rhs_u4, const uint16_t* scales_bf16,
+                                 const float* bias, float* dst_f32, float scalar_min,
+                                 float scalar_max, int num_threads);
+int orc_linear_w4a32_vnni(size_t m, size_t n, size_t k, const float* x, const uint8_t* rhs_u4,
+                          const uint16_t* scales_bf16, const float* bias, float* y, int num_threads);
+
 #ifdef __cplusplus
 }
 #endif

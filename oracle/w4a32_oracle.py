@@ -49,6 +49,10 @@ def lib():
         L.orc_dequant_qs4c32.argtypes = [sz, sz, sz, vp, vp, vp]
         L.orc_linear_w4a32.restype = None
         L.orc_linear_w4a32.argtypes = [sz, sz, sz, vp, vp, vp, vp, vp, ci]
+        L.orc_has_avx512_vnni.restype = ci
+        L.orc_has_avx512_vnni.argtypes = []
+        L.orc_linear_w4a32_vnni.restype = ci
+        L.orc_linear_w4a32_vnni.argtypes = [sz, sz, sz, vp, vp, vp, vp, vp, ci]
         _lib = L
     return _lib
 
@@ -129,4 +133,22 @@ def linear(x, u4, sc, bias=None, threads=1):
     y = np.empty((m, n), dtype=np.float32)
     b = _f32c(bias) if bias is not None else None
     lib().orc_linear_w4a32(m, n, k, _p(x), _p(u4), _p(sc), _p(b), _p(y), threads)
+    return y
+
+
+def has_vnni():
+    """True when this CPU runs the AVX-512 VNNI form of the product."""
+    return bool(lib().orc_has_avx512_vnni())
+
+
+def linear_vnni(x, u4, sc, bias=None, threads=1):
+    """linear() with the block dots on vpdpbusd: same results bit for bit; raises without AVX-512 VNNI."""
+    x = _f32c(x)
+    m, k = x.shape
+    n = u4.shape[0]
+    y = np.empty((m, n), dtype=np.float32)
+    b = _f32c(bias) if bias is not None else None
+    rc = lib().orc_linear_w4a32_vnni(m, n, k, _p(x), _p(u4), _p(sc), _p(b), _p(y), threads)
+    if rc != 0:
+        raise RuntimeError("AVX-512 VNNI form unavailable (CPU lacks it, or K is not a multiple of 32)")
     return y

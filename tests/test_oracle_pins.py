@@ -420,3 +420,29 @@ def test_oracle_equals_torch_dyn_quant_matmul_on_many_small_cases(orc):
         got = orc.linear(x, u4, sc, bias=bias)
         want = torch_dyn_quant_linear(x, u4, sc, bias)
         assert np.array_equal(got, want), (case, m, k, n, kind)
+
+
+# ---- the AVX-512 VNNI form of the product (benchmark's CPU-baseline leg) ----
+@pytest.mark.parametrize("m,k,n,bias,threads", [
+    (1, 32, 5, False, 1),        # one block: the masked tail group alone
+    (3, 96, 17, True, 2),        # three blocks: one partial group of four
+    (2, 160, 33, True, 3),       # a whole group and a one-block tail
+    (1, 1536, 256, True, 4),     # k/v_proj
+    (4, 1280, 64, False, 1),     # ViT width (40 blocks)
+    (1, 8960, 48, False, 2),     # down_proj's K
+])
+def test_vnni_product_is_bit_identical_to_the_scalar_one(orc, m, k, n, bias, threads):
+    if not orc.has_vnni():
+        pytest.skip("CPU without AVX-512 VNNI")
+    rng = np.random.default_rng(1000 + k + n)
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    w[0, :32] = 0.0                                   # an all-zero block (scale 0, every u4 = 8)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    x[0, ::7] *= 20.0                                 # outliers: a wide range, large |zero point|
+    if m > 1:
+        x[1] = np.abs(x[1])                           # one-sided row: offset at the end of its range
+    b = (rng.standard_normal(n) * 0.1).astype(np.float32) if bias else None
+    u4, sc = orc.quant_rhs(w)
+    ref = orc.linear(x, u4, sc, bias=b, threads=1)
+    got = orc.linear_vnni(x, u4, sc, bias=b, threads=threads)
+    assert np.array_equal(ref.view(np.uint32), got.view(np.uint32))
