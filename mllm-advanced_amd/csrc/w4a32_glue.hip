@@ -62,8 +62,24 @@ __device__ __forceinline__ float load_shared_across_wgs(const float* p) {
 __device__ __forceinline__ int load_shared_across_wgs(const int* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// All of this wavefront's stores above have reached the coherence point.
-__device__ __forceinline__ void stores_done() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); }
+// Hand-over of partial results to the last workgroup to arrive at a counter.
+// Writer: stores_done() after the device-scope stores and before the barrier / counter increment. A
+// workgroup-scope release fence alone does not have to wait for global stores that are still in flight,
+// so the wait is written out: on gfx9 stores count in vmcnt, and a device-scope (write-through) store is
+// acknowledged once it has reached the coherence point. After it every store this wavefront issued above
+// is visible to device-scope loads of any workgroup; the fence keeps the compiler from moving memory
+// accesses across it. No cache write-back or invalidate is involved.
+// Reader: the workgroup whose increment returns the last ticket calls arrivals_seen() before its
+// device-scope loads (which bypass the non-coherent cache levels); it only pins the order for the compiler,
+// the hardware issues a wavefront's memory instructions in program order behind the returned atomic.
+__device__ __forceinline__ void stores_done() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+__device__ __forceinline__ void arrivals_seen() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
 }  // namespace
 
 // ---------------------------------------------------------------------------------------------
@@ -484,6 +500,7 @@ __global__ __launch_bounds__(64 * kPfWaves) void attention_prefill_mfma_kernel(
     if (lane == 0) prev = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     prev = __shfl(prev, 0, 64);
     if (prev != (unsigned)nchunks - 1) return;
+    arrivals_seen();
     float cmax[kPfMaxChunks], csum[kPfMaxChunks];
     float all_max = -INFINITY;
 #pragma unroll
@@ -760,6 +777,7 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
   }
   __syncthreads();
   if (s_prev != (unsigned)ns - 1) return;
+  arrivals_seen();
   // Last workgroup of this head group: merge the shares of all key slices. Every thread requests
   // all headers and its own dim of all shares at once (ns <= kMaxAttnSplit, loads independent).
   for (int t = threadIdx.x; t < kGW * kHeadDim; t += 64 * kDecWaves) {
@@ -835,6 +853,7 @@ __global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ l
   }
   __syncthreads();
   if (s_prev != gridDim.x - 1) return;
+  arrivals_seen();
   bv = -INFINITY;
   bi = 0x7fffffff;
   for (int b = threadIdx.x; b < (int)gridDim.x; b += blockDim.x) {
