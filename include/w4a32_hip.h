@@ -27,7 +27,8 @@ enum {
   W4A32_EINVAL = -1,   /* null pointer, non-positive dimension, misaligned pointer */
   W4A32_ESHAPE = -2,   /* K not a multiple of 32, or M outside the kernel's range */
   W4A32_ELAUNCH = -3,  /* the HIP runtime refused the launch (see hipGetLastError) */
-  W4A32_ENOTSUP = -4   /* request needs a path this build does not provide */
+  W4A32_ENOTSUP = -4,  /* request needs a path this build does not provide */
+  W4A32_ETOOBIG = -5   /* w4a32_matmul_static_ws: the rows need more than W4A32_STATIC_WS_BYTES */
 };
 
 #define W4A32_BLOCK_LEN 32          /* k per weight scale (kai_linear.cpp:328 passes 32) */
@@ -152,6 +153,24 @@ int w4a32_matmul_quantized_splitk(float* d_y, const void* d_ws, const void* d_pa
  * then multiply. d_ws must hold w4a32_workspace_bytes(M, K). */
 int w4a32_matmul(float* d_y, const float* d_x, const void* d_packed, void* d_ws, int M, int K,
                  int N, void* stream);
+
+/* w4a32_matmul without a workspace argument, for callers that cannot allocate device memory (code under
+ * HIP graph capture, serving loops and harnesses that forbid hipMalloc). It has no counterpart in the
+ * reference, whose forward allocates its workspace on every call (mllm/Backends/Arm/Ops/LinearOp.cpp:74-78).
+ * The quantised rows go to a W4A32_STATIC_WS_BYTES array that is part of the library's device code: every
+ * GPU the library runs on holds one copy until the process ends, and the call allocates and frees
+ * nothing. Same kernels and results as w4a32_matmul, bit for bit.
+ *   - W4A32_ETOOBIG when w4a32_workspace_bytes(M, K) exceeds W4A32_STATIC_WS_BYTES (16 MiB: M = 512 rows
+ *     of K = 8960, or 3600 rows of K = 1536); nothing is launched then.
+ *   - All calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads) race.
+ *     Calls on one stream are ordered and need nothing more. The array keeps the last call's rows: a
+ *     call overwrites the M rows it multiplies, and what the product kernels read beyond them (up to 31
+ *     rows of padding) only feeds output rows that are never stored.
+ *   - The first call on a device looks the array's address up (hipGetSymbolAddress); make that call outside
+ *     stream capture. */
+#define W4A32_STATIC_WS_BYTES (16u << 20)
+int w4a32_matmul_static_ws(float* d_y, const float* d_x, const void* d_packed, int M, int K, int N,
+                           void* stream);
 
 /* Several Linears applied to the SAME activation rows, in one launch where the sizes allow:
  * d_y, d_packed and N are HOST arrays of `count` (<= W4A32_MAX_GROUP) entries; Linear i has blob

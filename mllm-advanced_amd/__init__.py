@@ -50,6 +50,7 @@ ABI = {
     "w4a32_quant_lhs_norm_parts": (_ci, [_vp, _vp, _ci, _vp, _ci, _vp, ctypes.c_float, _vp, _ci, _ci, _vp, _vp]),
     "w4a32_matmul": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a32_matmul_grouped": (_ci, [_vp, _vp, _vp, _vp, _ci, _vp, _ci, _ci, _vp]),
+    "w4a32_matmul_static_ws": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     # include/w4a32_decoder.h
     "w4a32_op_embedding": (_ci, [_vp, _vp, _ci, _ci, _ci, _vp, _vp]),
     "w4a32_op_rmsnorm": (_ci, [_vp, _vp, _vp, _ci, _ci, ctypes.c_float, _vp, _vp, _vp]),

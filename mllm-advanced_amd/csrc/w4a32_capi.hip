@@ -16,6 +16,33 @@ inline int shape_ok(int N, int K) {
 
 inline int from_hip(hipError_t e) { return e == hipSuccess ? W4A32_OK : W4A32_ELAUNCH; }
 
+constexpr int kMaxDevices = 64;
+
+}  // namespace
+
+// Activation workspace of w4a32_matmul_static_ws: one copy per GPU, part of the code object's
+// zero-initialised data, held until the process ends. In host code this name only identifies the
+// symbol; the memory's address on a device comes from hipGetSymbolAddress (static_ws_ptr below).
+static __device__ __align__(256) unsigned char scratch[W4A32_STATIC_WS_BYTES];
+
+namespace {
+
+// Address of `scratch` on each device, looked up on the first call made with that device current.
+std::atomic<void*> g_static_ws[kMaxDevices];
+
+int static_ws_ptr(void** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return W4A32_ELAUNCH;
+  if (dev < 0 || dev >= kMaxDevices) return W4A32_ENOTSUP;
+  void* p = g_static_ws[dev].load(std::memory_order_acquire);
+  if (!p) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return W4A32_ELAUNCH;
+    g_static_ws[dev].store(p, std::memory_order_release);  // racing first calls store the same address
+  }
+  *out = p;
+  return W4A32_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -27,6 +54,7 @@ const char* w4a32_error_string(int code) {
     case W4A32_ESHAPE: return "unsupported shape (K must be a multiple of 32; M must fit the kernel)";
     case W4A32_ELAUNCH: return "HIP launch failed";
     case W4A32_ENOTSUP: return "not supported by this build";
+    case W4A32_ETOOBIG: return "rows need more than the static workspace (W4A32_STATIC_WS_BYTES)";
     default: return "unknown error";
   }
 }
@@ -208,6 +236,16 @@ int w4a32_matmul(float* d_y, const float* d_x, const void* d_packed, void* d_ws,
   }
   if (int e = w4a32_quant_lhs(d_x, M, K, K, d_ws, stream)) return e;
   return w4a32_matmul_quantized(d_y, d_ws, d_packed, M, K, N, stream);
+}
+
+int w4a32_matmul_static_ws(float* d_y, const float* d_x, const void* d_packed, int M, int K, int N,
+                           void* stream) {
+  if (M <= 0) return W4A32_EINVAL;
+  if (int e = shape_ok(N, K)) return e;
+  if (w4::ws_geom(M, K).total_bytes > (size_t)W4A32_STATIC_WS_BYTES) return W4A32_ETOOBIG;
+  void* ws = nullptr;
+  if (int e = static_ws_ptr(&ws)) return e;
+  return w4a32_matmul(d_y, d_x, d_packed, ws, M, K, N, stream);
 }
 
 int w4a32_matmul_grouped(float* const* d_y, const float* d_x, const void* const* d_packed,

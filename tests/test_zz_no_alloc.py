@@ -1,0 +1,74 @@
+"""w4a32_matmul_static_ws: the whole op with its activation workspace in the library's own device array.
+
+Checked through the C ABI against w4a32_matmul (workspace lent by the caller), bit for bit, on calls in
+a row that share the array: a large one, then smaller ones (whose padding rows then hold the earlier
+call's data), decode sizes that use the workspace and ones that do not.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+from conftest import make_acts, make_weights
+
+pytestmark = pytest.mark.gpu
+
+STATIC_WS_BYTES = 16 << 20
+ETOOBIG = -5
+
+
+def _both(pkg, torch, x, packed, M, K, N):
+    L = pkg.lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    y_ref = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    ws = torch.empty(pkg.workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
+    rc = L.w4a32_matmul(y_ref.data_ptr(), x.data_ptr(), packed.data_ptr(), ws.data_ptr(), M, K, N, stream)
+    assert rc == 0
+    y = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    rc = L.w4a32_matmul_static_ws(y.data_ptr(), x.data_ptr(), packed.data_ptr(), M, K, N, stream)
+    assert rc == 0, L.w4a32_error_string(rc)
+    torch.cuda.synchronize()
+    return y, y_ref
+
+
+def test_static_workspace_calls_in_a_row_equal_the_lent_workspace_path(pkg, orc):
+    import torch
+
+    # (M, K, N): prefill, smaller prefill with a ragged last row block, decode through the
+    # workspace (row too long for the fused kernel), fused decode (workspace unused), prefill again
+    cases = [(512, 1536, 1536), (40, 1536, 256), (4, 8960, 1536), (1, 1536, 1536), (72, 8960, 256)]
+    for i, (M, K, N) in enumerate(cases):
+        print(f"static_ws case {i}: M={M} K={K} N={N}", flush=True)
+        w = make_weights(N, K, seed=10 + i)
+        bias = (np.random.default_rng(20 + i).standard_normal(N) * 0.02).astype(np.float32)
+        x = make_acts(M, K, seed=30 + i, outlier_frac=0.01 if M > 8 else 0.0)
+        packed = pkg.quant_pack_rhs(torch.from_numpy(w).cuda(), torch.from_numpy(bias).cuda())
+        xd = torch.from_numpy(x).cuda()
+        y, y_ref = _both(pkg, torch, xd, packed, M, K, N)
+        assert torch.isfinite(y_ref).all()
+        assert torch.equal(y, y_ref), f"case {i}: static workspace differs from the lent one"
+        if M * N * K <= 40 * 1536 * 256 * 4:  # the oracle on the small cases
+            u4, sc = orc.quant_rhs(w)
+            ref = orc.linear(x, u4, sc, bias=bias, threads=4)
+            err = float(np.abs(y.cpu().numpy() - ref).max() / np.abs(ref).max())
+            assert err <= 2e-5, f"case {i}: max-abs-rel {err}"
+
+
+def test_static_workspace_rejects_what_does_not_fit(pkg):
+    import torch
+
+    L = pkg.lib()
+    M, K, N = 4096, 8960, 256          # 4096 rows x 8960 x 3 bytes = 110 MB of quantised rows
+    assert pkg.workspace_bytes(M, K) > STATIC_WS_BYTES
+    y = torch.zeros((8, N), dtype=torch.float32, device="cuda")   # never written: the call must not launch
+    x = torch.zeros((8, K), dtype=torch.float32, device="cuda")
+    packed = torch.zeros(pkg.packed_bytes(N, K), dtype=torch.uint8, device="cuda")
+    rc = L.w4a32_matmul_static_ws(y.data_ptr(), x.data_ptr(), packed.data_ptr(), M, K, N, None)
+    assert rc == ETOOBIG
+    assert b"static workspace" in L.w4a32_error_string(rc)
+    # the largest shapes the header names do fit
+    assert pkg.workspace_bytes(512, 8960) <= STATIC_WS_BYTES
+    assert pkg.workspace_bytes(3600, 1536) <= STATIC_WS_BYTES
+    assert L.w4a32_matmul_static_ws(y.data_ptr(), x.data_ptr(), packed.data_ptr(), 0, K, N, None) == -1
+    assert L.w4a32_matmul_static_ws(y.data_ptr(), x.data_ptr(), packed.data_ptr(), 8, K + 1, N, None) == -2
+    torch.cuda.synchronize()
