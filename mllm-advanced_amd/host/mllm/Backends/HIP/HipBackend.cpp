@@ -9,12 +9,12 @@
 #include "mllm/Engine/Context.hpp"
 #include "mllm/Utils/Log.hpp"
 
-#define MLLM_CHECK_HIP(expr)                                                                    \
-  do {                                                                                          \
-    hipError_t e_ = (expr);                                                                     \
-    if (e_ != hipSuccess)                                                                       \
-      MLLM_ERROR_EXIT(::mllm::kHipError, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), \
-                      __FILE__, __LINE__);                                                      \
+#define MLLM_CHECK_HIP(expr)                                                                         \
+  do {                                                                                               \
+    hipError_t e_ = (expr);                                                                          \
+    if (e_ != hipSuccess) {                                                                          \
+      MLLM_ERROR_EXIT(::mllm::hip::kHipRuntimeError, "{} failed: {}", #expr, hipGetErrorString(e_)); \
+    }                                                                                                \
   } while (0)
 
 namespace mllm::hip {
@@ -69,11 +69,11 @@ HostBackend::HostBackend() : BackendBase(kCPU) { allocator_ = std::make_shared<H
 HipBackend::HipBackend() : BackendBase(kHIP) {
   int count = 0;
   MLLM_CHECK_HIP(hipGetDeviceCount(&count));
-  if (count < 1) MLLM_ERROR_EXIT(kHipError, "no HIP device is visible");
+  if (count < 1) { MLLM_ERROR_EXIT(kHipRuntimeError, "no HIP device is visible"); }
   MLLM_CHECK_HIP(hipSetDevice(0));
   hipDeviceProp_t prop{};
   MLLM_CHECK_HIP(hipGetDeviceProperties(&prop, 0));
-  MLLM_INFO("Found device: %s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+  MLLM_INFO("Found device: {} ({}, {} CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
   hipStream_t s = nullptr;
   MLLM_CHECK_HIP(hipStreamCreate(&s));  // default priority
   stream_ = s;
@@ -89,8 +89,7 @@ HipBackend::~HipBackend() {
 }
 
 Tensor& HipBackend::scratch(size_t bytes) {
-  if (scratch_.isNil() || scratch_.bytes() < bytes) {
-    synchronize();  // nothing in flight may still read the old buffer when it is freed
+  if (scratch_.isNil() || tensorBytes(scratch_) < bytes) {
     scratch_ = Tensor::empty({static_cast<int32_t>(bytes)}, kInt8, kHIP).alloc();
   }
   return scratch_;
@@ -104,9 +103,10 @@ std::shared_ptr<HipBackend> createHipBackend() { return std::make_shared<HipBack
 std::shared_ptr<HostBackend> createHostBackend() { return std::make_shared<HostBackend>(); }
 
 HipBackend& currentHipBackend() {
-  auto b = std::dynamic_pointer_cast<HipBackend>(MllmEngineCtx::instance().getBackend(kHIP));
-  if (!b) MLLM_ERROR_EXIT(kCoreError, "the backend registered for HIP is not a HipBackend");
-  return *b;
+  // BackendBase is not polymorphic: the device key is what identifies the backend registered under it
+  std::shared_ptr<BackendBase> b = MllmEngineCtx::instance().getBackend(kHIP);
+  if (!b || b->deviceType() != kHIP) { MLLM_ERROR_EXIT(kError, "no HIP backend is registered"); }
+  return *static_cast<HipBackend*>(b.get());
 }
 
 Tensor toDevice(const Tensor& host) {
@@ -114,7 +114,7 @@ Tensor toDevice(const Tensor& host) {
   Tensor d = Tensor::empty(host.shape(), host.dtype(), kHIP).alloc();
   d.setName(host.name());
   auto s = static_cast<hipStream_t>(currentHipBackend().stream());
-  MLLM_CHECK_HIP(hipMemcpyAsync(d.ptr<void>(), host.ptr<void>(), host.bytes(), hipMemcpyHostToDevice, s));
+  MLLM_CHECK_HIP(hipMemcpyAsync(d.ptr<char>(), host.ptr<char>(), tensorBytes(host), hipMemcpyHostToDevice, s));
   MLLM_CHECK_HIP(hipStreamSynchronize(s));  // the source may be pageable or go away
   return d;
 }
@@ -124,7 +124,7 @@ Tensor toHost(const Tensor& device) {
   Tensor h = Tensor::empty(device.shape(), device.dtype(), kCPU).alloc();
   h.setName(device.name());
   auto s = static_cast<hipStream_t>(currentHipBackend().stream());
-  MLLM_CHECK_HIP(hipMemcpyAsync(h.ptr<void>(), device.ptr<void>(), device.bytes(), hipMemcpyDeviceToHost, s));
+  MLLM_CHECK_HIP(hipMemcpyAsync(h.ptr<char>(), device.ptr<char>(), tensorBytes(device), hipMemcpyDeviceToHost, s));
   MLLM_CHECK_HIP(hipStreamSynchronize(s));
   return h;
 }

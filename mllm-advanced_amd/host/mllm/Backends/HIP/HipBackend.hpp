@@ -1,17 +1,31 @@
 // The MI355X backend: registers under kHIP, owns one HIP stream (default priority) and an
-// allocator, and provides the Linear and D2H op factories. Shape of a GPU backend in the
-// reference: mllm/Backends/CUDA/CUDABackend.cpp:18-24 (allocator + factory registration + D2H).
+// allocator, and provides the op factories of the W4A32 decoder path. Shape of a GPU backend in the
+// reference: mllm/Backends/CUDA/CUDABackend.cpp:18-24 (allocator + factory registration + D2H);
+// the operator set follows mllm/Backends/Arm/ArmBackend.cpp:42-52.
+//
+// This directory uses only names that exist in the reference's headers plus DeviceTypes::kHIP.
 #pragma once
 
 #include <memory>
 
 #include "mllm/Core/Tensor.hpp"
 #include "mllm/Engine/BackendBase.hpp"
+#include "mllm/Utils/Common.hpp"
 
 namespace mllm::hip {
 
+// Exit code for a failed HIP runtime or kernel-library call: the reference's one code for a GPU runtime
+// failure (mllm/Utils/Common.hpp:29), so that no enumerator has to be added there.
+inline constexpr ExitCode kHipRuntimeError = ExitCode::kCudaError;
+
+// Bytes a (dense) tensor's elements occupy. Tensor::bytes() is not const in the reference
+// (mllm/Core/Tensor.hpp:439) and operators receive their inputs as const references.
+inline size_t tensorBytes(const Tensor& t) { return t.numel() * dataTypeSize(t.dtype()); }
+
 // hipMalloc-backed allocator, 256-byte alignment (the kernels want 16-byte aligned blobs and
 // 256-byte aligned workspaces). Reference counterpart: mllm/Backends/CUDA/CUDAAllocator.cpp.
+// ctrlByMllmMemManager() is true: the engine's memory manager asks it for blocks and hands them out
+// again itself, so a tensor's birth and death do not reach hipMalloc / hipFree.
 class HipAllocator final : public Allocator {
  public:
   bool ctrlByMllmMemManager() override { return true; }
@@ -25,10 +39,10 @@ class HipAllocator final : public Allocator {
   [[nodiscard]] size_t alignSize() const override { return 256; }
 };
 
-// malloc-backed host allocator so host tensors can be created through the same Tensor API.
+// malloc-backed host allocator for a process that registers no CPU backend of the engine's own.
 class HostAllocator final : public Allocator {
  public:
-  bool ctrlByMllmMemManager() override { return true; }
+  bool ctrlByMllmMemManager() override { return false; }
   bool alloc(const std::shared_ptr<Storage>& storage) override;
   void free(const std::shared_ptr<Storage>& storage) override { free(storage.get()); }
   void free(Storage* storage) override;
@@ -47,7 +61,7 @@ class HostBackend final : public BackendBase {
 class HipBackend final : public BackendBase {
  public:
   HipBackend();
-  ~HipBackend() override;
+  ~HipBackend();  // BackendBase has no virtual destructor: hold a HipBackend through make_shared's pointer
 
   [[nodiscard]] void* stream() const { return stream_; }  // hipStream_t
   void synchronize() const;

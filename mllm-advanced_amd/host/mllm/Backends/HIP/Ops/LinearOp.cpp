@@ -15,11 +15,18 @@ namespace mllm::hip {
 namespace {
 
 void check(int rc, const char* what) {
-  if (rc != W4A32_OK) MLLM_ERROR_EXIT(kHipError, "%s failed: %s", what, w4a32_error_string(rc));
+  if (rc != W4A32_OK) { MLLM_ERROR_EXIT(kHipRuntimeError, "{} failed: {}", what, w4a32_error_string(rc)); }
 }
 
 void checkHip(hipError_t e, const char* what) {
-  if (e != hipSuccess) MLLM_ERROR_EXIT(kHipError, "%s failed: %s", what, hipGetErrorString(e));
+  if (e != hipSuccess) { MLLM_ERROR_EXIT(kHipRuntimeError, "{} failed: {}", what, hipGetErrorString(e)); }
+}
+
+// The six tile variants of KaiLinear_f32_qai8dxp_qsi4c32p_mxk_nxk (values 3..8 of LinearOpImplType,
+// mllm/Core/AOps/LinearOp.hpp:21-26): the one family this backend implements.
+bool isW4A32ImplType(LinearOpImplType t) {
+  const int v = static_cast<int>(t);
+  return v >= 3 && v <= 8;
 }
 
 // Packing parameters of the reference's six W4A32 tiles (ukernel table kai_linear.cpp:123-218): nr
@@ -48,14 +55,14 @@ size_t HipLinearOp::nativeBlobBytes(int N, int K) {
 void HipLinearOp::load(const std::shared_ptr<ParameterLoader>& ploader) {
   const int N = cargo_.out_channels, K = cargo_.in_channels;
   if (!isW4A32ImplType(cargo_.impl_type_)) {
-    MLLM_ERROR_EXIT(kCoreError, "%s: the HIP backend implements the W4A32 Linear family only "
-                    "(KaiLinear_f32_qai8dxp_qsi4c32p_mxk_nxk:*), impl type %d asked",
-                    name().c_str(), static_cast<int>(cargo_.impl_type_));
+    MLLM_ERROR_EXIT(kError, "{}: the HIP backend implements the W4A32 Linear family only "
+                    "(KaiLinear_f32_qai8dxp_qsi4c32p_mxk_nxk:*), impl type {} asked",
+                    name(), static_cast<int>(cargo_.impl_type_));
     return;
   }
   const size_t packed_bytes = w4a32_packed_bytes(N, K);
   if (packed_bytes == 0) {
-    MLLM_ERROR_EXIT(kShapeError, "%s: in_channels %d must be a positive multiple of 32", name().c_str(), K);
+    MLLM_ERROR_EXIT(kError, "{}: in_channels {} must be a positive multiple of 32", name(), K);
     return;
   }
   LinearOp::load(ploader);  // weight_/bias_ now alias the (host) parameter file
@@ -69,7 +76,7 @@ void HipLinearOp::load(const std::shared_ptr<ParameterLoader>& ploader) {
     Tensor b_dev;
     if (cargo_.bias) {
       if (bias_.dtype() != kFp32 || static_cast<int>(bias_.numel()) != N) {
-        MLLM_ERROR_EXIT(kShapeError, "%s.bias must be f32 [%d]", name().c_str(), N);
+        MLLM_ERROR_EXIT(kError, "{}.bias must be f32 [{}]", name(), N);
         return;
       }
       b_dev = toDevice(bias_);
@@ -82,11 +89,16 @@ void HipLinearOp::load(const std::shared_ptr<ParameterLoader>& ploader) {
     hb.synchronize();  // tmp, w_dev, b_dev are released on return
   } else if (weight_.dtype() == kInt8 && weight_.numel() == nativeBlobBytes(N, K)) {
     Tensor blob = toDevice(weight_);
+    const size_t u4_bytes = w4a32_native_u4_bytes(N, K), sc_bytes = w4a32_native_scale_bytes(N, K);
     const uint8_t* u4 = blob.ptr<uint8_t>();
-    const auto* sc = reinterpret_cast<const uint16_t*>(u4 + w4a32_native_u4_bytes(N, K));
-    const auto* bias = reinterpret_cast<const float*>(u4 + w4a32_native_u4_bytes(N, K) +
-                                                      w4a32_native_scale_bytes(N, K));
-    check(w4a32_repack_native(u4, sc, bias, N, K, packed.ptr<void>(), stream), "w4a32_repack_native");
+    const auto* sc = reinterpret_cast<const uint16_t*>(u4 + u4_bytes);
+    // The f32 bias follows the bf16 scales, so it is only 2-byte aligned when N * K/32 is odd (both in
+    // the file and in its device copy): the kernel gets a copy of its own, aligned like any tensor.
+    Tensor bias_host = Tensor::empty({N}, kFp32, kCPU).alloc();
+    std::memcpy(bias_host.ptr<char>(), weight_.ptr<char>() + u4_bytes + sc_bytes, (size_t)N * sizeof(float));
+    Tensor bias_dev = toDevice(bias_host);
+    check(w4a32_repack_native(u4, sc, bias_dev.ptr<float>(), N, K, packed.ptr<void>(), stream),
+          "w4a32_repack_native");
     hb.synchronize();
   } else if (const KaiTile kt = kaiTile(cargo_.impl_type_);
              weight_.dtype() == kInt8 && weight_.numel() == w4a32_kai_blob_bytes(N, K, kt.nr)) {
@@ -105,8 +117,8 @@ void HipLinearOp::load(const std::shared_ptr<ParameterLoader>& ploader) {
     check(w4a32_repack_native(u4, sc, bias, N, K, packed.ptr<void>(), stream), "w4a32_repack_native");
     hb.synchronize();
   } else {
-    MLLM_ERROR_EXIT(kShapeError, "%s.weight: expected f32 [%d,%d] or an int8 W4 blob of %zu bytes, "
-                    "got %s with %zu elements", name().c_str(), N, K, nativeBlobBytes(N, K),
+    MLLM_ERROR_EXIT(kError, "{}.weight: expected f32 [{},{}] or an int8 W4 blob of {} bytes, "
+                    "got {} with {} elements", name(), N, K, nativeBlobBytes(N, K),
                     dataTypes2Str(weight_.dtype()), weight_.numel());
     return;
   }
@@ -128,11 +140,11 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
   const auto& x = inputs[0];
   auto& y = outputs[0];
   if (x.device() != kHIP || x.dtype() != kFp32) {
-    MLLM_ERROR_EXIT(kCoreError, "%s: input must be an f32 tensor on the HIP device", name().c_str());
+    MLLM_ERROR_EXIT(kError, "{}: input must be an f32 tensor on the HIP device", name());
     return;
   }
   if (weight_.isNil() || weight_.device() != kHIP) {
-    MLLM_ERROR_EXIT(kCoreError, "%s: forward before load", name().c_str());
+    MLLM_ERROR_EXIT(kError, "{}: forward before load", name());
     return;
   }
   const int K = cargo_.in_channels, N = cargo_.out_channels;
@@ -140,7 +152,7 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
   // Arm/Ops/LinearOp.cpp:68; the engine only ever runs batch 1, where the two agree.)
   const int M = static_cast<int>(x.numel() / static_cast<size_t>(K));
   const size_t need = w4a32_workspace_bytes(M, K);
-  if (workspace_.isNil() || workspace_.bytes() < need) {
+  if (workspace_.isNil() || tensorBytes(workspace_) < need) {
     workspace_ = Tensor::empty({static_cast<int32_t>(need)}, kInt8, kHIP).alloc();
   }
   auto& hb = currentHipBackend();
@@ -150,7 +162,7 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
     Tensor& scratch = hb.scratch(lend);
     check(w4a32_quant_lhs(x.ptr<float>(), M, K, K, workspace_.ptr<void>(), hb.stream()), "w4a32_quant_lhs");
     check(w4a32_matmul_quantized_splitk(y.ptr<float>(), workspace_.ptr<void>(), weight_.ptr<void>(), M, K, N,
-                                        scratch.ptr<void>(), scratch.bytes(), hb.stream()),
+                                        scratch.ptr<void>(), tensorBytes(scratch), hb.stream()),
           "w4a32_matmul_quantized_splitk");
     return;
   }
@@ -160,13 +172,11 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
   // Stays asynchronous on the backend's stream: a host consumer goes through D2H, which waits.
 }
 
-void HipD2HOp::reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
-  outputs.emplace_back(Tensor::empty(inputs[0].shape(), inputs[0].dtype(), kCPU));
-}
+HipD2HOp::HipD2HOp(const D2HOpCargo& cargo) : D2HOp(cargo) {}
 
 void HipD2HOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
   auto s = static_cast<hipStream_t>(currentHipBackend().stream());
-  checkHip(hipMemcpyAsync(outputs[0].ptr<void>(), inputs[0].ptr<void>(), inputs[0].bytes(),
+  checkHip(hipMemcpyAsync(outputs[0].ptr<char>(), inputs[0].ptr<char>(), tensorBytes(inputs[0]),
                           hipMemcpyDeviceToHost, s), "hipMemcpyAsync(D2H)");
   checkHip(hipStreamSynchronize(s), "hipStreamSynchronize");
 }
@@ -176,7 +186,7 @@ Tensor quantizeLinearForFile(const Tensor& weight_f32, const Tensor& bias_f32_or
   const int N = weight_f32.shape()[0], K = weight_f32.shape()[1];
   const size_t u4_bytes = w4a32_native_u4_bytes(N, K), sc_bytes = w4a32_native_scale_bytes(N, K);
   if (u4_bytes == 0) {
-    MLLM_ERROR_EXIT(kShapeError, "quantize: in_channels %d must be a positive multiple of 32", K);
+    MLLM_ERROR_EXIT(kError, "quantize: in_channels {} must be a positive multiple of 32", K);
     return Tensor::nil();
   }
   auto& hb = currentHipBackend();

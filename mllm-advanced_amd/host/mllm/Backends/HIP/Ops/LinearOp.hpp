@@ -2,6 +2,7 @@
 // (reference counterpart: mllm/Backends/Arm/Ops/LinearOp.hpp:15-29, LinearOp.cpp:22-134,235-265).
 #pragma once
 
+#include "mllm/Core/AOps/D2HOp.hpp"
 #include "mllm/Core/AOps/LinearOp.hpp"
 
 namespace mllm::hip {
@@ -39,13 +40,11 @@ class HipLinearOpFactory : public TypedOpFactory<OpType::kLinear, LinearOpCargo>
   }
 };
 
-// Device -> host copy as an op (reference: mllm/Core/AOps/D2HOp.*, mllm/Backends/CUDA/Ops/D2HOp.cpp).
-struct D2HOpCargo : public BaseOpCargo<D2HOpCargo> {};
-
-class HipD2HOp final : public BaseOp {
+// Device -> host copy as an op (reference: mllm/Core/AOps/D2HOp.hpp, mllm/Backends/CUDA/Ops/D2HOp.cpp:18-22);
+// Tensor::cpu() dispatches it with from_device_type = the tensor's device, to_device_type = kCPU.
+class HipD2HOp final : public D2HOp {
  public:
-  explicit HipD2HOp(const D2HOpCargo&) : BaseOp(OpType::kD2H) {}
-  void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+  explicit HipD2HOp(const D2HOpCargo& cargo);
   void forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
 };
 

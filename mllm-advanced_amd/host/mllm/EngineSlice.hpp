@@ -1,9 +1,13 @@
 // The slice of the reference engine that the HIP backend is compiled against when it is built outside the
-// reference tree: device and data type keys, logging, storage and allocator, tensor, operator base classes,
-// the Linear operator's abstract half, backend base, context and the parameter file reader. Inside the
-// reference tree the headers of these names (the one-line files beside this one forward to here) are the
-// reference's own, and this file is not used. Signatures follow the reference so that mllm/Backends/HIP and
-// mllm/Models/ds_qwen2/HipQwen2.* compile unchanged against either; each part cites the file it stands for.
+// reference tree: exit codes and logging, device and data type keys, storage and allocator, tensor, operator
+// base classes and the abstract operators the backend implements, backend base, memory manager, context and
+// the parameter file reader. Inside the reference tree the headers of these names (the one-line files beside
+// this one forward to here) are the reference's own, and this file is not used.
+//
+// Everything mllm/Backends/HIP and mllm/Models/ds_qwen2/HipQwen2.* use from here has the reference's name,
+// signature, constness and enumerator values, so those sources compile unchanged against either tree (a test
+// compiles them against the reference's headers). Members marked "stand-in only" exist for this build's own
+// tests and are not used by the backend sources. Each part cites the file it stands for.
 #pragma once
 
 #include <cstddef>
@@ -11,29 +15,32 @@
 #include <cstdio>
 #include <cstdlib>
 #include <functional>
+#include <list>
 #include <memory>
+#include <sstream>
 #include <string>
 #include <typeinfo>
 #include <unordered_map>
 #include <vector>
 
 // ====================================================================================================
-// stands for mllm/Utils/Log.hpp
+// stands for mllm/Utils/Log.hpp and mllm/Utils/Common.hpp
 // ====================================================================================================
-// Error convention of the engine this layer plugs into: no exceptions, no status codes; an
-// unrecoverable condition prints and exits with a code (reference: mllm/Utils/Log.hpp:59-64,
-// codes mllm/Utils/Common.hpp:23-30). The handler is replaceable so tests can observe it.
-
+// Error convention of the engine: no exceptions, no status codes; an unrecoverable condition prints and
+// exits with a code (reference: mllm/Utils/Log.hpp:59-64, codes mllm/Utils/Common.hpp:23-30). Messages are
+// "{}"-style, as the reference's macros pass them to fmt::format. The reference's *_EXIT macros expand to
+// an `if` block followed by `exit(code)`: a caller must put them inside braces of their own.
+// The exit handler is replaceable so tests can observe it (stand-in only).
 
 namespace mllm {
 
-enum ExitCode : int {  // NOLINT
+enum ExitCode : int32_t {  // NOLINT
   kSuccess = 0,
-  kCoreError = 1,
-  kAssert = 2,
-  kIOError = 3,
-  kHipError = 4,
-  kShapeError = 5,
+  kError,
+  kAssert,
+  kSliceOB,
+  kMemory,
+  kCudaError,
 };
 
 inline std::function<void(int, const std::string&)>& errorHandler() {
@@ -45,24 +52,50 @@ inline std::function<void(int, const std::string&)>& errorHandler() {
   return h;
 }
 
-template <typename... Args>
-inline std::string formatMsg(const char* fmt, Args... args) {
-  char buf[1024];
-  std::snprintf(buf, sizeof buf, fmt, args...);
-  return std::string(buf);
-}
-inline std::string formatMsg(const char* fmt) { return std::string(fmt); }
+namespace detail {
 
+template <typename T>
+inline std::string showArg(const T& v) {
+  std::ostringstream os;
+  os << v;
+  return os.str();
+}
+
+// The subset of fmt::format the backend uses: "{}" takes the next argument, "{{" and "}}" are braces.
+template <typename... Args>
+inline std::string braceFormat(const std::string& fmt, const Args&... args) {
+  const std::vector<std::string> shown = {showArg(args)...};
+  std::string out;
+  size_t next = 0;
+  for (size_t i = 0; i < fmt.size(); ++i) {
+    if (fmt[i] == '{' && i + 1 < fmt.size() && fmt[i + 1] == '}') {
+      out += next < shown.size() ? shown[next] : std::string("{}");
+      ++next;
+      ++i;
+    } else if ((fmt[i] == '{' || fmt[i] == '}') && i + 1 < fmt.size() && fmt[i + 1] == fmt[i]) {
+      out += fmt[i];
+      ++i;
+    } else {
+      out += fmt[i];
+    }
+  }
+  return out;
+}
+
+}  // namespace detail
 }  // namespace mllm
 
-#define MLLM_ERROR_EXIT(code, ...) ::mllm::errorHandler()((code), ::mllm::formatMsg(__VA_ARGS__))
-#define MLLM_WARN(...) std::fprintf(stderr, "[mllm][WARN] %s\n", ::mllm::formatMsg(__VA_ARGS__).c_str())
-#define MLLM_INFO(...) std::fprintf(stderr, "[mllm][INFO] %s\n", ::mllm::formatMsg(__VA_ARGS__).c_str())
-#define MLLM_RT_ASSERT(expr)                                                                  \
-  do {                                                                                        \
-    if (!(expr)) MLLM_ERROR_EXIT(::mllm::kAssert, "assert failed: %s (%s:%d)", #expr, __FILE__, __LINE__); \
-  } while (0)
-#define MLLM_RT_ASSERT_EQ(a, b) MLLM_RT_ASSERT((a) == (b))
+#define MLLM_INFO(...) std::fprintf(stderr, "[INFO] %s\n", ::mllm::detail::braceFormat(__VA_ARGS__).c_str())
+#define MLLM_WARN(...) std::fprintf(stderr, "[WARN] %s\n", ::mllm::detail::braceFormat(__VA_ARGS__).c_str())
+#define MLLM_ERROR_EXIT(code, ...) ::mllm::errorHandler()((code), ::mllm::detail::braceFormat(__VA_ARGS__))
+#define MLLM_ASSERT_EXIT(code, ...) ::mllm::errorHandler()((code), ::mllm::detail::braceFormat(__VA_ARGS__))
+#define MLLM_RT_ASSERT(statement) \
+  if (!(statement)) { MLLM_ASSERT_EXIT(::mllm::ExitCode::kAssert, "{}", #statement); }
+#define MLLM_RT_ASSERT_EQ(statement1, statement2)                                      \
+  if ((statement1) != (statement2)) {                                                  \
+    MLLM_ASSERT_EXIT(::mllm::ExitCode::kAssert, "{} != {}", #statement1, #statement2); \
+  }
+#define NYI(...) std::fprintf(stderr, "[NYI] %s\n", ::mllm::detail::braceFormat(__VA_ARGS__).c_str())
 
 // ====================================================================================================
 // stands for mllm/Core/DeviceTypes.hpp
@@ -70,7 +103,6 @@ inline std::string formatMsg(const char* fmt) { return std::string(fmt); }
 // Device enum of the engine, with the one value this backend adds.
 // Reference: mllm/Core/DeviceTypes.hpp:18-27 has kCPU, kCUDA, kOpenCL, kQNN; a backend is looked
 // up by this key (mllm/Engine/Context.cpp:56-59), so a new device needs a new enumerator: kHIP.
-
 
 namespace mllm {
 
@@ -103,13 +135,15 @@ inline DeviceTypes str2DeviceType(const std::string& s) {
 // stands for mllm/Core/DataTypes.hpp
 // ====================================================================================================
 // The element types this path touches, with the numeric codes the .mllm container stores
-// (reference: mllm/Core/DataTypes.hpp:19-65 - Int8 = 2, Int32 = 4, Int64 = 5, Fp16 = 8, Fp32 = 9, BF16 = 24).
-
+// (reference: mllm/Core/DataTypes.hpp:19-65 - Int8 = 2, Int16 = 3, Int32 = 4, Int64 = 5, Fp16 = 8, Fp32 = 9,
+// BF16 = 24).
 
 namespace mllm {
 
 enum DataTypes : uint32_t {  // NOLINT
+  kDataTypes_Start = 0,
   kInt8 = 2,
+  kInt16 = 3,
   kInt32 = 4,
   kInt64 = 5,
   kFp16 = 8,
@@ -120,36 +154,36 @@ enum DataTypes : uint32_t {  // NOLINT
 inline size_t dataTypeSize(DataTypes t) {
   switch (t) {
     case kInt8: return 1;
+    case kInt16:
     case kFp16:
     case kBF16: return 2;
     case kInt32:
     case kFp32: return 4;
     case kInt64: return 8;
+    default: return 0;
   }
-  return 0;
 }
 
 inline const char* dataTypes2Str(DataTypes t) {
   switch (t) {
     case kInt8: return "Int8";
+    case kInt16: return "Int16";
     case kInt32: return "Int32";
     case kInt64: return "Int64";
     case kFp16: return "Fp16";
     case kFp32: return "Fp32";
     case kBF16: return "BF16";
+    default: return "Unknown";
   }
-  return "Unknown";
 }
 
 }  // namespace mllm
 
 // ====================================================================================================
-// stands for mllm/Engine/Allocator.hpp
+// stands for mllm/Core/Storage.hpp and mllm/Engine/Allocator.hpp
 // ====================================================================================================
-// Allocator interface a backend hands to the engine (reference: mllm/Engine/Allocator.hpp:18-32,
-// same nine virtuals with the same meaning).
-
-
+// Allocator interface a backend hands to the engine (reference: mllm/Engine/Allocator.hpp:18-32, the same
+// nine virtuals with the same meaning; like the reference's, the class has no virtual destructor).
 
 namespace mllm {
 
@@ -160,6 +194,7 @@ class Storage : public std::enable_shared_from_this<Storage> {
   void* ptr_ = nullptr;
   size_t size_ = 0;
   DeviceTypes device_ = kCPU;
+  uint32_t custom_32bit_uuid_ = 0xFFFFFFFFu;
 };
 
 class Allocator {
@@ -179,72 +214,155 @@ class Allocator {
 }  // namespace mllm
 
 // ====================================================================================================
-// stands for mllm/Core/Tensor.hpp
+// stands for mllm/Core/TensorImpl.hpp and mllm/Core/Tensor.hpp
 // ====================================================================================================
-// A contiguous tensor over reference-counted storage: the slice of the engine's Tensor that an
-// operator boundary needs (reference: mllm/Core/Tensor.hpp:52-140, mllm/Core/TensorImpl.hpp:43-142).
-// Tensor::empty() only describes a tensor; alloc() asks the device's allocator for memory, as
-// BaseOp::setup does for op outputs (mllm/Core/AOps/BaseOp.cpp:25-46).
-
-
+// A tensor view over reference-counted storage: the part of the engine's Tensor that an operator boundary
+// needs (reference: mllm/Core/Tensor.hpp:52-140, 255-440, mllm/Core/TensorImpl.hpp:20-160). Views here are
+// always dense row-major (an offset into the storage plus a shape); the reference's strided views are what
+// its CPU transpose/slice produce and no HIP operator creates them.
+// Tensor::empty() only describes a tensor; alloc() asks the memory manager for memory, as BaseOp::setup does
+// for op outputs (mllm/Core/AOps/BaseOp.cpp:25-46).
 
 namespace mllm {
 
-enum TensorMemTypes : int {  // NOLINT
-  kNormal = 0,  // owned: freed through the allocator when the last reference goes
-  kParams = 1,  // aliases a mapped parameter file or caller memory: never freed here
+enum TensorMemTypes : int32_t {  // NOLINT
+  kTensorMemTypes_Start = 0,
+  kNormal,  // owned: returned to the memory manager when the last reference goes
+  kExtraInput,
+  kExtraOutput,
+  kManual,
+  kGlobal,
+  kParams,  // aliases a mapped parameter file: never freed by the tensor
+  kReference,
+  kQnnAppReadWrite,
+  kTensorMemTypes_End,
 };
 
-class TensorStorage : public Storage {
+class TensorStorage final : public Storage {
  public:
   ~TensorStorage() override;
+  static std::shared_ptr<TensorStorage> create(const std::vector<int32_t>& shape, DataTypes dtype,
+                                               DeviceTypes device);
+  std::string name_;
+  DataTypes dtype_ = kFp32;
   TensorMemTypes mem_type_ = kNormal;
-  std::shared_ptr<void> keep_alive_;  // e.g. the mapped file a kParams tensor aliases
+  std::shared_ptr<void> keep_alive_;  // stand-in only: the mapped file a kParams storage aliases
 };
 
-class TensorViewImpl {
+class TensorViewImpl : public std::enable_shared_from_this<TensorViewImpl> {
  public:
+  using storage_t = std::shared_ptr<TensorStorage>;
   using shape_t = std::vector<int32_t>;
+  using dtype_t = DataTypes;
+  using device_t = DeviceTypes;
+
+  TensorViewImpl() = default;
+  TensorViewImpl(const TensorViewImpl&) = delete;
+
+  DataTypes dtype() const { return storage_->dtype_; }
+  DeviceTypes device() const { return storage_->device_; }
+  storage_t storage() const { return storage_; }
+  [[nodiscard]] std::string name() const { return storage_->name_; }
+  [[nodiscard]] TensorMemTypes memType() const { return storage_->mem_type_; }
+  [[nodiscard]] uint32_t uuid() const { return storage_->custom_32bit_uuid_; }
+  uint64_t address() const { return reinterpret_cast<uint64_t>(storage_->ptr_); }
+  [[nodiscard]] void* rptr() const {
+    return static_cast<char*>(storage_->ptr_) + static_cast<size_t>(storage_offset_) * dataTypeSize(dtype());
+  }
+  size_t size() const { return numel() * dataTypeSize(dtype()); }  // bytes, not aligned
+  size_t numel() const;
+  [[nodiscard]] std::vector<int32_t> shape() const { return shape_; }
+  [[nodiscard]] std::vector<int32_t> stride() const;
+  bool isContiguous() const { return true; }
+  int32_t storageOffset() const { return storage_offset_; }
+
+  static std::shared_ptr<TensorViewImpl> create(const std::vector<int32_t>& shape,
+                                                const std::shared_ptr<TensorStorage>& storage);
+  static std::shared_ptr<TensorViewImpl> create(int32_t storage_offset, const std::vector<int32_t>& shape,
+                                                const std::shared_ptr<TensorStorage>& storage);
+
+  template <typename T>
+  T* ptr() {
+    return static_cast<T*>(rptr());
+  }
+
+ private:
+  int32_t storage_offset_ = 0;  // in elements
   shape_t shape_;
-  DataTypes dtype_ = kFp32;
-  std::string name_;
-  std::shared_ptr<TensorStorage> storage_;
+  std::shared_ptr<TensorStorage> storage_ = nullptr;
 };
 
 class Tensor {
  public:
   using shape_t = TensorViewImpl::shape_t;
+  using dtype_t = TensorViewImpl::dtype_t;
+  using device_t = TensorViewImpl::device_t;
 
   Tensor() = default;
   explicit Tensor(const std::shared_ptr<TensorViewImpl>& impl) : impl_(impl) {}
 
-  [[nodiscard]] bool isNil() const { return impl_ == nullptr; }
-  static Tensor nil() { return {}; }
+  [[nodiscard]] inline bool isNil() const { return impl_ == nullptr; }
+  static inline Tensor nil() { return {}; }
 
   // Describes a tensor; no memory yet.
-  static Tensor empty(const shape_t& shape, DataTypes dtype = kFp32, DeviceTypes device = kCPU);
-  // Wraps memory owned by someone else (a mapped file, a caller's buffer).
-  static Tensor wrap(void* ptr, const shape_t& shape, DataTypes dtype, DeviceTypes device,
-                     std::shared_ptr<void> keep_alive = nullptr);
-
+  static Tensor empty(const std::vector<int32_t>& shape, DataTypes dtype = kFp32, DeviceTypes device = kCPU);
   Tensor& alloc();
 
-  [[nodiscard]] const shape_t& shape() const { return impl_->shape_; }
-  [[nodiscard]] DataTypes dtype() const { return impl_->dtype_; }
-  [[nodiscard]] DeviceTypes device() const { return impl_->storage_->device_; }
-  [[nodiscard]] size_t numel() const;
-  [[nodiscard]] size_t bytes() const { return numel() * dataTypeSize(dtype()); }
-  [[nodiscard]] const std::string& name() const { return impl_->name_; }
-  void setName(const std::string& n) { impl_->name_ = n; }
-  [[nodiscard]] const std::shared_ptr<TensorViewImpl>& impl() const { return impl_; }
+  [[nodiscard]] std::string name() const { return impl_->name(); }
+  [[nodiscard]] TensorMemTypes memType() const { return impl_->memType(); }
+  Tensor& setName(const std::string& name);
+  Tensor& setMemType(TensorMemTypes mem_type);
+  [[nodiscard]] DataTypes dtype() const { return impl_->dtype(); }
+  [[nodiscard]] DeviceTypes device() const { return impl_->device(); }
+  [[nodiscard]] std::vector<int32_t> shape() const { return impl_->shape(); }
+  [[nodiscard]] size_t numel() const { return impl_->numel(); }
+  [[nodiscard]] uint32_t uuid() const { return impl_->uuid(); }
+  [[nodiscard]] bool isContiguous() const { return impl_->isContiguous(); }
+  Tensor contiguous() { return *this; }
+  // Same storage under another shape; goes through the backend's View operator as in the reference
+  // (mllm/Core/Tensor.cpp: view() dispatches OpType::kView).
+  Tensor view(const std::vector<int>& indicies);
+  [[nodiscard]] inline std::shared_ptr<TensorViewImpl> impl() const { return impl_; }
 
   template <typename T>
-  [[nodiscard]] T* ptr() const {
-    return static_cast<T*>(impl_->storage_->ptr_);
+  T* ptr() const {
+    return impl_->ptr<T>();
   }
 
+  size_t bytes() { return impl_->size(); }  // not const in the reference either (Tensor.hpp:439)
+
  private:
-  std::shared_ptr<TensorViewImpl> impl_;
+  std::shared_ptr<TensorViewImpl> impl_ = nullptr;
+};
+
+}  // namespace mllm
+
+// ====================================================================================================
+// stands for mllm/Engine/SymbolTable.hpp
+// ====================================================================================================
+
+namespace mllm {
+
+// reference: mllm/Engine/SymbolTable.hpp:19-66 - registering a key twice and reading a missing key exit.
+template <typename KeyT, typename ValueT>
+class SymbolTable {
+ public:
+  void reg(const KeyT& name, const ValueT& v) {
+    if (has(name)) { MLLM_ERROR_EXIT(kError, "When registing new value, found symbol table already has a value key"); }
+    symbol_table_.insert({name, v});
+  }
+  bool has(const KeyT& name) { return symbol_table_.count(name) != 0; }
+  void remove(const KeyT& name) { symbol_table_.erase(name); }
+  ValueT& operator[](const KeyT& name) {
+    if (!has(name)) {
+      MLLM_ERROR_EXIT(kError, "When accessing symbol in symbol table. Found symbol key not in symbol table");
+    }
+    return symbol_table_[name];
+  }
+  std::unordered_map<KeyT, ValueT>& _ref_raw_data() { return symbol_table_; }
+
+ private:
+  std::unordered_map<KeyT, ValueT> symbol_table_;
 };
 
 }  // namespace mllm
@@ -252,40 +370,79 @@ class Tensor {
 // ====================================================================================================
 // stands for mllm/Core/AOps/BaseOp.hpp
 // ====================================================================================================
-// Abstract operator API (reference: mllm/Core/AOps/BaseOp.hpp:118-234): the engine calls
+// Abstract operator API (reference: mllm/Core/AOps/BaseOp.hpp:21-234): the engine calls
 // reshape -> setup -> forward on an op that a backend's factory created from a type-erased cargo.
-
-
 
 namespace mllm {
 
 class ParameterLoader;
 
-// Only the values this layer uses; kLinear keeps the reference's position-independent name.
-enum class OpType : int32_t {
+// Same enumerators in the same order as the reference (BaseOp.hpp:21-77).
+enum class OpType : int32_t {  // NOLINT
   kOpType_Start = 0,
+  kFill,
+  kAdd,
+  kSub,
+  kMul,
+  kDiv,
+  kMatMul,
+  kLLMEmbeddingToken,
   kLinear,
+  kRoPE,
+  kSoftmax,
+  kTranspose,
+  kRMSNorm,
+  kSiLU,
+  kKVCache,
+  kCausalMask,
+  kCastType,
   kD2H,
+  kH2D,
+  kSplit,
+  kView,
+  kFlashAttention_2,
+  kRepeat,
+  kPermute,
+  kConv3D,
+  kConv2D,
+  kConv1D,
+  kGELU,
+  kLayerNorm,
+  kMultimodalRoPE,
+  kVisionRoPE,
+  kQuickGELU,
+  kCopy,
+  kClone,
+  kNeg,
+  kConcat,
   kOpType_End,
 };
 
-inline const char* opType2Str(OpType t) {
-  switch (t) {
-    case OpType::kLinear: return "Linear";
-    case OpType::kD2H: return "D2H";
-    default: return "Unknown";
-  }
-}
+const char* opType2Str(OpType type);
 
-// CRTP base of cargos (reference BaseOp.hpp:120-148): per-op thread count, default 4.
+// CRTP base of cargos (reference BaseOp.hpp:120-148): per-op thread count, default 4, and the
+// inputs' / outputs' element types.
 template <typename DerivedT>
 class BaseOpCargo {
  public:
+  BaseOpCargo() = default;
+  DerivedT& setInputsDtype(size_t pos, DataTypes dtype) {
+    if (pos >= inputs_dtypes_.size()) inputs_dtypes_.resize(pos + 1, kFp32);
+    inputs_dtypes_[pos] = dtype;
+    return *static_cast<DerivedT*>(this);
+  }
+  DerivedT& setOutputsDtype(size_t pos, DataTypes dtype) {
+    if (pos >= outputs_dtypes_.size()) outputs_dtypes_.resize(pos + 1, kFp32);
+    outputs_dtypes_[pos] = dtype;
+    return *static_cast<DerivedT*>(this);
+  }
   [[nodiscard]] int thread() const { return threads_; }
   void setThreads(int threads) { threads_ = threads; }
 
  private:
   int threads_ = 4;
+  std::vector<DataTypes> inputs_dtypes_;
+  std::vector<DataTypes> outputs_dtypes_;
 };
 
 // Type-erased cargo; as<T>() throws std::bad_cast on a wrong type (reference BaseOp.hpp:151-181).
@@ -320,9 +477,10 @@ class BaseOp : public std::enable_shared_from_this<BaseOp> {
   virtual ~BaseOp() = default;
 
   virtual void load(const std::shared_ptr<ParameterLoader>& ploader) {}
+  virtual void trace(void* trace_context, const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {}
   virtual void forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {}
   virtual void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {}
-  // Allocates every output through its device's allocator (reference BaseOp.cpp:25-46).
+  // Allocates every output that has no memory yet (reference BaseOp.cpp:25-46).
   virtual void setup(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs);
   virtual params_t params() { return {}; }
 
@@ -330,7 +488,6 @@ class BaseOp : public std::enable_shared_from_this<BaseOp> {
   void setName(const std::string& name) { name_ = name; }
   [[nodiscard]] DeviceTypes device() const { return device_type_; }
   void setDeviceType(DeviceTypes d) { device_type_ = d; }
-  [[nodiscard]] OpType opType() const { return op_type_; }
 
  private:
   DeviceTypes device_type_ = kCPU;
@@ -364,8 +521,6 @@ class TypedOpFactory : public BaseOpFactory {
 // Linear: cargo, implementation selector and the device-independent part of the op
 // (reference: mllm/Core/AOps/LinearOp.hpp:17-99, mllm/Core/AOps/LinearOp.cpp:17-106).
 
-
-
 namespace mllm {
 
 // Same enumerators and values as the reference (LinearOp.hpp:17-35): model configs and quantizer
@@ -388,25 +543,21 @@ enum class LinearOpImplType {
   kKai_End = 256,
 };
 
-inline bool isW4A32ImplType(LinearOpImplType t) {
-  const int v = static_cast<int>(t);
-  return v >= 3 && v <= 8;
-}
-
 struct LinearOpCargo : public BaseOpCargo<LinearOpCargo> {
   int32_t in_channels = 0;
   int32_t out_channels = 0;
   bool bias = true;
   bool transpose = false;
-  LinearOpImplType impl_type_ = LinearOpImplType::kDefault;
 
   // "<family>:<tile>" -> enum; unknown strings warn and fall back to kDefault (LinearOp.cpp:53-55).
   static LinearOpImplType parseLinearOpImplTypeStr(const std::string& type_str);
+
+  LinearOpImplType impl_type_ = LinearOpImplType::kDefault;
 };
 
 class LinearOp : public BaseOp {
  public:
-  explicit LinearOp(const LinearOpCargo& cargo) : BaseOp(OpType::kLinear), cargo_(cargo) {}
+  explicit LinearOp(const LinearOpCargo& cargo);
 
   // weight = "<name>.weight", bias = "<name>.bias" when cargo.bias (LinearOp.cpp:60-63)
   void load(const std::shared_ptr<ParameterLoader>& ploader) override;
@@ -414,9 +565,9 @@ class LinearOp : public BaseOp {
   void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
   params_t params() override;
 
-  Tensor& weight() { return weight_; }
-  Tensor& bias() { return bias_; }
-  [[nodiscard]] const LinearOpCargo& cargo() const { return cargo_; }
+  inline Tensor& weight() { return weight_; }
+  inline Tensor& bias() { return bias_; }
+  inline const LinearOpCargo& cargo() const { return cargo_; }
 
  protected:
   Tensor weight_;
@@ -427,23 +578,231 @@ class LinearOp : public BaseOp {
 }  // namespace mllm
 
 // ====================================================================================================
+// stands for mllm/Core/AOps/D2HOp.hpp
+// ====================================================================================================
+
+namespace mllm {
+
+// reference: mllm/Core/AOps/D2HOp.hpp:16-38, D2HOp.cpp:15-45 (output = input's shape and type on
+// cargo.to_device_type); Tensor::cpu() dispatches it (mllm/Core/Tensor.cpp).
+struct D2HOpCargo : public BaseOpCargo<D2HOpCargo> {
+  DeviceTypes from_device_type;
+  DeviceTypes to_device_type;
+};
+
+class D2HOp : public BaseOp {
+ public:
+  explicit D2HOp(const D2HOpCargo& cargo);
+  void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+
+ protected:
+  D2HOpCargo cargo_;
+};
+
+}  // namespace mllm
+
+// ====================================================================================================
+// stands for mllm/Core/AOps/{View,RMSNorm,RoPE,KVCache,FlashAttention2,MatMul,SiLU,Elewise,LLMEmbeddingToken}Op.hpp
+// ====================================================================================================
+// The abstract halves of the decoder's operators: cargos with the reference's fields and defaults, and the
+// device-independent load / reshape / params of each (reference file:line at each class). The layouts are
+// the ones the reference's flash-attention model variant uses (modeling_ds_qwen2_fa2_fp16.hpp:88-133):
+// activations [B, S, H, D], RoPE with layout kBSHD, KV cache with layout kBSHD_NO_REPEAT.
+
+namespace mllm {
+
+// reference: mllm/Core/AOps/ViewOp.hpp:15-38, ViewOp.cpp:34-90 (one -1 dimension is inferred; the output
+// shares the input's storage, forward does nothing)
+struct ViewOpCargo : public BaseOpCargo<ViewOpCargo> {
+  std::vector<int32_t> to_shape_;
+};
+
+class ViewOp : public BaseOp {
+ public:
+  explicit ViewOp(const ViewOpCargo& cargo);
+  void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+  void setup(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+  inline std::vector<int32_t> toWhichShape() { return cargo_.to_shape_; }
+
+ protected:
+  ViewOpCargo cargo_;
+};
+
+// reference: mllm/Core/AOps/RMSNormOp.hpp:15-43, RMSNormOp.cpp (weight = "<name>.weight", output like input)
+struct RMSNormOpCargo : public BaseOpCargo<RMSNormOpCargo> {
+  float epsilon;
+  bool add_unit_offset = false;  // Gemma
+};
+
+class RMSNormOp : public BaseOp {
+ public:
+  explicit RMSNormOp(const RMSNormOpCargo& cargo);
+  void load(const std::shared_ptr<ParameterLoader>& ploader) override;
+  void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+  params_t params() override;
+
+ protected:
+  Tensor weight_;
+  RMSNormOpCargo cargo_;
+};
+
+// reference: mllm/Core/AOps/RoPEOp.hpp:15-56
+enum class RoPETypes : int32_t {
+  kRoPETypes_Start = 0,
+  kLlama2,
+  kRoPETypes_End,
+};
+
+struct RoPEOpCargo : public BaseOpCargo<RoPEOpCargo> {
+  enum RoPELayoutType {
+    kBHSD = 0,  // eager attention
+    kBSHD = 1,  // flash attention
+  };
+  RoPETypes type = RoPETypes::kLlama2;
+  float theta;
+  int max_position_embeddings;
+  int dims;
+  RoPELayoutType layout_type = kBHSD;
+};
+
+class RoPEOp : public BaseOp {
+ public:
+  explicit RoPEOp(const RoPEOpCargo& cargo);
+  void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+
+ protected:
+  int cur_seq_cnt_ = 0;
+  RoPEOpCargo cargo_;
+};
+
+// reference: mllm/Core/AOps/KVCacheOp.hpp:17-52
+struct KVCacheOpCargo : public BaseOpCargo<KVCacheOpCargo> {
+  enum KVCacheLayoutType {
+    kBHSD_REPEAT = 0,     // eager attention
+    kBSHD_NO_REPEAT = 1,  // flash attention
+  };
+  int32_t heads_num = 1;
+  int32_t dim_per_head = 0;
+  int32_t head_repeat_times = 1;
+  DataTypes cached_elements_dtype = kFp32;
+  int32_t pre_alloc_seq_len = 1024;
+  int32_t re_alloc_multiplier = 2;
+  KVCacheLayoutType layout_type = KVCacheLayoutType::kBHSD_REPEAT;
+};
+
+class KVCacheOp : public BaseOp {
+ public:
+  explicit KVCacheOp(const KVCacheOpCargo& cargo);
+
+ protected:
+  Tensor cache_;
+  KVCacheOpCargo cargo_;
+};
+
+// reference: mllm/Core/AOps/FlashAttention2Op.hpp:15-46, FlashAttention2Op.cpp:35-44 (output like the query)
+struct FlashAttn2OpCargo : public BaseOpCargo<FlashAttn2OpCargo> {
+  int32_t B;
+  int32_t q_head;
+  int32_t kv_head;
+  int32_t D;
+  int32_t threads = 4;
+  bool hp_exp = false;
+  bool causal_mask = true;
+};
+
+class FlashAttn2Op : public BaseOp {
+ public:
+  explicit FlashAttn2Op(const FlashAttn2OpCargo& cargo);
+  void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+
+ protected:
+  FlashAttn2OpCargo cargo_;
+};
+
+// reference: mllm/Core/AOps/MatMulOp.hpp:15-44, MatMulOp.cpp (output [..., M, N] from [..., M, K] and
+// [..., K, N], either operand transposed on request)
+struct MatMulOpCargo : public BaseOpCargo<MatMulOpCargo> {
+  bool transpose_a = false;
+  bool transpose_b = false;
+};
+
+class MatMulOp : public BaseOp {
+ public:
+  explicit MatMulOp(const MatMulOpCargo& cargo);
+  void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+  inline bool transposeA() { return cargo_.transpose_a; }
+  inline bool transposeB() { return cargo_.transpose_b; }
+
+ protected:
+  MatMulOpCargo cargo_;
+};
+
+// reference: mllm/Core/AOps/SiLUOp.hpp:15-38
+struct SiLUOpCargo : public BaseOpCargo<SiLUOpCargo> {};
+
+class SiLUOp : public BaseOp {
+ public:
+  explicit SiLUOp(const SiLUOpCargo& cargo);
+  void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+
+ protected:
+  SiLUOpCargo cargo_;
+};
+
+// reference: mllm/Core/AOps/ElewiseOp.hpp:15-66 (no cargo fields; output like input 0; the reference gives
+// every element-wise class OpType::kAdd in its constructor, ElewiseOp.hpp:30)
+struct AddOpCargo : public BaseOpCargo<AddOpCargo> {};
+struct MulOpCargo : public BaseOpCargo<MulOpCargo> {};
+
+class AddOp : public BaseOp {
+ public:
+  AddOp();
+  void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+};
+
+class MulOp : public BaseOp {
+ public:
+  MulOp();
+  void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+};
+
+// reference: mllm/Core/AOps/LLMEmbeddingTokenOp.hpp:15-45, LLMEmbeddingTokenOp.cpp (weight =
+// "<name>.weight" [vocab, hidden]; ids [B, S] -> [B, S, hidden] in the weight's type)
+struct LLMEmbeddingTokenOpCargo : public BaseOpCargo<LLMEmbeddingTokenOpCargo> {
+  int vocab_size = 0;
+  int hidden_size = 0;
+};
+
+class LLMEmbeddingTokenOp : public BaseOp {
+ public:
+  explicit LLMEmbeddingTokenOp(const LLMEmbeddingTokenOpCargo& cargo);
+  void load(const std::shared_ptr<ParameterLoader>& ploader) override;
+  void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+  params_t params() override;
+
+ protected:
+  Tensor weight_;
+  LLMEmbeddingTokenOpCargo cargo_;
+};
+
+}  // namespace mllm
+
+// ====================================================================================================
 // stands for mllm/Engine/BackendBase.hpp
 // ====================================================================================================
-// What a device backend is to the engine (reference: mllm/Engine/BackendBase.hpp:20-46): a device
-// key, an allocator and a table of op factories.
-
-
+// What a device backend is to the engine (reference: mllm/Engine/BackendBase.hpp:20-46): a device key, an
+// allocator and a table of op factories. As in the reference the class has no virtual member: a backend is
+// recognised by deviceType(), not by dynamic_cast, and a derived destructor is not an override.
 
 namespace mllm {
 
 class BackendBase {
  public:
   explicit BackendBase(DeviceTypes device) : device_(device) {}
-  virtual ~BackendBase() = default;
 
-  template <typename... Factories>
+  template <typename... Args>
   void regOpFactory() {
-    (..., regOne<Factories>());
+    (..., (_reg_one_op_factory<Args>()));
   }
 
   [[nodiscard]] std::shared_ptr<Allocator> getAllocator() const { return allocator_; }
@@ -452,68 +811,85 @@ class BackendBase {
 
  private:
   template <typename T>
-  void regOne() {
-    auto f = std::make_shared<T>();
-    op_factory_table_[static_cast<int>(f->opType())] = f;
+  void _reg_one_op_factory() {
+    auto ptr = std::make_shared<T>();
+    op_factory_table_.reg(ptr->opType(), ptr);
   }
 
  protected:
   DeviceTypes device_;
-  std::unordered_map<int, std::shared_ptr<BaseOpFactory>> op_factory_table_;
+  SymbolTable<OpType, std::shared_ptr<BaseOpFactory>> op_factory_table_;
   std::shared_ptr<Allocator> allocator_ = nullptr;
 };
 
 }  // namespace mllm
 
 // ====================================================================================================
-// stands for mllm/Engine/Context.hpp
+// stands for mllm/Engine/MemManager.hpp and mllm/Engine/Context.hpp
 // ====================================================================================================
-// The engine context, reduced to what calls the Linear path (reference:
-// mllm/Engine/Context.hpp:26-106, Context.cpp:56-122): a process-wide registry of backends keyed
-// by device, their allocators, and eager dispatch = reshape -> setup -> forward.
-
-
+// The memory manager and the engine context, reduced to what calls this path (reference:
+// mllm/Engine/MemManager.hpp:63-140, mllm/Engine/Context.hpp:26-106, Context.cpp:56-122): a process-wide
+// registry of backends keyed by device, and eager dispatch = reshape -> setup -> forward.
+//
+// Like the reference's manager (a buddy allocator over 128 MiB segments it gets from the backend's
+// allocator, MemManager.cpp:40-75, 140-160) this one does not go to the device allocator per tensor: blocks
+// of a device whose allocator says ctrlByMllmMemManager() are rounded up to a size class and, when their
+// tensor dies, kept in a per-device free list for the next tensor of that class. A device allocation
+// (hipMalloc) and a device free (which synchronises the device) happen only when a class runs dry and in
+// releaseCached(). Reuse without synchronisation is safe because a backend issues all its work on one
+// stream: the new owner's kernels are ordered behind the old owner's.
 
 namespace mllm {
 
 class MemManager {
  public:
-  void regAllocator(DeviceTypes device, const std::shared_ptr<Allocator>& a) { table_[device] = a; }
-  std::shared_ptr<Allocator> allocator(DeviceTypes device) const;
+  ~MemManager();
   void alloc(const std::shared_ptr<Storage>& s);
   void free(Storage* s);
+  void regAllocator(DeviceTypes device, const std::shared_ptr<Allocator>& allocator);
+
+  // stand-in only
+  void releaseCached();                                 // gives every cached block back to its allocator
+  [[nodiscard]] size_t deviceAllocCalls() const { return device_alloc_calls_; }
 
  private:
-  std::unordered_map<int, std::shared_ptr<Allocator>> table_;
+  static size_t sizeClass(size_t bytes);
+  SymbolTable<DeviceTypes, std::shared_ptr<Allocator>> allocators_st_;
+  std::unordered_map<int, std::unordered_map<size_t, std::list<void*>>> free_blocks_;  // [device][class]
+  std::unordered_map<void*, size_t> block_class_;                                        // live + cached
+  size_t device_alloc_calls_ = 0;
 };
 
 class MllmEngineCtx {
  public:
   static MllmEngineCtx& instance();
 
-  void registerBackend(const std::shared_ptr<BackendBase>& backend);
+  void registerBackend(const std::shared_ptr<BackendBase>& new_backend);
   std::shared_ptr<BackendBase> getBackend(DeviceTypes device);
-  [[nodiscard]] std::shared_ptr<MemManager> mem() const { return mem_; }
+  [[nodiscard]] std::shared_ptr<MemManager> mem() const { return main_thread_mem_; }
+  uint32_t getUUID() { return custom_uuid_giver_++; }
 
   // Named layers: created once (Module::reg time in the reference), dispatched by name.
-  void regLayerOp(const std::string& name, const std::shared_ptr<BaseOp>& op) { layer_ops_[name] = op; }
   std::vector<Tensor> dispatch(const std::string& name, const std::vector<Tensor>& inputs);
   // Anonymous ops: created on the backend of inputs[0]'s device, then run.
-  std::vector<Tensor> dispatch(OpType op_type, const BaseOpCargoBase& cargo,
+  std::vector<Tensor> dispatch(OpType op_type, const BaseOpCargoBase& base_cargo,
                                const std::vector<Tensor>& inputs);
-
-  void setPerf(bool on) { perf_ = on; }
   void shutdown();
 
+  bool perf_ = false;
+
+  // stand-in only: the reference keeps named layer ops in its thread object (Thread.hpp:46)
+  void regLayerOp(const std::string& name, const std::shared_ptr<BaseOp>& op) { layer_ops_[name] = op; }
+
  private:
-  MllmEngineCtx() : mem_(std::make_shared<MemManager>()) {}
+  MllmEngineCtx() : main_thread_mem_(std::make_shared<MemManager>()) {}
   std::vector<Tensor> run(const std::shared_ptr<BaseOp>& op, const std::vector<Tensor>& inputs,
                           const std::string& what);
 
-  std::shared_ptr<MemManager> mem_;
-  std::unordered_map<int, std::shared_ptr<BackendBase>> backends_;
+  std::shared_ptr<MemManager> main_thread_mem_;
+  SymbolTable<DeviceTypes, std::shared_ptr<BackendBase>> backends_table_;
   std::unordered_map<std::string, std::shared_ptr<BaseOp>> layer_ops_;
-  bool perf_ = false;
+  uint32_t custom_uuid_giver_ = 0;
 };
 
 }  // namespace mllm
@@ -525,8 +901,6 @@ class MllmEngineCtx {
 // (reference: mllm/Engine/ParameterReader.hpp:27-57 structs, ParameterReader.cpp:41-104 loader,
 // :114-181 writer; the Python writer pads each tensor to 64 bytes, tools/convertor.py:173,207-211,
 // which the offsets in the descriptors already account for).
-
-
 
 namespace mllm {
 
@@ -558,14 +932,14 @@ class ParameterLoader {
   ParameterLoader() = default;
   explicit ParameterLoader(const std::string& file_name);  // mmaps; tensors alias the mapping
 
-  // Exits with kIOError if the name is missing, as the reference's table lookup would.
+  // Exits with kError if the name is missing, as the reference's table lookup does.
   std::shared_ptr<TensorViewImpl> operator[](const std::string& name);
-  [[nodiscard]] bool has(const std::string& name) const { return params_.count(name) != 0; }
   std::unordered_map<std::string, std::shared_ptr<TensorViewImpl>>& params() { return params_; }
-  [[nodiscard]] const std::string& modelName() const { return model_name_; }
 
-  // In-memory registration (what the quantizer does when it replaces a tensor).
-  void insert(const std::string& name, const Tensor& t);
+  // stand-in only
+  [[nodiscard]] bool has(const std::string& name) const { return params_.count(name) != 0; }
+  [[nodiscard]] const std::string& modelName() const { return model_name_; }
+  void insert(const std::string& name, const Tensor& t);  // in-memory registration
 
  private:
   std::shared_ptr<void> mapping_;
@@ -575,8 +949,12 @@ class ParameterLoader {
 
 std::shared_ptr<ParameterLoader> load(const std::string& file_path);
 
-// Writes host tensors in the unpadded C++ layout of the reference writer.
-void write(const std::shared_ptr<ParameterLoader>& params, const std::string& file_path,
-           const std::string& model_name = "mllm");
+// Writes host tensors in the unpadded layout of the reference's C++ writer (ParameterReader.cpp:114-181),
+// with the reference's signatures (ParameterReader.hpp:124-130).
+void write(const std::string& file_path, const std::unordered_map<std::string, Tensor>& params,
+           const std::string& model_name);
+void write(const std::string& file_path,
+           const std::unordered_map<std::string, std::shared_ptr<TensorViewImpl>>& params,
+           const std::string& model_name);
 
 }  // namespace mllm

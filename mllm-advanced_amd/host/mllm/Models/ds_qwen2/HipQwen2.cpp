@@ -12,11 +12,11 @@ namespace mllm::models {
 namespace {
 
 void check(int rc, const char* what) {
-  if (rc != W4A32_OK) MLLM_ERROR_EXIT(kHipError, "%s failed: %s", what, w4a32_error_string(rc));
+  if (rc != W4A32_OK) { MLLM_ERROR_EXIT(hip::kHipRuntimeError, "{} failed: {}", what, w4a32_error_string(rc)); }
 }
 
 void checkHip(hipError_t e, const char* what) {
-  if (e != hipSuccess) MLLM_ERROR_EXIT(kHipError, "%s failed: %s", what, hipGetErrorString(e));
+  if (e != hipSuccess) { MLLM_ERROR_EXIT(hip::kHipRuntimeError, "{} failed: {}", what, hipGetErrorString(e)); }
 }
 
 }  // namespace
@@ -31,7 +31,7 @@ struct HipQWenForCausalLM::Impl {
   }
 };
 
-HipQWenForCausalLM::HipQWenForCausalLM(const QWenConfig& cfg) : cfg_(cfg), impl_(new Impl) {
+HipQWenForCausalLM::HipQWenForCausalLM(const HipQWenConfig& cfg) : cfg_(cfg), impl_(new Impl) {
   dcfg_.hidden = cfg.hidden_size;
   dcfg_.n_heads = cfg.num_attention_heads;
   dcfg_.n_kv_heads = cfg.num_key_value_heads;
@@ -66,7 +66,7 @@ void HipQWenForCausalLM::load(const std::shared_ptr<ParameterLoader>& ploader) {
   auto f32 = [&](const std::string& name, size_t numel) -> const float* {
     Tensor host((*ploader)[name]);
     if (host.dtype() != kFp32 || host.numel() != numel) {
-      MLLM_ERROR_EXIT(kShapeError, "%s: expected %zu f32 values, got %s x %zu", name.c_str(), numel,
+      MLLM_ERROR_EXIT(kError, "{}: expected {} f32 values, got {} x {}", name, numel,
                       dataTypes2Str(host.dtype()), host.numel());
     }
     Tensor dev = hip::toDevice(host);
@@ -95,9 +95,16 @@ void HipQWenForCausalLM::load(const std::shared_ptr<ParameterLoader>& ploader) {
 
   const size_t bytes = w4a32_decoder_state_bytes(&dcfg_);
   if (bytes == 0) {
-    MLLM_ERROR_EXIT(kShapeError, "unsupported decoder shape (head_dim must be 128, sizes multiples of 32)");
+    MLLM_ERROR_EXIT(kError, "unsupported decoder shape (head_dim must be 128, sizes multiples of 32)");
   }
-  state_ = Tensor::empty({static_cast<int32_t>(bytes)}, kInt8, kHIP).alloc();
+  // A tensor dimension is an int32: the state (mostly the KV cache, 2 * layers * kv_heads * max_seq * 512
+  // bytes) is counted in 8-byte elements, which reaches 16 GiB.
+  const size_t words = (bytes + 7) / 8;
+  if (words > 0x7FFFFFFFull) {
+    MLLM_ERROR_EXIT(kMemory, "decoder state of {} bytes (max_cache_length {}) exceeds one tensor", bytes,
+                    dcfg_.max_seq);
+  }
+  state_ = Tensor::empty({static_cast<int32_t>(words)}, kInt64, kHIP).alloc();
   token_ = Tensor::empty({1}, kInt64, kHIP).alloc();
   auto& hb = hip::currentHipBackend();
   check(w4a32_decoder_init(&dcfg_, state_.ptr<void>(), hb.stream()), "w4a32_decoder_init");
@@ -110,9 +117,9 @@ void HipQWenForCausalLM::reset() { position_ = 0; }
 int64_t HipQWenForCausalLM::prefill(const std::vector<int64_t>& tokens) {
   auto& hb = hip::currentHipBackend();
   auto stream = static_cast<hipStream_t>(hb.stream());
-  if (tokens.empty()) MLLM_ERROR_EXIT(kCoreError, "prefill: empty prompt");
+  if (tokens.empty()) { MLLM_ERROR_EXIT(kError, "prefill: empty prompt"); }
   if (position_ + (int)tokens.size() > dcfg_.max_seq) {
-    MLLM_ERROR_EXIT(kShapeError, "prefill: %zu tokens at position %d exceed max_cache_length %d",
+    MLLM_ERROR_EXIT(kError, "prefill: {} tokens at position {} exceed max_cache_length {}",
                     tokens.size(), position_, dcfg_.max_seq);
   }
   Tensor ids = Tensor::empty({static_cast<int32_t>(tokens.size())}, kInt64, kHIP).alloc();
@@ -136,7 +143,7 @@ int64_t HipQWenForCausalLM::step() {
   auto& hb = hip::currentHipBackend();
   auto stream = static_cast<hipStream_t>(hb.stream());
   if (position_ >= dcfg_.max_seq) {
-    MLLM_ERROR_EXIT(kShapeError, "step: the cache (max_cache_length %d) is full", dcfg_.max_seq);
+    MLLM_ERROR_EXIT(kError, "step: the cache (max_cache_length {}) is full", dcfg_.max_seq);
   }
   if (!impl_->warmed) {
     // The very first step runs eagerly: it brings the decode kernels' code objects in, which must

@@ -27,9 +27,10 @@
 
 namespace mllm::models {
 
-// The fields of the reference's QWenConfig (configuration_ds_qwen2.hpp:18-90) this model reads;
-// same names, same defaults.
-struct QWenConfig {
+// The fields of the reference's QWenConfig (configuration_ds_qwen2.hpp:18-90) this model reads, under the
+// same names and with the same defaults; a struct of its own name so that it can live beside the reference's
+// (whose constructor wants a JSON file) in one program.
+struct HipQWenConfig {
   int32_t num_attention_heads = 12;
   int32_t num_hidden_layers = 28;
   int32_t num_key_value_heads = 2;
@@ -48,7 +49,7 @@ struct QWenConfig {
 
 class HipQWenForCausalLM {
  public:
-  explicit HipQWenForCausalLM(const QWenConfig& cfg);
+  explicit HipQWenForCausalLM(const HipQWenConfig& cfg);
   ~HipQWenForCausalLM();
   HipQWenForCausalLM(const HipQWenForCausalLM&) = delete;
   HipQWenForCausalLM& operator=(const HipQWenForCausalLM&) = delete;
@@ -70,7 +71,7 @@ class HipQWenForCausalLM {
 
  private:
   struct Impl;
-  QWenConfig cfg_;
+  HipQWenConfig cfg_;
   w4a32_decoder_config dcfg_{};
   std::vector<std::shared_ptr<hip::HipLinearOp>> linears_;  // keep the device blobs alive
   std::vector<Tensor> f32_params_;

@@ -44,7 +44,7 @@ int main(int argc, char** argv) {
   ctx.registerBackend(hip::createHostBackend());
   ctx.registerBackend(hip::createHipBackend());
 
-  models::QWenConfig cfg;
+  models::HipQWenConfig cfg;
   cfg.num_attention_heads = 2;
   cfg.num_key_value_heads = 1;
   cfg.num_hidden_layers = 2;
@@ -82,7 +82,7 @@ int main(int argc, char** argv) {
     }
     addParam(params, "model.norm.weight", {H}, gen, 0.1f, 1.0f);
     addParam(params, "lm_head.weight", {V, H}, gen, 0.05f, 0.0f);
-    write(params, path, "tiny-qwen2");
+    write(path, params->params(), "tiny-qwen2");
   }
   auto loaded = load(path);
   EXPECT(loaded->has("model.layers.1.mlp.down_proj.weight") && loaded->has("lm_head.weight"));

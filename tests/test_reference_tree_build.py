@@ -1,0 +1,78 @@
+"""The HIP backend sources, compiled against the reference's own headers.
+
+mllm/Backends/HIP/** and mllm/Models/ds_qwen2/HipQwen2.* are meant to be dropped into the reference tree as
+they are. This test puts them into an overlay directory in front of the reference's include root, together
+with the one change the reference needs (the enumerator DeviceTypes::kHIP), and runs the compiler's syntax
+pass over every .cpp with the reference's headers (fmt and half come from the headers torch ships). It needs
+the reference tree, which exists only where this repository was written: skipped elsewhere. CPU only.
+"""
+import glob
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HOST = os.path.join(ROOT, "mllm-advanced_amd", "host")
+REFERENCE = "/root/reference"
+
+# What a maintainer adds to mllm/Core/DeviceTypes.hpp (the same lines INTEGRATION.md lists).
+DEVICE_TYPES_PATCH = [
+    (r"^(\s*)kQNN,\s*$", r"\1kQNN,\n\1kHIP,"),
+    (r'^(\s*)case DeviceTypes::kQNN: return "QNN";\s*$',
+     r'\1case DeviceTypes::kQNN: return "QNN";\n\1case DeviceTypes::kHIP: return "HIP";'),
+]
+
+
+def _overlay(tmp_path):
+    over = tmp_path / "overlay"
+    shutil.copytree(os.path.join(HOST, "mllm", "Backends", "HIP"), over / "mllm" / "Backends" / "HIP",
+                    ignore=shutil.ignore_patterns("*.o"))
+    (over / "mllm" / "Models" / "ds_qwen2").mkdir(parents=True)
+    for f in glob.glob(os.path.join(HOST, "mllm", "Models", "ds_qwen2", "HipQwen2.?pp")):
+        shutil.copy(f, over / "mllm" / "Models" / "ds_qwen2")
+    text = open(os.path.join(REFERENCE, "mllm", "Core", "DeviceTypes.hpp")).read()
+    for pat, rep in DEVICE_TYPES_PATCH:
+        text, n = re.subn(pat, rep, text, count=1, flags=re.M)
+        assert n == 1, f"the reference's DeviceTypes.hpp no longer has the line {pat!r}"
+    (over / "mllm" / "Core").mkdir(parents=True)
+    (over / "mllm" / "Core" / "DeviceTypes.hpp").write_text(text)
+    return over
+
+
+@pytest.mark.skipif(not os.path.isdir(os.path.join(REFERENCE, "mllm")), reason="needs the reference tree")
+def test_hip_backend_sources_compile_against_the_reference_headers(tmp_path):
+    import torch
+
+    torch_inc = os.path.join(os.path.dirname(torch.__file__), "include")
+    over = _overlay(tmp_path)
+    sources = sorted(str(p) for p in over.rglob("*.cpp"))
+    assert len(sources) >= 3
+    for src in sources:
+        # none of these may lean on the stand-in header this repository builds against
+        assert "EngineSlice" not in open(src).read()
+        cmd = ["g++", "-std=c++20", "-fsyntax-only", "-DFMT_HEADER_ONLY", "-D__HIP_PLATFORM_AMD__",
+               f"-I{over}", f"-I{REFERENCE}", f"-I{torch_inc}", f"-I{os.path.join(ROOT, 'include')}",
+               "-I/opt/rocm/include", src]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        errors = [ln for ln in r.stderr.splitlines() if "error" in ln]
+        assert r.returncode == 0 and not errors, f"{os.path.relpath(src, over)}:\n" + "\n".join(errors[:20])
+
+
+def test_exit_macros_are_always_inside_braces():
+    """The reference's MLLM_*_EXIT macros are an `if` block followed by `exit(code)`: used as the body of
+    an unbraced `if` they would exit unconditionally. Every use in the backend sources must be the first
+    statement of a braced block or stand alone on its line."""
+    bad = []
+    files = glob.glob(os.path.join(HOST, "mllm", "Backends", "HIP", "**", "*.?pp"), recursive=True)
+    files += glob.glob(os.path.join(HOST, "mllm", "Models", "ds_qwen2", "*.?pp"))
+    assert files
+    for path in files:
+        for no, line in enumerate(open(path), 1):
+            if re.search(r"\bif\s*\(.*\)\s*MLLM_(ERROR|ASSERT|WARN|FATAL)_EXIT", line):
+                bad.append(f"{path}:{no}: {line.strip()}")
+            if re.search(r'MLLM_\w+\(.*"[^"]*%[sdzuf]', line):
+                bad.append(f"{path}:{no}: printf-style message: {line.strip()}")
+    assert not bad, "\n".join(bad)
