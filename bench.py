@@ -469,7 +469,13 @@ def main():
             e1.record(stream)
             stream.synchronize()
             decode_ms = e0.elapsed_time(e1)
-            assert dec.position == 512 + n_new and first == int(first)
+            # the timed tokens are real: the position advanced once per replay, the last step's logits are
+            # finite and its token is the first maximum of those logits
+            logits = dec.logits
+            assert dec.position == 512 + n_new
+            assert bool(torch.isfinite(logits).all()), "decoder produced non-finite logits"
+            assert int(dec.token) == int(torch.argmax(logits)), "token is not the argmax of the logits"
+            assert 0 <= first < V
         extra["decoder_config4"] = {
             "workload": "28 layers, hidden 1536, 12 q / 2 kv heads x 128, MLP 8960, vocab 151936, rope theta 1e6, "
                         "f32 KV cache; batch 1, 512 random prompt ids, 256 greedy steps; all Linears W4A32 "

@@ -338,8 +338,11 @@ def test_decoder_runner_at_the_model_s_widths(pkg, prompt_len):
     # its input rows to int8, and a 1e-7 difference in a row (f32 summation order of the attention) flips a
     # few roundings; one flip moves an output by weight x step (down_proj: 0.02 x 0.03), a row of 8960
     # collects about 15 of them, and the logits end up 0 (no flip), 1e-7 or about 1e-2 apart - measured on
-    # operators that each agree with the oracle to 3e-7 on the oracle's own inputs. So 5e-2 here; the
-    # operators are held to 2e-5 in their own tests.
+    # operators that each agree with the oracle to 3e-7 on the oracle's own inputs. So 5e-2 here: this test
+    # shows that the runner strings the operators together correctly (and picks the greedy token of its own
+    # logits); that no operator at these widths is off by more than 2e-5 is the business of
+    # test_prefill_layer_at_the_model_s_widths_every_operator_on_its_own_inputs, which feeds the oracle the
+    # HIP path's own quantised rows so that nothing is amplified.
     import decoder_oracle as do
 
     rng = np.random.default_rng(prompt_len)
@@ -369,6 +372,115 @@ def test_decoder_runner_at_the_model_s_widths(pkg, prompt_len):
             assert int(dec.token) == do.greedy(got)
     finally:
         do.Linear.threads = 1
+
+
+def _lhs_raw(aq, recip, neg_zp):
+    """The oracle's packed row format (f32 reciprocal scale, i32 negated zero point, K int8 values) from
+    what w4a32_export_lhs returns: the rows exactly as the product kernel consumed them."""
+    m, k = aq.shape
+    raw = np.empty((m, k + 8), dtype=np.int8)
+    raw[:, 0:4] = recip.reshape(m, 1).view(np.int8)
+    raw[:, 4:8] = neg_zp.reshape(m, 1).view(np.int8)
+    raw[:, 8:] = aq
+    return raw
+
+
+@pytest.mark.parametrize("M", [300, 520])
+def test_prefill_layer_at_the_model_s_widths_every_operator_on_its_own_inputs(pkg, orc, M):
+    """One decoder layer at hidden 1536, 12 / 2 heads, MLP 8960, issued as the runner's prefill issues it
+    (fused add + norm + quantiser, grouped q,k,v, rope + append, matrix-core attention, o, gate,up pair,
+    split-K down whose parts the next quantiser adds up), with every operator checked against the oracle
+    on the HIP path's OWN inputs: the quantised rows are exported from the workspace and fed to the
+    oracle's product, so no difference can be amplified by a re-quantisation in between and every Linear
+    is held to 2e-5 (block sums are exact integers on both sides; only f32 summation order differs)."""
+    import decoder_oracle as do
+
+    H, Hq, Hkv, I, D = 1536, 12, 2, 8960, 128
+    eps = 1e-6
+    rng = np.random.default_rng(1000 + M)
+    w = {n: (rng.standard_normal(shape) * 0.02).astype(np.float32) for n, shape in
+         [("q", (Hq * D, H)), ("k", (Hkv * D, H)), ("v", (Hkv * D, H)), ("o", (H, Hq * D)),
+          ("gate", (I, H)), ("up", (I, H)), ("down", (H, I))]}
+    bias = {n: (rng.standard_normal(w[n].shape[0]) * 0.1).astype(np.float32) for n in ("q", "k", "v")}
+    norm1 = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    norm2 = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    q4 = {n: orc.quant_rhs(w[n]) for n in w}
+    packed = {n: pkg.repack_native(dev(q4[n][0]), dev(q4[n][1].view(np.int16)),
+                                   dev(bias[n]) if n in bias else None, *w[n].shape) for n in w}
+    rows = np.unique(np.concatenate([np.arange(0, M, 23), [M - 1, 31, 32, 255, 256]]))
+
+    def product_ok(ws, K, name, got, what):
+        aq, recip, nzp = (t.cpu().numpy() for t in pkg.export_lhs(ws, M, K))
+        raw = _lhs_raw(aq[rows], recip[rows], nzp[rows])
+        ref = orc.matmul_packed(raw, *q4[name], bias=bias.get(name), threads=16)
+        err = max_abs_rel(got.cpu().numpy()[rows], ref)
+        assert err <= 2e-5, (what, err)
+        return raw
+
+    h0 = (rng.standard_normal((M, H)) * 2).astype(np.float32)
+    d0 = rng.standard_normal((M, H)).astype(np.float32)
+
+    # [add + norm + quantiser]: the sum is exact, the quantised rows reconstruct the normalised rows to half a step
+    ws1, h1 = pkg.quant_lhs_norm(dev(h0), dev(norm1), eps, delta=dev(d0))
+    assert np.array_equal(h1.cpu().numpy(), h0 + d0)
+    aq, recip, nzp = (t.cpu().numpy() for t in pkg.export_lhs(ws1, M, H))
+    want_rows = do.rmsnorm(h0 + d0, norm1, eps)
+    back = (aq.astype(np.float32) + nzp[:, None]) * recip[:, None]
+    assert np.all(np.abs(back - want_rows) <= recip[:, None] * 0.5001 + 1e-6)
+
+    # [q, k, v grouped]
+    qkv = pkg.matmul_quantized_grouped(ws1, [packed["q"], packed["k"], packed["v"]], [Hq * D, Hkv * D, Hkv * D], M, H)
+    for name, y in zip("qkv", qkv):
+        product_ok(ws1, H, name, y, name + "_proj")
+
+    # [rope + append] [attention] on the HIP path's own q, k, v
+    q_h, k_h, v_h = (t.cpu().numpy() for t in qkv)
+    sin, cos = pkg.op_rope_table(M, D, 1e6)
+    kc = torch.zeros((Hkv, M, D), dtype=torch.float32, device="cuda")
+    vc = torch.zeros_like(kc)
+    q_rot = qkv[0].clone()
+    pkg.op_rope_kv(q_rot, qkv[1], qkv[2], sin, cos, kc, vc, Hq, Hkv, D, 0)
+    attn = pkg.op_attention_prefill(q_rot, kc, vc, Hq, Hkv, D, 0)
+    s_ref, c_ref = do.rope_tables(M, D, 1e6)
+    q_ref = do.rope(q_h.reshape(M, Hq, D), s_ref, c_ref, 0)
+    k_ref = do.rope(k_h.reshape(M, Hkv, D), s_ref, c_ref, 0)
+    assert max_abs_rel(q_rot.cpu().numpy(), q_ref.reshape(M, -1)) <= 6e-5      # one ulp of powf at 500 rad
+    kc_h, vc_h = kc.cpu().numpy(), vc.cpu().numpy()
+    assert max_abs_rel(kc_h, k_ref.transpose(1, 0, 2)) <= 6e-5
+    assert np.array_equal(vc_h, v_h.reshape(M, Hkv, D).transpose(1, 0, 2))
+    arows = rows[::3]
+    a_ref = np.stack([do.attention(q_rot.cpu().numpy().reshape(M, Hq, D)[r:r + 1], kc_h, vc_h, int(r))[0]
+                      for r in arows])
+    assert max_abs_rel(attn.cpu().numpy()[arows], a_ref) <= 2e-5
+
+    # [quantiser] [o]
+    ws2 = pkg.quant_lhs(attn)
+    o_out = pkg.matmul_quantized(ws2, packed["o"], M, Hq * D, H)
+    product_ok(ws2, Hq * D, "o", o_out, "o_proj")
+
+    # [add + norm + quantiser] [gate, up pair -> silu * mul]
+    ws3, h2 = pkg.quant_lhs_norm(h1, dev(norm2), eps, delta=o_out)
+    assert torch.equal(h2, h1 + o_out)
+    act = pkg.matmul_quantized_silu_pair(ws3, packed["gate"], packed["up"], M, H, I)
+    aq, recip, nzp = (t.cpu().numpy() for t in pkg.export_lhs(ws3, M, H))
+    raw3 = _lhs_raw(aq[rows], recip[rows], nzp[rows])
+    g_ref = orc.matmul_packed(raw3, *q4["gate"], threads=16)
+    u_ref = orc.matmul_packed(raw3, *q4["up"], threads=16)
+    assert max_abs_rel(act.cpu().numpy()[rows], do.silu_mul(g_ref, u_ref)) <= 2e-5
+
+    # [quantiser] [down, split over K; its parts are added by the next layer's add + norm + quantiser]
+    ws4 = pkg.quant_lhs(act)
+    scratch, parts = pkg.matmul_quantized_splitk_parts(ws4, packed["down"], M, I, H)
+    assert parts > 1, "down_proj at these sizes is expected to run split over K"
+    part_sum = scratch[:parts * M * H * 4].view(torch.float32).reshape(parts, M, H).cpu().numpy()
+    total = part_sum[0].copy()
+    for i in range(1, parts):
+        total += part_sum[i]
+    product_ok(ws4, I, "down", torch.from_numpy(total), "down_proj parts")
+    down_whole = pkg.matmul_quantized_splitk(ws4, packed["down"], M, I, H)
+    product_ok(ws4, I, "down", down_whole, "down_proj")
+    _, h3 = pkg.quant_lhs_norm_parts(h2, scratch, parts, packed["down"], I, dev(norm1), eps)
+    assert np.array_equal(h3.cpu().numpy(), h2.cpu().numpy() + total)
 
 
 def test_decoder_step_replays_from_a_graph(pkg):
@@ -489,3 +601,67 @@ def test_decode_linear_fusions_match_separate_operators(pkg, orc, K, Ns, pair):
     base = pkg.matmul_grouped(dev(x), packed, Ns) if len(Ns) > 1 else [pkg.matmul(dev(x), packed[0], Ns[0])]
     for a, b in zip(plain, base):
         assert torch.equal(a, b)
+
+
+def test_full_size_decoder_properties(pkg):
+    """The configuration the tokens/s figure is quoted on, at full depth: 28 layers, hidden 1536, 12 / 2
+    heads, MLP 8960, vocabulary 151936, 512-token prompt, then greedy steps replayed from a captured graph.
+    No CPU model finishes this in seconds, so it is held to properties: every step's logits are finite, its
+    token is the first maximum of its logits, the position advances by one, and the replayed graph gives,
+    bit for bit, the tokens and logits of eagerly launched steps from the same state."""
+    H, Hq, Hkv, I, V, L = 1536, 12, 2, 8960, 151936, 28
+    g = torch.Generator(device="cuda").manual_seed(4)
+    rw = lambda n, k: pkg.quant_pack_rhs(torch.randn((n, k), generator=g, device="cuda") * 0.02)
+    rb = lambda n, k: pkg.quant_pack_rhs(torch.randn((n, k), generator=g, device="cuda") * 0.02,
+                                         torch.randn((n,), generator=g, device="cuda") * 0.02)
+    norm = lambda: 1 + 0.1 * torch.randn((H,), generator=g, device="cuda")
+    layers = [{"q": rb(Hq * 128, H), "k": rb(Hkv * 128, H), "v": rb(Hkv * 128, H), "o": rw(H, Hq * 128),
+               "gate": rw(I, H), "up": rw(I, H), "down": rw(H, I), "attn_norm": norm(), "ffn_norm": norm()}
+              for _ in range(L)]
+    emb = torch.randn((V, H), generator=g, device="cuda")
+    final_norm, lm_head = norm(), rw(V, H)
+    prompt = torch.randint(0, V, (512,), generator=g, device="cuda", dtype=torch.int64)
+    steps = 36
+
+    def make():
+        return pkg.Decoder(H, Hq, Hkv, I, V, layers, emb, final_norm, lm_head, max_seq=1024,
+                           max_batch_tokens=512, rope_theta=1e6, rms_eps=1e-6)
+
+    eager = make()
+    eager.prefill(prompt)
+    torch.cuda.synchronize()
+    first_logits = eager.logits.clone()
+    assert bool(torch.isfinite(first_logits).all()) and float(first_logits.abs().max()) > 0
+    assert int(eager.token) == int(torch.argmax(first_logits)) and eager.position == 512
+    toks, logits = [], []
+    for i in range(steps):
+        eager.step()
+        lg = eager.logits.clone()
+        assert bool(torch.isfinite(lg).all()), i
+        assert int(eager.token) == int(torch.argmax(lg)), i          # torch.argmax: first maximum too
+        assert eager.position == 513 + i
+        toks.append(int(eager.token))
+        logits.append(lg)
+    assert len(set(toks)) > 1                                        # not stuck on one token
+
+    dec = make()
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        dec.prefill(prompt)
+        dec.step()                                                   # warm-up outside the capture
+        dec.prefill(prompt)                                          # rewind to the state the eager run started from
+        s.synchronize()
+        assert torch.equal(dec.logits, first_logits)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            dec.step()
+        s.synchronize()
+        assert dec.position == 512                                   # a capture executes nothing
+        for i in range(steps):
+            graph.replay()
+            s.synchronize()
+            assert int(dec.token) == toks[i], i
+            assert torch.equal(dec.logits, logits[i]), i
+            if i % 8 == 0:
+                _ = (dec.logits * 2).sum().item()                    # unrelated eager work between replays
+        assert dec.position == 512 + steps

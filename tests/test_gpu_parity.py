@@ -33,6 +33,12 @@ VIT_SHAPES = [
     ("vit_fc1", 1280, 5120, True),
     ("vit_fc2", 5120, 1280, True),
 ]
+# the Qwen2-VL patch merger: four patches' 1280 features side by side -> 5120 -> 1536, both with bias
+# (mllm/Models/qwen2vl/modeling_qwen2vl.hpp:112-137); 1024 patches give 256 rows
+MERGER_SHAPES = [
+    ("merger_fc1", 5120, 5120, True),
+    ("merger_fc2", 5120, 1536, True),
+]
 
 
 def dev(a):
@@ -210,7 +216,7 @@ def test_grouped_linears_equal_separate_calls(pkg, m, k, ns):
         assert np.array_equal(host(yg), host(pkg.matmul(x, p, n)))
 
 
-@pytest.mark.parametrize("m", [1, 8])
+@pytest.mark.parametrize("m", [1, 4, 8])
 def test_gemv_lm_head(pkg, orc, m):
     name, k, n, has_bias = LM_HEAD
     y, ref = run_linear(pkg, orc, m, k, n, has_bias)
@@ -267,6 +273,16 @@ def test_gemm_large_m_on_sampled_rows(pkg, orc, name, k, n, has_bias):
     y, ref = run_linear(pkg, orc, m, k, n, has_bias, outliers=0.01, rows=rows)
     err = max_abs_rel(y, ref)
     assert err <= GEMM_TOL and err <= TIGHT, (name, err)
+
+
+@pytest.mark.parametrize("name,k,n,has_bias", MERGER_SHAPES)
+@pytest.mark.parametrize("m", [1, 256, 1024])
+def test_merger_linears_match_oracle(pkg, orc, name, k, n, has_bias, m):
+    # M = 256 is the image of the vision config (1024 patches merged four to one); 1 and 1024 bracket it
+    rows = None if m == 1 else np.unique(np.concatenate([np.arange(0, m, 29), [m - 1, 31, 32, 33]]))
+    y, ref = run_linear(pkg, orc, m, k, n, has_bias, outliers=0.0 if m == 1 else 0.01, rows=rows)
+    err = max_abs_rel(y, ref)
+    assert err <= (GEMV_TOL if m <= 8 else GEMM_TOL) and err <= TIGHT, (name, m, err)
 
 
 @pytest.mark.parametrize("m", [9, 15, 16, 17, 32, 33, 63, 65, 100, 129, 257, 300])

@@ -327,6 +327,17 @@ def test_reference_test_case_is_close_to_dense_matmul(orc):
     assert np.corrcoef(y.ravel(), dense.ravel())[0, 1] > 0.995
 
 
+def test_input_generator_is_glibc_rand_scaled_to_minus_one_one(orc):
+    # glibc's rand() after srand(1) is a published sequence (1804289383, 846930886, 1681692777, 1714636915,
+    # 1957747793, ...), and the reference's generator is (float)((double)rand() / RAND_MAX) * 2 - 1 filled
+    # row by row (tests/Arm/KaiLinearTest.hpp:154-161): a known-answer pin that does not use the oracle.
+    seq = [1804289383, 846930886, 1681692777, 1714636915, 1957747793, 424238335]
+    want = np.array([np.float32(np.float32(v / 2147483647.0) * np.float32(2.0)) - np.float32(1.0) for v in seq],
+                    dtype=np.float32)
+    got = orc.fill_uniform_random(2, 3, 1)
+    assert got.shape == (2, 3) and np.array_equal(got.ravel(), want)
+
+
 # --------------------------------------------------------------------------- an independent library routine
 
 def torch_dyn_quant_linear(x, u4, sc_bits, bias):
