@@ -154,6 +154,32 @@ typedef struct {
 } w4a32_decode_linear_args;
 int w4a32_decode_linear(const w4a32_decode_linear_args* args, void* stream);
 
+/* ---- operators of the engine's op-by-op path ------------------------------------------------
+ * What the reference's model code dispatches one by one and the decoder runner below fuses away. They exist
+ * so that a backend can offer every operator of mllm/Models/ds_qwen2/modeling_ds_qwen2_fa2_fp16.hpp:88-133
+ * (activations [B, S, H, D], RoPE layout kBSHD, KV cache layout kBSHD_NO_REPEAT). n % 4 == 0. */
+
+/* out = x / (1 + exp(-x)) (ArmSiLUOp, mllm/Backends/Arm/Ops/SiLUOp.cpp) and out = a * b (ArmMulOp,
+ * mllm/Backends/Arm/Ops/ElewiseOps.cpp). SiLU followed by Mul equals w4a32_op_silu_mul bit for bit. */
+int w4a32_op_silu(const float* d_x, float* d_out, size_t n, void* stream);
+int w4a32_op_mul(const float* d_a, const float* d_b, float* d_out, size_t n, void* stream);
+
+/* y[m][h][:] = RoPE of x[m][h][:] at position pos0 + m, rows [M][n_heads][head_dim] (normal_hf_rope_shd,
+ * mllm/Backends/Arm/Kernels/rope.cpp, layout kBSHD); tables as w4a32_op_rope_table builds them, with
+ * table_rows rows. d_y may be d_x. */
+int w4a32_op_rope(const float* d_x, float* d_y, const float* d_sin, const float* d_cos, int M, int n_heads,
+                  int head_dim, int pos0, int table_rows, void* stream);
+
+/* Causal attention with K and V laid out [n_keys][n_kv_heads][head_dim] (the kBSHD_NO_REPEAT cache at batch
+ * 1, mllm/Backends/Arm/Ops/KVCacheOp.cpp:74-88): query m at position pos0 + m sees keys 0..pos0 + m.
+ * ArmFlashAttn2Op::forward, mllm/Backends/Arm/Ops/FlashAttention2Op.cpp:221-245. head_dim must be 128. */
+int w4a32_op_attention_bshd(const float* d_q, const float* d_k, const float* d_v, float* d_out, int M,
+                            int n_heads, int n_kv_heads, int head_dim, int n_keys, int pos0, void* stream);
+
+/* C[M][N] = A[M][K] B[N][K]^T, dense f32 (MatMulOp with transpose_b, mllm/Backends/Arm/Ops/MatMulOp.cpp:131-167:
+ * how the reference applies lm_head, modeling_ds_qwen2.hpp:209-213). K % 4 == 0. M <= 8 streams B once. */
+int w4a32_op_matmul_f32_nt(const float* d_a, const float* d_b, float* d_c, int M, int N, int K, void* stream);
+
 /* ---- decoder runner -------------------------------------------------------------------- */
 
 typedef struct {

@@ -69,6 +69,11 @@ ABI = {
     "w4a32_op_rope_attention_decode": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci,
                                              _vp, _ci, _vp, _vp]),
     "w4a32_op_argmax": (_ci, [_vp, _ci, _vp, _vp, _vp, _vp]),
+    "w4a32_op_silu": (_ci, [_vp, _vp, _sz, _vp]),
+    "w4a32_op_mul": (_ci, [_vp, _vp, _vp, _sz, _vp]),
+    "w4a32_op_rope": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp]),
+    "w4a32_op_attention_bshd": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _vp]),
+    "w4a32_op_matmul_f32_nt": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a32_decode_linear": (_ci, [_vp, _vp]),
     "w4a32_decoder_state_bytes": (_sz, [_vp]),
     "w4a32_decoder_state_offset": (_sz, [_vp, _ci]),
@@ -444,6 +449,54 @@ def op_im2col_conv3d(x, kernel, stride, ld_out=None):
     out = torch.empty((rows, ld), dtype=torch.float32, device="cuda")
     _check(lib().w4a32_op_im2col_conv3d(_ptr(x), _ptr(out), B, C, T, H, W, kt, kh, kw, st, sh, sw, ld,
                                         _stream()), "w4a32_op_im2col_conv3d")
+    return out
+
+
+def op_silu(x):
+    import torch
+
+    out = torch.empty_like(x)
+    _check(lib().w4a32_op_silu(_ptr(x), _ptr(out), x.numel(), _stream()), "w4a32_op_silu")
+    return out
+
+
+def op_mul(a, b):
+    import torch
+
+    out = torch.empty_like(a)
+    _check(lib().w4a32_op_mul(_ptr(a), _ptr(b), _ptr(out), a.numel(), _stream()), "w4a32_op_mul")
+    return out
+
+
+def op_rope(x, sin, cos, n_heads, head_dim, pos0):
+    """Rows x [M][n_heads*head_dim] rotated at positions pos0.. (a new tensor)."""
+    import torch
+
+    out = torch.empty_like(x)
+    _check(lib().w4a32_op_rope(_ptr(x), _ptr(out), _ptr(sin), _ptr(cos), x.shape[0], n_heads, head_dim, pos0,
+                               sin.shape[0], _stream()), "w4a32_op_rope")
+    return out
+
+
+def op_attention_bshd(q, k, v, n_heads, n_kv_heads, head_dim, pos0):
+    """Causal attention on k, v laid out [n_keys][n_kv_heads][head_dim]; q [M][n_heads*head_dim]."""
+    import torch
+
+    M, n_keys = q.shape[0], k.shape[0]
+    out = torch.empty((M, n_heads * head_dim), dtype=torch.float32, device="cuda")
+    _check(lib().w4a32_op_attention_bshd(_ptr(q), _ptr(k), _ptr(v), _ptr(out), M, n_heads, n_kv_heads, head_dim,
+                                         n_keys, pos0, _stream()), "w4a32_op_attention_bshd")
+    return out
+
+
+def op_matmul_f32_nt(a, b):
+    """a [M][K] x b [N][K]^T, dense f32."""
+    import torch
+
+    (M, K), N = a.shape, b.shape[0]
+    out = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    _check(lib().w4a32_op_matmul_f32_nt(_ptr(a), _ptr(b), _ptr(out), M, N, K, _stream()),
+           "w4a32_op_matmul_f32_nt")
     return out
 
 

@@ -239,7 +239,8 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(const float* __re
                                                                const float* __restrict__ vc,
                                                                float* __restrict__ out, int Hq, int Hkv,
                                                                int max_seq, const int* __restrict__ d_pos0,
-                                                               int pos0, float scale) {
+                                                               int pos0, float scale, int key_stride,
+                                                               int head_stride) {
   __shared__ __align__(16) float s_q[kHeadDim];
   const int h = blockIdx.x, lane = threadIdx.x;
   const int hk = h / (Hq / Hkv);
@@ -251,15 +252,17 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(const float* __re
   s_q[lane + 64] = qv[lane + 64];
   __syncthreads();
 
-  const float* kbase = kc + (size_t)hk * max_seq * kHeadDim;
-  const float* vbase = vc + (size_t)hk * max_seq * kHeadDim;
+  // key `i` of KV head `hk` starts at hk * head_stride + i * key_stride floats: (128, max_seq * 128) for the
+  // head-major cache of the decoder runner, (Hkv * 128, 128) for a [keys][Hkv][128] cache
+  const float* kbase = kc + (size_t)hk * head_stride;
+  const float* vbase = vc + (size_t)hk * head_stride;
   float run_max = -INFINITY, run_sum = 0.0f;
   float acc0 = 0.0f, acc1 = 0.0f;  // output dims 2*lane, 2*lane + 1
 
   for (int base = 0; base < end; base += 64) {
     const int key = base + lane;
     const bool valid = key < end;
-    const float4* krow = reinterpret_cast<const float4*>(kbase + (size_t)(valid ? key : end - 1) * kHeadDim);
+    const float4* krow = reinterpret_cast<const float4*>(kbase + (size_t)(valid ? key : end - 1) * key_stride);
     float dot = 0.0f;
 #pragma unroll 8
     for (int i = 0; i < kHeadDim / 4; ++i) {
@@ -286,7 +289,7 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(const float* __re
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         const int i = i0 + u < cnt ? i0 + u : cnt - 1;
-        vv[u] = *reinterpret_cast<const float2*>(vbase + (size_t)(base + i) * kHeadDim + 2 * lane);
+        vv[u] = *reinterpret_cast<const float2*>(vbase + (size_t)(base + i) * key_stride + 2 * lane);
         const float w = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), i));
         pi[u] = i0 + u < cnt ? w : 0.0f;
       }
@@ -1006,8 +1009,18 @@ hipError_t launch_attention_prefill(const float* q, const float* kc, const float
                        s, q, kc, vc, out, M, Hq, Hkv, max_seq, d_pos0, pos0, scale, nullptr, nullptr);
   } else {
     hipLaunchKernelGGL(attention_prefill_kernel, dim3(Hq, M), dim3(64), 0, s, q, kc, vc, out, Hq, Hkv,
-                       max_seq, d_pos0, pos0, scale);
+                       max_seq, d_pos0, pos0, scale, kHeadDim, max_seq * kHeadDim);
   }
+  return hipGetLastError();
+}
+
+// The one-wavefront-per-query kernel on K / V laid out [keys][Hkv][128] (the reference's kBSHD_NO_REPEAT
+// cache at batch 1): what the engine's FlashAttn2 operator is handed.
+hipError_t launch_attention_bshd(const float* q, const float* k, const float* v, float* out, int M, int Hq,
+                                 int Hkv, int n_keys, int pos0, hipStream_t s) {
+  const float scale = 1.0f / sqrtf((float)kHeadDim);
+  hipLaunchKernelGGL(attention_prefill_kernel, dim3(Hq, M), dim3(64), 0, s, q, k, v, out, Hq, Hkv, n_keys,
+                     nullptr, pos0, scale, Hkv * kHeadDim, kHeadDim);
   return hipGetLastError();
 }
 

@@ -103,6 +103,14 @@ size_t attention_prefill_part_bytes(int M, int Hq);
 hipError_t launch_attention_prefill(const float* q, const float* kc, const float* vc, float* out,
                                     int M, int Hq, int Hkv, int max_seq, const int* d_pos0, int pos0,
                                     float* part, size_t part_bytes, unsigned int* counters, hipStream_t s);
+hipError_t launch_attention_bshd(const float* q, const float* k, const float* v, float* out, int M, int Hq,
+                                 int Hkv, int n_keys, int pos0, hipStream_t s);
+// operators of the engine's op-by-op path (w4a32_engine_ops.hip)
+hipError_t launch_silu(const float* x, float* out, size_t n, hipStream_t s);
+hipError_t launch_mul(const float* a, const float* b, float* out, size_t n, hipStream_t s);
+hipError_t launch_rope_rows(const float* x, float* y, const float* sin_t, const float* cos_t, int M, int H,
+                            int D, int pos0, hipStream_t s);
+hipError_t launch_matmul_f32_nt(const float* a, const float* b, float* c, int M, int N, int K, hipStream_t s);
 hipError_t launch_attention_decode(const float* q, float* kc, float* vc, float* out, int Hq, int Hkv,
                                    int max_seq, const int* d_pos0, int pos0, int nsplit, float* part,
                                    unsigned int* counters, const float* k_new, const float* v_new,

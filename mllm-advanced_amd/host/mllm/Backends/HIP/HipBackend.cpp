@@ -5,9 +5,11 @@
 #include <cstdlib>
 #include <cstring>
 
+#include "mllm/Backends/HIP/Ops/DecoderOps.hpp"
 #include "mllm/Backends/HIP/Ops/LinearOp.hpp"
 #include "mllm/Engine/Context.hpp"
 #include "mllm/Utils/Log.hpp"
+#include "w4a32_decoder.h"
 
 #define MLLM_CHECK_HIP(expr)                                                                         \
   do {                                                                                               \
@@ -78,7 +80,9 @@ HipBackend::HipBackend() : BackendBase(kHIP) {
   MLLM_CHECK_HIP(hipStreamCreate(&s));  // default priority
   stream_ = s;
   allocator_ = std::make_shared<HipAllocator>();
-  regOpFactory<HipLinearOpFactory, HipD2HOpFactory>();
+  regOpFactory<HipLinearOpFactory, HipD2HOpFactory, HipViewOpFactory, HipRMSNormOpFactory, HipRoPEOpFactory,
+               HipKVCacheOpFactory, HipFlashAttn2OpFactory, HipMatMulOpFactory, HipSiLUOpFactory, HipAddOpFactory,
+               HipMulOpFactory, HipLLMEmbeddingTokenOpFactory>();
 }
 
 HipBackend::~HipBackend() {
@@ -93,6 +97,23 @@ Tensor& HipBackend::scratch(size_t bytes) {
     scratch_ = Tensor::empty({static_cast<int32_t>(bytes)}, kInt8, kHIP).alloc();
   }
   return scratch_;
+}
+
+void HipBackend::ropeTables(float theta, int max_pos, int dims, Tensor* sin, Tensor* cos) {
+  for (auto& t : rope_tables_) {
+    if (t.theta == theta && t.max_pos == max_pos && t.dims == dims) {
+      *sin = t.sin;
+      *cos = t.cos;
+      return;
+    }
+  }
+  RopeTables t{theta, max_pos, dims, Tensor::empty({max_pos, dims / 2}, kFp32, kHIP).alloc(),
+               Tensor::empty({max_pos, dims / 2}, kFp32, kHIP).alloc()};
+  const int rc = w4a32_op_rope_table(t.sin.ptr<float>(), t.cos.ptr<float>(), max_pos, dims, theta, stream_);
+  if (rc != W4A32_OK) { MLLM_ERROR_EXIT(kHipRuntimeError, "w4a32_op_rope_table failed: {}", w4a32_error_string(rc)); }
+  rope_tables_.push_back(t);
+  *sin = t.sin;
+  *cos = t.cos;
 }
 
 void HipBackend::synchronize() const {

@@ -7,6 +7,7 @@
 #pragma once
 
 #include <memory>
+#include <vector>
 
 #include "mllm/Core/Tensor.hpp"
 #include "mllm/Engine/BackendBase.hpp"
@@ -71,9 +72,19 @@ class HipBackend final : public BackendBase {
   // run in order on the backend's one stream, so the next borrower cannot overlap the previous one.
   Tensor& scratch(size_t bytes);
 
+  // RoPE sin / cos tables [max_pos][dims / 2] on the device, built once per (theta, max_pos, dims) and
+  // shared by every RoPE op (the reference shares its tables through global tensors, RoPEOp.cpp:20-50).
+  void ropeTables(float theta, int max_pos, int dims, Tensor* sin, Tensor* cos);
+
  private:
+  struct RopeTables {
+    float theta;
+    int max_pos, dims;
+    Tensor sin, cos;
+  };
   void* stream_ = nullptr;
   Tensor scratch_;
+  std::vector<RopeTables> rope_tables_;
 };
 
 std::shared_ptr<HipBackend> createHipBackend();

@@ -665,3 +665,51 @@ def test_full_size_decoder_properties(pkg):
             if i % 8 == 0:
                 _ = (dec.logits * 2).sum().item()                    # unrelated eager work between replays
         assert dec.position == 512 + steps
+
+
+def test_engine_path_operators(pkg):
+    """The operators that only the engine's op-by-op path uses: SiLU then Mul equals the fused operator bit for
+    bit; RoPE on one tensor equals what the fused rope + cache-append operator does to q and k; attention on a
+    [keys][kv_heads][128] cache equals attention on the head-major cache; the dense matmul against torch."""
+    g = torch.Generator(device="cuda").manual_seed(11)
+    a = torch.randn((3, 8960), generator=g, device="cuda") * 4
+    b = torch.randn((3, 8960), generator=g, device="cuda")
+    assert torch.equal(pkg.op_mul(pkg.op_silu(a), b), pkg.op_silu_mul(a, b))
+    assert max_abs_rel(pkg.op_silu(a).cpu().numpy(), torch.nn.functional.silu(a).cpu().numpy()) < 1e-5
+    assert torch.equal(pkg.op_mul(a, b), a * b)
+
+    Hq, Hkv, D, max_seq = 12, 2, 128, 96
+    sin, cos = pkg.op_rope_table(max_seq, D, 1e6)
+    for M, pos0 in [(1, 0), (1, 37), (20, 5), (64, 32)]:
+        q = torch.randn((M, Hq * D), generator=g, device="cuda")
+        k = torch.randn((M, Hkv * D), generator=g, device="cuda")
+        v = torch.randn((M, Hkv * D), generator=g, device="cuda")
+        kc = torch.randn((Hkv, max_seq, D), generator=g, device="cuda")   # earlier positions: any values
+        vc = torch.randn((Hkv, max_seq, D), generator=g, device="cuda")
+        q_fused = q.clone()
+        pkg.op_rope_kv(q_fused, k, v, sin, cos, kc, vc, Hq, Hkv, D, pos0)
+        q_rot = pkg.op_rope(q, sin, cos, Hq, D, pos0)
+        k_rot = pkg.op_rope(k, sin, cos, Hkv, D, pos0)
+        assert torch.equal(q_rot, q_fused)
+        assert torch.equal(k_rot.view(M, Hkv, D).transpose(0, 1), kc[:, pos0:pos0 + M])
+        # the same keys and values as [keys][Hkv][D]
+        n_keys = pos0 + M
+        k_bshd = kc[:, :n_keys].transpose(0, 1).contiguous()
+        v_bshd = vc[:, :n_keys].transpose(0, 1).contiguous()
+        want = pkg.op_attention(q_rot, kc, vc, Hq, Hkv, D, pos0) if M < 16 else None
+        got = pkg.op_attention_bshd(q_rot, k_bshd, v_bshd, Hq, Hkv, D, pos0)
+        if want is not None:
+            assert torch.equal(got, want)       # the same kernel under other strides
+        qh = q_rot.view(M, Hq, D).transpose(0, 1)                       # [Hq][M][D]
+        kh = kc[:, :n_keys].repeat_interleave(Hq // Hkv, dim=0)
+        vh = vc[:, :n_keys].repeat_interleave(Hq // Hkv, dim=0)
+        mask = torch.arange(n_keys, device="cuda")[None, :] <= (pos0 + torch.arange(M, device="cuda"))[:, None]
+        ref = torch.nn.functional.scaled_dot_product_attention(qh, kh, vh, attn_mask=mask)
+        assert max_abs_rel(got.cpu().numpy(), ref.transpose(0, 1).reshape(M, Hq * D).cpu().numpy()) < 2e-5
+
+    for M, K, N in [(1, 1536, 151936), (4, 1536, 1000), (8, 96, 50), (9, 64, 70), (200, 256, 300), (64, 1536, 128)]:
+        x = torch.randn((M, K), generator=g, device="cuda")
+        w = torch.randn((N, K), generator=g, device="cuda") * 0.05
+        y = pkg.op_matmul_f32_nt(x, w)
+        ref = (x.double() @ w.double().T)
+        assert max_abs_rel(y.cpu().numpy(), ref.cpu().numpy()) < 1e-5, (M, K, N)

@@ -11,6 +11,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HOST = os.path.join(ROOT, "mllm-advanced_amd", "host")
 BIN = os.path.join(HOST, "tests", "hip_linear_test")
 BIN_MODEL = os.path.join(HOST, "tests", "hip_qwen2_test")
+BIN_OPS = os.path.join(HOST, "tests", "hip_decoder_ops_test")
 LIB = os.path.join(ROOT, "mllm-advanced_amd", "libmllm_hip_backend.so")
 
 
@@ -18,7 +19,7 @@ def test_backend_library_is_built_and_loads():
     assert os.path.exists(LIB), "run __graft_entry__.build()"
     ctypes.CDLL(os.path.join(ROOT, "mllm-advanced_amd", "libw4a32_hip.so"), mode=ctypes.RTLD_GLOBAL)
     ctypes.CDLL(LIB)
-    assert os.path.exists(BIN) and os.path.exists(BIN_MODEL)
+    assert os.path.exists(BIN) and os.path.exists(BIN_MODEL) and os.path.exists(BIN_OPS)
 
 
 def test_container_structs_have_the_on_disk_sizes():
@@ -113,3 +114,16 @@ def test_cpp_model_generates_what_the_oracle_generates(tmp_path):
         if i + 1 < len(tokens):
             logits = ref.forward([tok])
     assert max(margins) > 0.01        # the comparison was not vacuous
+
+
+@pytest.mark.gpu
+def test_cpp_decoder_operator_by_operator_matches_the_runner(tmp_path):
+    """Every decoder operator as an op class of the HIP backend (created by its factory from the reference's
+    cargo, loaded by the reference's parameter names, run through MllmEngineCtx::dispatch in the order of
+    the reference's flash-attention model variant) generates what the fused runner generates; the dense MatMul
+    operator matches a double-precision product; repeated steps take no new device allocation."""
+    out = subprocess.run([BIN_OPS, str(tmp_path)], capture_output=True, text=True, timeout=300)
+    print(out.stdout[-4000:])
+    print(out.stderr[-2000:])
+    assert out.returncode == 0 and "[ PASSED ]" in out.stdout
+    assert "TIMING:" in out.stdout and "Trying to expand KVCache" in out.stderr
