@@ -485,6 +485,133 @@ def main():
                                                    "frac": round(big_tflops / 2500.0, 4)}},
             "M512_gate_proj_kernel_TFLOPs": g512["kernel_TFLOPs"]}
 
+    # ---- config 4: the whole decoder (same Linears plus the f32 operators between them), batch 1,
+    # 512-token random-id prompt, then 256 greedy steps replayed from one captured HIP graph
+    if not args.no_decoder:
+        H, V, I = 1536, 151936, 8960
+        dgen = torch.Generator(device="cuda")
+        dgen.manual_seed(2)
+        emb = torch.randn((V, H), generator=dgen, device="cuda")
+        norm = lambda: 1 + 0.1 * torch.randn((H,), generator=dgen, device="cuda")
+        dl = []
+        for layer in layers:
+            d = {n: lin.packed for n, lin in zip(("q", "k", "v", "o", "gate", "up", "down"), layer)}
+            d["attn_norm"], d["ffn_norm"] = norm(), norm()
+            dl.append(d)
+        with torch.cuda.stream(stream):
+            dec = pkg.Decoder(H, 12, 2, I, V, dl, emb, norm(), lm_head.packed, max_seq=1024,
+                              max_batch_tokens=512, rope_theta=1e6, rms_eps=1e-6)
+            prompt = torch.randint(0, V, (512,), generator=dgen, device="cuda", dtype=torch.int64)
+            dec.prefill(prompt)                      # warm-up (allocations, code objects)
+            stream.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            dec.prefill(prompt)
+            e1.record(stream)
+            stream.synchronize()
+            prefill_ms = e0.elapsed_time(e1)
+            first = int(dec.token)
+            dec.step()                               # warm-up of the step, then rewind by prefilling again
+            dec.prefill(prompt)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                dec.step()
+            stream.synchronize()
+            n_new = 256
+            e0.record(stream)
+            for _ in range(n_new):
+                graph.replay()
+            e1.record(stream)
+            stream.synchronize()
+            decode_ms = e0.elapsed_time(e1)
+            # the timed tokens are real: the position advanced once per replay, the last step's logits are
+            # finite and its token is the first maximum of those logits
+            logits = dec.logits
+            assert dec.position == 512 + n_new
+            assert bool(torch.isfinite(logits).all()), "decoder produced non-finite logits"
+            assert int(dec.token) == int(torch.argmax(logits)), "token is not the argmax of the logits"
+            assert 0 <= first < V
+        extra["decoder_config4"] = {
+            "workload": "28 layers, hidden 1536, 12 q / 2 kv heads x 128, MLP 8960, vocab 151936, rope theta 1e6, "
+                        "f32 KV cache; batch 1, 512 random prompt ids, 256 greedy steps; all Linears W4A32 "
+                        "(lm_head included), random-init weights",
+            "prefill_ms_512_tokens": round(prefill_ms, 2),
+            "prefill_tokens_per_s": round(512 / (prefill_ms * 1e-3), 1),
+            "decode_ms_per_token": round(decode_ms / n_new, 4),
+            "decode_tokens_per_s": round(n_new / (decode_ms * 1e-3), 1),
+            "decode_weight_GBps": round(step_bytes / (decode_ms / n_new * 1e-3) / 1e9, 1),
+            "note": "one decode step = 143 launches (embedding, 28 x [add+norm+qkv, rope+cache+attention, o, "
+                    "add+norm+gate/up+silu*mul, down], add+norm+lm_head, argmax), captured once and replayed; "
+                    "positions and cache lengths are read from device memory",
+        }
+        # config 5, language side: prefill of the 256 merged vision tokens through the same decoder
+        with torch.cuda.stream(stream):
+            p256 = prompt[:256].contiguous()
+            dec.prefill(p256)
+            stream.synchronize()
+            e0.record(stream)
+            dec.prefill(p256)
+            e1.record(stream)
+            stream.synchronize()
+            lm256_ms = e0.elapsed_time(e1)
+        del dec, emb
+
+        # config 5, vision side: Qwen2-VL-2B ViT Linears at M = 1024 patch tokens (32 layers of
+        # qkv 1280->3840, proj 1280->1280, fc1 1280->5120, fc2 5120->1280), the patch embedding as
+        # im2col + Linear (K = 3*2*14*14 = 1176 padded to 1184, N = 1280) and the merger (5120->5120->1536
+        # on 256 rows)
+        vgen = torch.Generator(device="cuda")
+        vgen.manual_seed(3)
+        vit = {}
+        with torch.cuda.stream(stream):
+            def time_linear(M, K, N, reps=20):
+                w = torch.randn((N, K), generator=vgen, device="cuda") * 0.02
+                b = torch.randn((N,), generator=vgen, device="cuda") * 0.02
+                packed = pkg.quant_pack_rhs(w, b)
+                x = torch.randn((M, K), generator=vgen, device="cuda")
+                ws = torch.empty(pkg.workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
+                y = torch.empty((M, N), device="cuda")
+                for _ in range(3):
+                    pkg.matmul(x, packed, N, ws=ws, out=y)
+                e0.record(stream)
+                for _ in range(reps):
+                    pkg.matmul(x, packed, N, ws=ws, out=y)
+                e1.record(stream)
+                stream.synchronize()
+                ms = e0.elapsed_time(e1) / reps
+                return {"ms": round(ms, 4), "TFLOPs": round(2.0 * M * N * K / (ms * 1e-3) / 1e12, 1)}
+            layer_ms, layer_flop = 0.0, 0.0
+            for name, K, N in (("qkv", 1280, 3840), ("proj", 1280, 1280), ("fc1", 1280, 5120), ("fc2", 5120, 1280)):
+                vit[name] = time_linear(1024, K, N)
+                layer_ms += vit[name]["ms"]
+                layer_flop += 2.0 * 1024 * N * K
+            vit["merger_fc1"] = time_linear(256, 5120, 5120)
+            vit["merger_fc2"] = time_linear(256, 5120, 1536)
+            img = torch.randn((1, 3, 2, 448, 448), generator=vgen, device="cuda")
+            wpe = torch.zeros((1280, 1184), device="cuda")
+            wpe[:, :1176] = torch.randn((1280, 1176), generator=vgen, device="cuda") * 0.02
+            pe_packed = pkg.quant_pack_rhs(wpe)
+            for _ in range(2):
+                pkg.matmul(pkg.op_im2col_conv3d(img, (2, 14, 14), (2, 14, 14)), pe_packed, 1280)
+            e0.record(stream)
+            for _ in range(10):
+                pkg.matmul(pkg.op_im2col_conv3d(img, (2, 14, 14), (2, 14, 14)), pe_packed, 1280)
+            e1.record(stream)
+            stream.synchronize()
+            vit["patch_embed_im2col_plus_linear_ms"] = round(e0.elapsed_time(e1) / 10, 4)
+        extra["vit_config5"] = {
+            "workload": "Qwen2-VL-2B-shaped vision Linears as W4A32 GEMM, 1024 patch tokens (one 448x448 image), "
+                        "whole op (row quant + product) per Linear; python-side allocation of the im2col "
+                        "buffer is inside the patch-embed figure",
+            "per_linear_M1024": vit,
+            "vit_layer_linears_ms": round(layer_ms, 4),
+            "vit_32_layers_linears_ms": round(32 * layer_ms, 3),
+            "vit_layer_TFLOPs": round(layer_flop / (layer_ms * 1e-3) / 1e12, 1),
+            "lm_prefill_256_tokens_ms": round(lm256_ms, 3),
+        }
+
+    # ---- CPU baseline: scalar restatement of the reference path, bounded sample
+    cpu = None
     if not args.no_cpu:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import w4a32_oracle as orc
