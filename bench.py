@@ -144,6 +144,38 @@ def main():
             if rc:
                 raise pkg.W4A32Error(f"w4a32_matmul_grouped -> {rc}")
 
+    # The pass with down_proj split over K: its 96 tile rows alone occupy 96 of the 256 CUs, so each tile row's
+    # k range goes to three workgroups, which leave three partial rows; the launch that reads them (the next
+    # layer's q,k,v) adds them up while it loads its row. Same Linears, same bytes, same number of launches.
+    kparts = int(L.w4a32_decode_kparts(8960, 1536))
+    parts_buf = torch.randn((3, 1536), generator=xgen, device="cuda") * 0.5
+    parts_calls = []
+    if kparts > 1:
+        for li, layer in enumerate(layers):
+            q, k, v, o, gate, up, down = layer
+            a = pkg.DecodeLinearArgs()
+            a.d_x, a.K, a.count, a.in_parts = parts_buf.data_ptr(), 1536, 3, kparts
+            for i, (lin, yt) in enumerate(zip((q, k, v), (y_by_n[1536], y_by_n[256], y_extra[("k", 256)]))):
+                a.d_packed[i], a.N[i], a.d_y[i] = lin.packed.data_ptr(), lin.N, yt.data_ptr()
+            parts_calls.append(("decode", a))
+            parts_calls.append(("grouped", grouped_calls[4 * li + 1]))
+            parts_calls.append(("grouped", grouped_calls[4 * li + 2]))
+            d = pkg.DecodeLinearArgs()
+            d.d_x, d.K, d.count, d.out_parts = x_by_k[8960].data_ptr(), 8960, 1, kparts
+            d.d_packed[0], d.N[0], d.d_y[0] = down.packed.data_ptr(), 1536, parts_buf.data_ptr()
+            parts_calls.append(("decode", d))
+        parts_calls.append(("grouped", grouped_calls[-1]))
+
+    def parts_pass():
+        for kind, c in parts_calls:
+            if kind == "decode":
+                rc = L.w4a32_decode_linear(ctypes.byref(c), sptr)
+            else:
+                (ya, pa, na, cnt), K = c
+                rc = L.w4a32_matmul_grouped(ya, x_by_k[K].data_ptr(), pa, na, cnt, ws_by_k[K].data_ptr(), 1, K, sptr)
+            if rc:
+                raise pkg.W4A32Error(f"parts pass ({kind}) -> {rc}")
+
     def product_only_pass():
         for l in step_linears:
             rc = L.w4a32_matmul_quantized(y_by_n[l.N].data_ptr(), ws_by_k[l.K].data_ptr(),
@@ -215,7 +247,12 @@ def main():
 
     # Every call is ONE kernel (row quantisation inside): gemv_fused_kernel for the decoder
     # Linears (q,k,v in one launch, gate,up in one launch), gemv_wide_kernel for lm_head.
-    ms_step, wall_ms = timed(grouped_pass, args.steps, args.warmup, use_graph)
+    ms_unsplit, wall_unsplit = timed(grouped_pass, args.steps, args.warmup, use_graph)
+    ms_step, wall_ms, split_down = ms_unsplit, wall_unsplit, False
+    if parts_calls:
+        ms_parts, wall_parts = timed(parts_pass, args.steps, args.warmup, use_graph)
+        if ms_parts < ms_unsplit:
+            ms_step, wall_ms, split_down = ms_parts, wall_parts, True
     n_launch = len(grouped_calls)
     roof_avg_us = ms_step * 1e3 / n_launch
     roof_bytes = step_bytes / n_launch
@@ -246,6 +283,9 @@ def main():
     ms_prod, _ = timed(product_only_pass, args.steps, args.warmup, use_graph)
 
     extra = {"decode_linears_tokens_per_s": round(1e3 / ms_step, 1),
+             "down_proj_split_over_k": {"used_for_value": split_down, "parts": kparts,
+                                        "ms_per_step_unsplit": round(ms_unsplit, 4),
+                                        "ms_per_step_split": round(ms_parts, 4) if parts_calls else None},
              "wall_ms_per_step": round(wall_ms, 4), "graph": use_graph,
              "one_launch_per_linear": {"launches": len(step_linears), "ms_per_step": round(ms_single, 4),
                                        "GBps": round(step_bytes / (ms_single * 1e-3) / 1e9, 1)},
@@ -328,11 +368,19 @@ def main():
     name_bytes = {l.name: l.bytes[1] for l in layers[0]}
     with torch.cuda.stream(stream):
         for label, slot, names in kinds:
-            calls = [grouped_calls[4 * i + slot] for i in range(LAYERS)]
+            if split_down and slot in (0, 3):     # the launches the pass is made of: the split forms
+                calls = [parts_calls[4 * i + slot] for i in range(LAYERS)]
+                label += " (reads three partial rows)" if slot == 0 else " (k range in three parts)"
+            else:
+                calls = [("grouped", grouped_calls[4 * i + slot]) for i in range(LAYERS)]
 
             def kind_round(calls=calls):
-                for (ya, pa, na, cnt), K in calls:
-                    L.w4a32_matmul_grouped(ya, x_by_k[K].data_ptr(), pa, na, cnt, ws_by_k[K].data_ptr(), 1, K, sptr)
+                for kind, c in calls:
+                    if kind == "decode":
+                        L.w4a32_decode_linear(ctypes.byref(c), sptr)
+                    else:
+                        (ya, pa, na, cnt), K = c
+                        L.w4a32_matmul_grouped(ya, x_by_k[K].data_ptr(), pa, na, cnt, ws_by_k[K].data_ptr(), 1, K, sptr)
             kind_round()
             stream.synchronize()
             run = kind_round
@@ -681,7 +729,10 @@ def main():
         "config": {"workload": "config 2 at M=1: Qwen2-1.5B decode Linears, 28 layers x "
                                "{q,k,v,o,gate,up,down} + lm_head, distinct weights per layer, whole op "
                                "(row quant + product) per Linear; Linears that share an input (q,k,v; "
-                               "gate,up) are issued as one grouped call",
+                               "gate,up) are issued as one grouped call"
+                               + ("; down_proj's k range is dealt to three workgroups per tile row and its three "
+                                  "partial rows are added up by the launch that reads them (the next layer's "
+                                  "q,k,v)" if split_down else ""),
                    "M": 1, "linears": len(step_linears), "launches": n_launch,
                    "algorithmic_bytes_per_step": step_bytes},
         "roofline": roofline, "cpu_baseline": cpu,

@@ -151,8 +151,21 @@ typedef struct {
   int N[4];
   float* d_y[4];
   int silu_pair;
+  int in_parts;   /* 0 or 1: a single row. 2 or 3: the row is given in that many partial rows, K floats apart, which
+                     the launch adds up ((r0 + r1) + r2) before it does anything else - at d_delta when
+                     d_norm_weight is given (d_delta is then required), else at d_x. Not with silu_pair. */
+  int out_parts;  /* 0 or 1: d_y holds the Linears' outputs. > 1 (count == 1, no norm, no pair, in_parts <= 1;
+                     must equal w4a32_decode_kparts(K, N[0])): the Linear's k range is dealt to that many workgroups
+                     per tile row and d_y[0] receives [out_parts][N[0]] partial rows whose sum is the output (bias
+                     included), for a reader that adds them up - the next w4a32_decode_linear via in_parts. */
 } w4a32_decode_linear_args;
 int w4a32_decode_linear(const w4a32_decode_linear_args* args, void* stream);
+
+/* Parts into which w4a32_decode_linear would split a [N][K] Linear's k range: 3 for a long K with few output
+ * rows (down_proj, K = 8960, N = 1536: its 96 tile rows alone would leave 160 of 256 CUs idle), else 1 (no
+ * split). 0 on an invalid shape. No counterpart in the reference, which runs a decode Linear as one task
+ * (kai_linear.cpp:366-396). */
+int w4a32_decode_kparts(int K, int N);
 
 /* ---- operators of the engine's op-by-op path ------------------------------------------------
  * What the reference's model code dispatches one by one and the decoder runner below fuses away. They exist

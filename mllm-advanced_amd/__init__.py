@@ -75,6 +75,7 @@ ABI = {
     "w4a32_op_attention_bshd": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _vp]),
     "w4a32_op_matmul_f32_nt": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a32_decode_linear": (_ci, [_vp, _vp]),
+    "w4a32_decode_kparts": (_ci, [_ci, _ci]),
     "w4a32_decoder_state_bytes": (_sz, [_vp]),
     "w4a32_decoder_state_offset": (_sz, [_vp, _ci]),
     "w4a32_decoder_init": (_ci, [_vp, _vp, _vp]),
@@ -88,7 +89,8 @@ class DecodeLinearArgs(ctypes.Structure):
     _fields_ = [("d_x", ctypes.c_void_p), ("d_delta", ctypes.c_void_p), ("d_sum_out", ctypes.c_void_p),
                 ("d_norm_weight", ctypes.c_void_p), ("norm_eps", ctypes.c_float), ("K", ctypes.c_int),
                 ("count", ctypes.c_int), ("d_packed", ctypes.c_void_p * 4), ("N", ctypes.c_int * 4),
-                ("d_y", ctypes.c_void_p * 4), ("silu_pair", ctypes.c_int)]
+                ("d_y", ctypes.c_void_p * 4), ("silu_pair", ctypes.c_int), ("in_parts", ctypes.c_int),
+                ("out_parts", ctypes.c_int)]
 
 
 class DecoderConfig(ctypes.Structure):
@@ -558,20 +560,22 @@ def op_argmax(logits, scratch, d_pos=None):
 
 
 def decode_linear(x, packed_list, n_list, norm_weight=None, eps=1e-6, delta=None, want_sum=False,
-                  silu_pair=False):
+                  silu_pair=False, in_parts=0, out_parts=0):
     """One f32 row x [1][K] through 1..4 Linears with the decoder's fusions (see w4a32_decode_linear).
-    Returns (outputs, sum) where sum is x + delta when want_sum."""
+    Returns (outputs, sum) where sum is x + delta when want_sum. in_parts > 1: x (delta with a norm) holds
+    that many partial rows [in_parts][K]; out_parts > 1: the single output is [out_parts][N] partial rows."""
     import torch
 
     K = x.shape[-1]
     cnt = len(packed_list)
-    ys = [torch.empty((1, n), dtype=torch.float32, device="cuda") for n in n_list]
+    ys = [torch.empty((max(out_parts, 1), n), dtype=torch.float32, device="cuda") for n in n_list]
     if silu_pair:
         ys = ys[:1]
-    total = torch.empty_like(x) if want_sum else None
+    total = torch.empty((1, K), dtype=torch.float32, device="cuda") if want_sum else None
     a = DecodeLinearArgs()
     a.d_x, a.d_delta, a.d_sum_out = x.data_ptr(), _ptr(delta), _ptr(total)
     a.d_norm_weight, a.norm_eps, a.K, a.count, a.silu_pair = _ptr(norm_weight), eps, K, cnt, int(silu_pair)
+    a.in_parts, a.out_parts = in_parts, out_parts
     for i in range(cnt):
         a.d_packed[i], a.N[i] = packed_list[i].data_ptr(), n_list[i]
         a.d_y[i] = ys[i].data_ptr() if i < len(ys) else None

@@ -87,7 +87,7 @@ StateGeom state_geom(const w4a32_decoder_config* c) {
   g.k_off = take(sizeof(float) * Mb * kvd);
   g.v_off = take(sizeof(float) * Mb * kvd);
   g.attn_off = take(sizeof(float) * Mb * qd);
-  g.delta_off = take(sizeof(float) * Mb * c->hidden);
+  g.delta_off = take(sizeof(float) * std::max<size_t>(Mb, 3) * c->hidden);  // decode: down_proj's rows in up to 3 parts
   g.gate_off = take(sizeof(float) * Mb * c->intermediate);
   g.up_off = take(sizeof(float) * Mb * c->intermediate);
   g.act_off = take(sizeof(float) * Mb * c->intermediate);
@@ -266,9 +266,14 @@ int run_decode_fused(const w4a32_decoder_config* c, const w4a32_decoder_weights*
     const uint8_t* pk[1] = {static_cast<const uint8_t*>(packed)};
     float* ys[1] = {y};
     const int ns[1] = {N};
-    return from_hip(w4::launch_gemv_decode(ys, x, pk, ns, 1, K, nullptr, nullptr, nullptr, 0.0f, false, s));
+    return from_hip(w4::launch_gemv_decode(ys, x, pk, ns, 1, K, nullptr, nullptr, nullptr, 0.0f, false, 1, s));
   };
 
+  // down_proj (K = intermediate, few tile rows) runs with its k range dealt to three workgroups per tile row;
+  // its partial rows are added up by the launch that reads them, the next layer's [add+norm+q,k,v]. The last
+  // layer's feeds the lm_head launch, which takes a single row, and runs unsplit.
+  const int down_parts = w4::gemv_kparts(I, H);
+  int delta_parts = 1;
   for (int l = 0; l < c->n_layers; ++l) {
     const w4a32_layer_weights& lw = w->layers[l];
     float* kc = reinterpret_cast<float*>(st + g.kcache_off) + (size_t)l * g.cache_layer;
@@ -279,7 +284,8 @@ int run_decode_fused(const w4a32_decoder_config* c, const w4a32_decoder_weights*
       float* ys[3] = {q, k, v};
       const int ns[3] = {qd, kvd, kvd};
       W4_TRY(from_hip(w4::launch_gemv_decode(ys, hcur, pk, ns, 3, H, l == 0 ? nullptr : delta,
-                                             l == 0 ? nullptr : hnext, lw.attn_norm, c->rms_eps, false, s)));
+                                             l == 0 ? nullptr : hnext, lw.attn_norm, c->rms_eps, false,
+                                             delta_parts, s)));
       if (l != 0) std::swap(hcur, hnext);
     }
     W4_TRY(from_hip(w4::launch_attention_decode(
@@ -292,17 +298,23 @@ int run_decode_fused(const w4a32_decoder_config* c, const w4a32_decoder_weights*
       float* ys[2] = {act, nullptr};
       const int ns[2] = {I, I};
       W4_TRY(from_hip(w4::launch_gemv_decode(ys, hcur, pk, ns, 2, H, delta, hnext, lw.ffn_norm, c->rms_eps,
-                                             true, s)));
+                                             true, 1, s)));
       std::swap(hcur, hnext);
     }
-    W4_TRY(one(act, lw.down, I, H, delta));
+    if (down_parts > 1 && l + 1 < c->n_layers) {
+      W4_TRY(from_hip(w4::launch_gemv_kparts(delta, act, static_cast<const uint8_t*>(lw.down), I, H, s)));
+      delta_parts = down_parts;
+    } else {
+      W4_TRY(one(act, lw.down, I, H, delta));
+      delta_parts = 1;
+    }
   }
   {
     const uint8_t* pk[1] = {static_cast<const uint8_t*>(w->lm_head)};
     float* ys[1] = {logits};
     const int ns[1] = {c->vocab};
     W4_TRY(from_hip(w4::launch_gemv_decode(ys, hcur, pk, ns, 1, H, delta, nullptr, w->final_norm, c->rms_eps,
-                                           false, s)));
+                                           false, 1, s)));
   }
   return from_hip(w4::launch_argmax(logits, c->vocab, reinterpret_cast<float*>(scratch + sg.amax_val_off),
                                     reinterpret_cast<int*>(scratch + sg.amax_idx_off),
@@ -510,9 +522,28 @@ int w4a32_decode_linear(const w4a32_decode_linear_args* a, void* stream) {
     pk[i] = static_cast<const uint8_t*>(a->d_packed[i]);
   }
   if (reinterpret_cast<uintptr_t>(a->d_x) % 16 != 0) return W4A32_EINVAL;
+  if (a->in_parts < 0 || a->out_parts < 0) return W4A32_EINVAL;
+  if (a->out_parts > 1) {
+    // one plain Linear, its result left as partial rows
+    if (a->count != 1 || pair || a->d_norm_weight || a->in_parts > 1) return W4A32_EINVAL;
+    if (a->out_parts != w4::gemv_kparts(a->K, a->N[0])) return W4A32_ESHAPE;
+    return from_hip(w4::launch_gemv_kparts(a->d_y[0], a->d_x, pk[0], a->K, a->N[0], S(stream)));
+  }
   if (!w4::gemv_decode_applies(a->K, a->N, a->count, pair)) return W4A32_ENOTSUP;
+  if (a->in_parts > 1) {
+    if (a->in_parts > 3 || pair || (a->d_norm_weight && !a->d_delta)) return W4A32_EINVAL;
+    for (int i = 0; i < a->count; ++i) {
+      if (a->N[i] >= 32768) return W4A32_ENOTSUP;  // the one-wavefront-per-tile-row kernel takes a single row
+    }
+  }
   return from_hip(w4::launch_gemv_decode(a->d_y, a->d_x, pk, a->N, a->count, a->K, a->d_delta,
-                                         a->d_sum_out, a->d_norm_weight, a->norm_eps, pair, S(stream)));
+                                         a->d_sum_out, a->d_norm_weight, a->norm_eps, pair, a->in_parts,
+                                         S(stream)));
+}
+
+int w4a32_decode_kparts(int K, int N) {
+  if (K <= 0 || N <= 0 || K % 32 != 0) return 0;
+  return w4::gemv_kparts(K, N);
 }
 
 size_t w4a32_decoder_state_bytes(const w4a32_decoder_config* cfg) {

@@ -248,6 +248,7 @@ struct GroupArgs {
   int N[kMaxGroup];
   int first[kMaxGroup + 1];  // first[i] = tile rows of Linears 0..i-1; first[count] = grid size
   int count;
+  int in_parts;  // > 1: the input row (the delta row with a norm in front) is the sum of that many rows, K floats apart
 };
 
 // Whole op in one launch: x f32 [M][K] (row stride ldx) -> y.
@@ -351,6 +352,29 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
       }
     }
   }
+  // A producer that ran split over K (gemv_kparts_kernel) leaves its result as up to three partial rows:
+  // they are requested here with everything else and added up, ((r0 + r1) + r2), before the row is used.
+  // Grouped kernels at M = 1 only (a consumer with parts is launched through the group table).
+  constexpr bool kParts = kGrouped && M == 1;
+  const int in_parts = kParts ? ga.in_parts : 1;
+  float pv[2][kParts ? kFusedR : 1][8];
+  if (kParts && in_parts > 1) {
+    const float* base = kNorm ? pro_delta : x;
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      const float* row = base + (size_t)(p + 1 < in_parts ? p + 1 : 0) * K;  // a repeat where there is no part
+#pragma unroll
+      for (int r = 0; r < kFusedR; ++r) {
+        const int c = threadIdx.x + r * nthreads;
+        const int cc = c < groups ? c : groups - 1;
+        const float4 v0 = *reinterpret_cast<const float4*>(row + 8 * cc);
+        const float4 v1 = *reinterpret_cast<const float4*>(row + 8 * cc + 4);
+        const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pv[p][r][e] = f[e];
+      }
+    }
+  }
   u32x4 wq[kSets][kCPW];
   u32x2 sc[kSets][kCPW];
 #pragma unroll
@@ -379,6 +403,21 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
     }
   }
 
+  if (kParts && in_parts > 1) {
+#pragma unroll
+    for (int r = 0; r < kFusedR; ++r) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if constexpr (kNorm) {
+          dv[0][r][e] += pv[0][r][e];
+          if (in_parts > 2) dv[0][r][e] += pv[1][r][e];
+        } else {
+          xv[0][r][e] += pv[0][r][e];
+          if (in_parts > 2) xv[0][r][e] += pv[1][r][e];
+        }
+      }
+    }
+  }
   if (kNorm) {
     // complete the row, sum its squares, normalise: all before the quantiser sees it
 #pragma unroll
@@ -530,6 +569,120 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
   }
 }
 
+// One decode row through ONE Linear with a long K, the k range dealt to kDecodeParts workgroups per tile row
+// (down_proj: 96 tile rows would otherwise occupy 96 of 256 CUs with 14 wavefronts each). Workgroup
+// (part p, tile row nt) quantises the row as gemv_fused_kernel does (the range needs the whole row; only
+// the part's own k range is converted and kept), multiplies its chunks kc0 .. kc0 + KCp - 1 and stores
+//   part 0:  (sum/16 + off * rsum[n]) * lhs_scale + bias[n]        parts 1..:  (sum/16) * lhs_scale
+// to y[p][n]: the parts add up to the Linear's output (up to f32 rounding) and whoever reads it next adds
+// them, so no workgroup waits for another. W wavefronts hold three chunks each (KCp <= 3 W).
+constexpr int kDecodeParts = 3;
+template <int kFusedR>
+__global__ __launch_bounds__(1024) void gemv_kparts_kernel(const float* __restrict__ x, int K, int KC, int KCp,
+                                                           int W, const uint8_t* packed, int N, int NT,
+                                                           float* y) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  constexpr int kCPW = 3;
+  const int p = (int)blockIdx.x / NT, nt = (int)blockIdx.x - p * NT;
+  const int kc0 = p * KCp, kc1 = kc0 + KCp < KC ? kc0 + KCp : KC;
+  const float* rsum = reinterpret_cast<const float*>(packed + (size_t)NT * KC * kTileBytes);
+  const int nthreads = 64 * W;
+  int8_t* s_a = reinterpret_cast<int8_t*>(smem);                            // [KCp * 128]
+  float* s_red = reinterpret_cast<float*>(smem + (size_t)KCp * kTileK);      // [W][16]
+  float2* s_mm = reinterpret_cast<float2*>(s_red + W * 16);                  // [W] (min, max)
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int g = lane >> 4, j = lane & 15;
+
+  const int groups = K >> 3;
+  float xv[kFusedR][8];
+#pragma unroll
+  for (int r = 0; r < kFusedR; ++r) {
+    const int c = threadIdx.x + r * nthreads;
+    const int cc = c < groups ? c : groups - 1;
+    const float4 v0 = *reinterpret_cast<const float4*>(x + 8 * cc);
+    const float4 v1 = *reinterpret_cast<const float4*>(x + 8 * cc + 4);
+    const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) xv[r][e] = f[e];
+  }
+  const uint8_t* tiles = packed + (size_t)nt * KC * kTileBytes;
+  u32x4 wq[kCPW];
+  u32x2 sc[kCPW];
+#pragma unroll
+  for (int i = 0; i < kCPW; ++i) {
+    const int kc = kc0 + wave + i * W < kc1 ? kc0 + wave + i * W : kc1 - 1;  // masked where used
+    wq[i] = load_global<u32x4>(tiles + (size_t)kc * kTileBytes + 16 * lane);
+    sc[i] = load_global<u32x2>(tiles + (size_t)kc * kTileBytes + kTileQBytes + 8 * j);
+  }
+  float rs = 0.0f, bs = 0.0f;
+  const int n_out = kTileRows * nt + j;
+  if (p == 0 && threadIdx.x < 16 && n_out < N) {
+    rs = load_global<float>(rsum + n_out);
+    bs = load_global<float>(rsum + NT * kTileRows + n_out);
+  }
+
+  float lo = xv[0][0], hi = xv[0][0];
+#pragma unroll
+  for (int r = 0; r < kFusedR; ++r) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      lo = fminf(lo, xv[r][e]);
+      hi = fmaxf(hi, xv[r][e]);
+    }
+  }
+  wave_minmax_pair(lo, hi);
+  if (lane == 63) s_mm[wave] = make_float2(lo, hi);
+  __syncthreads();
+  float2 v = s_mm[j < W ? j : W - 1];
+  row16_minmax_pair(v.x, v.y);
+  const RowQuant par = row_quant_params(v.x, v.y);
+
+  // this part's k range into LDS (the tile padding, k >= K, is 0)
+  const int c0 = kc0 * (kTileK / 8), c1 = kc1 * (kTileK / 8);
+#pragma unroll
+  for (int r = 0; r < kFusedR; ++r) {
+    const int c = threadIdx.x + r * nthreads;
+    if (c >= c0 && c < c1) {
+      uint2 out = quant_group8(xv[r], par);
+      if (c >= groups) out = make_uint2(0, 0);
+      *reinterpret_cast<uint2*>(s_a + 8 * (c - c0)) = out;
+    }
+  }
+  // groups of the padding that no thread owns (K not a multiple of 128: at most 15 groups of the last chunk)
+  for (int c = groups + threadIdx.x; c < c1; c += nthreads) {
+    if (c >= c0) *reinterpret_cast<uint2*>(s_a + 8 * (c - c0)) = make_uint2(0, 0);
+  }
+  __syncthreads();
+
+  float acc[1] = {0.0f};
+#pragma unroll
+  for (int i = 0; i < kCPW; ++i) {
+    const bool valid = kc0 + wave + i * W < kc1;
+    const int kc = valid ? kc0 + wave + i * W : kc1 - 1;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const int8_t* a_base = s_a + kTileK * (kc - kc0) + kBlockLen * d + 8 * g;
+      const uint32_t sw = sc[i][d >> 1];
+      const uint32_t sbits = valid ? ((d & 1) ? (sw & 0xFFFF0000u) : (sw << 16)) : 0u;
+      block_products<1>(wq[i][d], __uint_as_float(sbits), a_base, 0, j, acc);
+    }
+  }
+  store_row_sums<1>(acc, s_red + wave * 16, lane);
+  __syncthreads();
+  if (threadIdx.x < 16 && n_out < N) {
+    float sum = 0.0f;
+    for (int w = 0; w < W; ++w) sum += s_red[w * 16 + threadIdx.x];
+    float out;
+    if (p == 0) {
+      out = __fmaf_rn((float)(-par.zp), rs, sum * 0.0625f);
+      out = __fmaf_rn(out, par.recip, bs);
+    } else {
+      out = (sum * 0.0625f) * par.recip;
+    }
+    *(W4_GLOBAL float*)(y + (size_t)p * N + n_out) = out;
+  }
+}
+
 static int pick_waves(int KC) { return KC < 16 ? KC : 16; }
 
 template <typename Kern>
@@ -597,7 +750,7 @@ static hipError_t launch_fused_m(const GroupArgs& ga, const float* x, int ldx, i
                      (size_t)W * M * 3 * sizeof(float);
   const dim3 grid(kPair ? ga.first[1] : ga.first[ga.count]), block(64 * W);
   static LdsLimitOnce raised1, raisedg;
-  if (ga.count == 1 || kPair) {
+  if ((ga.count == 1 && ga.in_parts <= 1) || kPair) {
     auto kern = gemv_fused_kernel<M, R, false, CPW, kNorm, kPair>;
     if (hipError_t e = raise_lds_limit(kern, lds, &raised1); e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, grid, block, lds, s, x, ldx, K, KC, W, ga.packed[0], ga.N[0], pro.delta, pro.norm_w,
@@ -969,6 +1122,36 @@ hipError_t launch_gemv_group(float* const* y, const float* x, int ldx, const uin
   return launch_fused_group(ga, x, ldx, M, K, nullptr, false, s);
 }
 
+// Parts the K-split decode kernel would leave for one row through an [N][K] Linear: kDecodeParts when K is
+// long, the tile rows are few (the unsplit launch would leave most CUs idle) and the shape fits the kernel,
+// else 1 (no split).
+int gemv_kparts(int K, int N) {
+  const int KC = (K + kTileK - 1) / kTileK, NT = (N + kTileRows - 1) / kTileRows;
+  if (KC < 48 || NT > 128 || wide_applies(K, N)) return 1;
+  const int KCp = (KC + kDecodeParts - 1) / kDecodeParts;
+  const int W = (KCp + 2) / 3;
+  if (W > kMaxWaves || (KC * (kTileK / 8) + 64 * W - 1) / (64 * W) > 3) return 1;
+  return kDecodeParts;
+}
+
+hipError_t launch_gemv_kparts(float* y_parts, const float* x, const uint8_t* packed, int K, int N,
+                              hipStream_t s) {
+  if (gemv_kparts(K, N) != kDecodeParts) return hipErrorInvalidValue;
+  const int KC = (K + kTileK - 1) / kTileK, NT = (N + kTileRows - 1) / kTileRows;
+  const int KCp = (KC + kDecodeParts - 1) / kDecodeParts;
+  const int W = (KCp + 2) / 3;
+  const int R = (KC * (kTileK / 8) + 64 * W - 1) / (64 * W);
+  const size_t lds = (size_t)KCp * kTileK + (size_t)W * 16 * sizeof(float) + (size_t)W * sizeof(float2);
+  const dim3 grid(NT * kDecodeParts), block(64 * W);
+#define W4_KPARTS(r) \
+  hipLaunchKernelGGL(gemv_kparts_kernel<r>, grid, block, lds, s, x, K, KC, KCp, W, packed, N, NT, y_parts)
+  if (R == 1) W4_KPARTS(1);
+  else if (R == 2) W4_KPARTS(2);
+  else W4_KPARTS(3);
+#undef W4_KPARTS
+  return hipGetLastError();
+}
+
 // One decode row (M = 1) through 1..4 Linears with the decoder's extras: residual add + RMSNorm in
 // front (norm_w != null), silu(y0) * y1 behind (pair: two Linears of equal N, result in y[0]).
 bool gemv_decode_applies(int K, const int* N, int count, bool pair) {
@@ -985,8 +1168,15 @@ bool gemv_decode_applies(int K, const int* N, int count, bool pair) {
 
 hipError_t launch_gemv_decode(float* const* y, const float* x, const uint8_t* const* packed,
                               const int* N, int count, int K, const float* delta, float* sum_out,
-                              const float* norm_w, float eps, bool pair, hipStream_t s) {
+                              const float* norm_w, float eps, bool pair, int in_parts, hipStream_t s) {
   const RowPrologue pro{delta, sum_out, norm_w, eps};
+  if (in_parts > 1) {
+    // partial rows are added up by the grouped kernels only: no pair, no wide layer, a delta when there is a norm
+    if (in_parts > kDecodeParts || pair || (norm_w && !delta)) return hipErrorInvalidValue;
+    for (int i = 0; i < count; ++i) {
+      if (wide_applies(K, N[i])) return hipErrorInvalidValue;
+    }
+  }
   if (count == 1 && wide_applies(K, N[0])) {
     if (norm_w) return launch_wide<1, true, true>(y[0], x, K, nullptr, packed[0], K, N[0], pro, s);
     return launch_wide<1, true, false>(y[0], x, K, nullptr, packed[0], K, N[0], pro, s);
@@ -1000,6 +1190,7 @@ hipError_t launch_gemv_decode(float* const* y, const float* x, const uint8_t* co
     ga.first[i + 1] = ga.first[i] + (N[i] + kTileRows - 1) / kTileRows;
   }
   ga.count = count;
+  ga.in_parts = in_parts > 1 ? in_parts : 1;
   return launch_fused_group(ga, x, K, 1, K, norm_w ? &pro : nullptr, pair, s);
 }
 

@@ -51,9 +51,15 @@ hipError_t launch_gemv_group(float* const* y, const float* x, int ldx, const uin
 // one decode row through 1..4 Linears, optionally with (residual add +) RMSNorm in front and
 // silu(y0) * y1 behind
 bool gemv_decode_applies(int K, const int* N, int count, bool pair);
+// in_parts > 1: the row (the delta row when there is a norm) is the sum of that many rows, K floats apart
 hipError_t launch_gemv_decode(float* const* y, const float* x, const uint8_t* const* packed,
                               const int* N, int count, int K, const float* delta, float* sum_out,
-                              const float* norm_w, float eps, bool pair, hipStream_t s);
+                              const float* norm_w, float eps, bool pair, int in_parts, hipStream_t s);
+// one decode row through one Linear with its k range dealt to gemv_kparts(K, N) workgroups per tile row, the
+// result left as that many partial rows y_parts[p][N] for the reader to add up (1: the shape is not split)
+int gemv_kparts(int K, int N);
+hipError_t launch_gemv_kparts(float* y_parts, const float* x, const uint8_t* packed, int K, int N,
+                              hipStream_t s);
 hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M, int K, int N,
                        int kernel, hipStream_t s);
 // the f16 kernel with every tile's k range dealt to several workgroups (partial sums in `part`,

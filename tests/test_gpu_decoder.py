@@ -713,3 +713,53 @@ def test_engine_path_operators(pkg):
         y = pkg.op_matmul_f32_nt(x, w)
         ref = (x.double() @ w.double().T)
         assert max_abs_rel(y.cpu().numpy(), ref.cpu().numpy()) < 1e-5, (M, K, N)
+
+
+@pytest.mark.parametrize("K,N", [(8960, 1536), (6144, 256), (8992, 1000), (12288, 2048)])
+def test_decode_linear_split_over_k_and_the_launch_that_reads_its_parts(pkg, orc, K, N):
+    """A decode Linear with a long K and few output rows leaves its result as three partial rows (its k range
+    dealt to three workgroups per tile row); the next launch adds them up while it loads its row. The parts
+    must add up to the unsplit Linear's output (f32 rounding apart) and match the oracle; a reader given the
+    parts must produce, bit for bit, what it produces from the row added up beforehand in the same order."""
+    L = pkg.lib()
+    assert L.w4a32_decode_kparts(K, N) == 3
+    assert L.w4a32_decode_kparts(1536, 1536) == 1 and L.w4a32_decode_kparts(1536, 8960) == 1
+    assert L.w4a32_decode_kparts(8960, 151936) == 1 and L.w4a32_decode_kparts(100, 16) == 0
+    rng = np.random.default_rng(K + N)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    u4, sc = orc.quant_rhs(w)
+    packed = pkg.repack_native(dev(u4), dev(sc.view(np.int16)), dev(bias), N, K)
+    (parts,), _ = pkg.decode_linear(dev(x), [packed], [N], out_parts=3)
+    assert parts.shape == (3, N)
+    total = (parts[0] + parts[1]) + parts[2]
+    whole = pkg.matmul(dev(x), packed, N)
+    ref = orc.linear(x, u4, sc, bias=bias, threads=8)
+    assert max_abs_rel(total.cpu().numpy()[None], whole.cpu().numpy()) < 1e-6
+    assert max_abs_rel(total.cpu().numpy()[None], ref) <= 2e-5
+    assert float(parts[1].abs().max()) > 0 and float(parts[2].abs().max()) > 0
+
+    if N % 32:
+        return
+    # readers: three Linears on the row that arrives in parts (K of the reader = N of the producer)
+    ns = [256, 64, 48]
+    rd = [pkg.quant_pack_rhs(dev((rng.standard_normal((n, N)) * 0.05).astype(np.float32)),
+                             dev((rng.standard_normal(n) * 0.1).astype(np.float32))) for n in ns]
+    summed = total[None].contiguous()
+    for cnt in (3, 1):
+        got, _ = pkg.decode_linear(parts, rd[:cnt], ns[:cnt], in_parts=3)
+        want, _ = pkg.decode_linear(summed, rd[:cnt], ns[:cnt])
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
+    two = (parts[0] + parts[1])[None].contiguous()
+    got, _ = pkg.decode_linear(parts, rd, ns, in_parts=2)
+    want, _ = pkg.decode_linear(two, rd, ns)
+    assert all(torch.equal(a, b) for a, b in zip(got, want))
+    # ... and with the residual add + RMSNorm in front: the parts are the delta
+    h = dev(rng.standard_normal((1, N)).astype(np.float32) * 2)
+    nw = dev((1 + 0.1 * rng.standard_normal(N)).astype(np.float32))
+    got, sum_got = pkg.decode_linear(h, rd, ns, norm_weight=nw, delta=parts, want_sum=True, in_parts=3)
+    want, sum_want = pkg.decode_linear(h, rd, ns, norm_weight=nw, delta=summed, want_sum=True)
+    assert torch.equal(sum_got, sum_want) and torch.equal(sum_got, h + summed)
+    assert all(torch.equal(a, b) for a, b in zip(got, want))
