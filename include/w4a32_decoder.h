@@ -234,7 +234,11 @@ int w4a32_decoder_prefill(const w4a32_decoder_config* cfg, const w4a32_decoder_w
 /* One greedy decode step at the state's current position (AutoLLM generate loop, AutoLLM.hpp:40-66):
  * reads *d_token_in, writes *d_token_out (may be the same address), advances the position. The launch
  * sequence does not depend on the position: capture it once, replay it per token. The caller keeps
- * the position below max_seq. */
+ * the position below max_seq: the step itself cannot refuse (the position is device memory, and a replayed
+ * graph never returns to the host). A step issued at position >= max_seq stays inside the cache - the
+ * attention treats the position as max_seq - 1 and overwrites the last row - but its token is meaningless
+ * and the counter keeps advancing; w4a32_decoder_prefill, whose pos0 is a host argument, returns W4A32_ESHAPE
+ * when pos0 + n_tokens exceeds max_seq. */
 int w4a32_decoder_step(const w4a32_decoder_config* cfg, const w4a32_decoder_weights* w, void* d_state,
                        const int64_t* d_token_in, int64_t* d_token_out, void* stream);
 

@@ -631,10 +631,17 @@ class Decoder:
         _check(lib().w4a32_decoder_prefill(ctypes.byref(self.cfg), ctypes.byref(self.weights),
                                            _ptr(self.state), _ptr(tokens), tokens.numel(), pos0,
                                            _ptr(self.token), _stream()), "w4a32_decoder_prefill")
+        self._host_pos = pos0 + tokens.numel()
         return self.token
 
     def step(self):
-        """One greedy step: consumes self.token, replaces it with the next token."""
+        """One greedy step: consumes self.token, replaces it with the next token. The position lives in device
+        memory; this object also counts the steps it issues (or records into a graph) and refuses the one that
+        would run past the cache. A caller that replays a captured step keeps count itself: past the end the
+        kernels stay inside the cache (the last row is overwritten) but the tokens are meaningless."""
+        if getattr(self, "_host_pos", 0) >= self.cfg.max_seq:
+            raise W4A32Error(f"decoder step at position {self._host_pos}: the cache holds {self.cfg.max_seq}")
+        self._host_pos = getattr(self, "_host_pos", 0) + 1
         _check(lib().w4a32_decoder_step(ctypes.byref(self.cfg), ctypes.byref(self.weights),
                                         _ptr(self.state), _ptr(self.token), _ptr(self.token), _stream()),
                "w4a32_decoder_step")

@@ -763,3 +763,21 @@ def test_decode_linear_split_over_k_and_the_launch_that_reads_its_parts(pkg, orc
     want, sum_want = pkg.decode_linear(h, rd, ns, norm_weight=nw, delta=summed, want_sum=True)
     assert torch.equal(sum_got, sum_want) and torch.equal(sum_got, h + summed)
     assert all(torch.equal(a, b) for a, b in zip(got, want))
+
+
+def test_decoder_refuses_to_run_past_its_cache(pkg):
+    # prefill checks capacity in the C ABI (its position is a host argument); the Python plumbing counts the
+    # steps it issues and refuses the one that would overwrite the last cache row
+    rng = np.random.default_rng(3)
+    H, Hq, Hkv, I, V, L = 256, 2, 1, 384, 640, 1
+    dec = to_device_model(pkg, tiny_model(rng, H, Hq, Hkv, I, V, L), Hq, Hkv, max_seq=16, max_batch_tokens=16)
+    with pytest.raises(pkg.W4A32Error):
+        dec.prefill(dev(rng.integers(0, V, size=14).astype(np.int64)), pos0=3)     # 3 + 14 > 16
+    dec.prefill(dev(rng.integers(0, V, size=14).astype(np.int64)))
+    dec.step()
+    dec.step()
+    torch.cuda.synchronize()
+    assert dec.position == 16
+    with pytest.raises(pkg.W4A32Error):
+        dec.step()
+    assert dec.position == 16
