@@ -145,7 +145,7 @@ def main():
                 raise pkg.W4A32Error(f"w4a32_matmul_grouped -> {rc}")
 
     # The pass with down_proj split over K: its 96 tile rows alone occupy 96 of the 256 CUs, so each tile row's
-    # k range goes to three workgroups, which leave three partial rows; the launch that reads them (the next
+    # k range goes to several (two) workgroups, which leave partial rows; the launch that reads them (the next
     # layer's q,k,v) adds them up while it loads its row. Same Linears, same bytes, same number of launches.
     kparts = int(L.w4a32_decode_kparts(8960, 1536))
     parts_buf = torch.randn((3, 1536), generator=xgen, device="cuda") * 0.5
@@ -370,7 +370,7 @@ def main():
         for label, slot, names in kinds:
             if split_down and slot in (0, 3):     # the launches the pass is made of: the split forms
                 calls = [parts_calls[4 * i + slot] for i in range(LAYERS)]
-                label += " (reads three partial rows)" if slot == 0 else " (k range in three parts)"
+                label += f" (reads {kparts} partial rows)" if slot == 0 else f" (k range in {kparts} parts)"
             else:
                 calls = [("grouped", grouped_calls[4 * i + slot]) for i in range(LAYERS)]
 
@@ -730,7 +730,7 @@ def main():
                                "{q,k,v,o,gate,up,down} + lm_head, distinct weights per layer, whole op "
                                "(row quant + product) per Linear; Linears that share an input (q,k,v; "
                                "gate,up) are issued as one grouped call"
-                               + ("; down_proj's k range is dealt to three workgroups per tile row and its three "
+                               + (f"; down_proj's k range is dealt to {kparts} workgroups per tile row and its "
                                   "partial rows are added up by the launch that reads them (the next layer's "
                                   "q,k,v)" if split_down else ""),
                    "M": 1, "linears": len(step_linears), "launches": n_launch,

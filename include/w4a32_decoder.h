@@ -161,7 +161,7 @@ typedef struct {
 } w4a32_decode_linear_args;
 int w4a32_decode_linear(const w4a32_decode_linear_args* args, void* stream);
 
-/* Parts into which w4a32_decode_linear would split a [N][K] Linear's k range: 3 for a long K with few output
+/* Parts into which w4a32_decode_linear would split a [N][K] Linear's k range: 2 for a long K with few output
  * rows (down_proj, K = 8960, N = 1536: its 96 tile rows alone would leave 160 of 256 CUs idle), else 1 (no
  * split). 0 on an invalid shape. No counterpart in the reference, which runs a decode Linear as one task
  * (kai_linear.cpp:366-396). */

@@ -87,7 +87,7 @@ StateGeom state_geom(const w4a32_decoder_config* c) {
   g.k_off = take(sizeof(float) * Mb * kvd);
   g.v_off = take(sizeof(float) * Mb * kvd);
   g.attn_off = take(sizeof(float) * Mb * qd);
-  g.delta_off = take(sizeof(float) * std::max<size_t>(Mb, 3) * c->hidden);  // decode: down_proj's rows in up to 3 parts
+  g.delta_off = take(sizeof(float) * std::max<size_t>(Mb, 3) * c->hidden);  // decode: down_proj's row in partial rows (at most 3)
   g.gate_off = take(sizeof(float) * Mb * c->intermediate);
   g.up_off = take(sizeof(float) * Mb * c->intermediate);
   g.act_off = take(sizeof(float) * Mb * c->intermediate);
@@ -269,7 +269,7 @@ int run_decode_fused(const w4a32_decoder_config* c, const w4a32_decoder_weights*
     return from_hip(w4::launch_gemv_decode(ys, x, pk, ns, 1, K, nullptr, nullptr, nullptr, 0.0f, false, 1, s));
   };
 
-  // down_proj (K = intermediate, few tile rows) runs with its k range dealt to three workgroups per tile row;
+  // down_proj (K = intermediate, few tile rows) runs with its k range dealt to two workgroups per tile row;
   // its partial rows are added up by the launch that reads them, the next layer's [add+norm+q,k,v]. The last
   // layer's feeds the lm_head launch, which takes a single row, and runs unsplit.
   const int down_parts = w4::gemv_kparts(I, H);

@@ -362,7 +362,8 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
     const float* base = kNorm ? pro_delta : x;
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
-      const float* row = base + (size_t)(p + 1 < in_parts ? p + 1 : 0) * K;  // a repeat where there is no part
+      if (p + 1 >= in_parts) break;  // wavefront-uniform: a part that does not exist is not requested
+      const float* row = base + (size_t)(p + 1) * K;
 #pragma unroll
       for (int r = 0; r < kFusedR; ++r) {
         const int c = threadIdx.x + r * nthreads;
@@ -576,7 +577,10 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
 //   part 0:  (sum/16 + off * rsum[n]) * lhs_scale + bias[n]        parts 1..:  (sum/16) * lhs_scale
 // to y[p][n]: the parts add up to the Linear's output (up to f32 rounding) and whoever reads it next adds
 // them, so no workgroup waits for another. W wavefronts hold three chunks each (KCp <= 3 W).
-constexpr int kDecodeParts = 3;
+// Two parts measured best for down_proj (K = 8960, N = 1536: 192 workgroups of 12 wavefronts, 4.9 us against
+// 5.2 us in three parts and 6.7 us unsplit); a reader adds up to kMaxInParts partial rows.
+constexpr int kDecodeParts = 2;
+constexpr int kMaxInParts = 3;
 template <int kFusedR>
 __global__ __launch_bounds__(1024) void gemv_kparts_kernel(const float* __restrict__ x, int K, int KC, int KCp,
                                                            int W, const uint8_t* packed, int N, int NT,
@@ -1172,7 +1176,7 @@ hipError_t launch_gemv_decode(float* const* y, const float* x, const uint8_t* co
   const RowPrologue pro{delta, sum_out, norm_w, eps};
   if (in_parts > 1) {
     // partial rows are added up by the grouped kernels only: no pair, no wide layer, a delta when there is a norm
-    if (in_parts > kDecodeParts || pair || (norm_w && !delta)) return hipErrorInvalidValue;
+    if (in_parts > kMaxInParts || pair || (norm_w && !delta)) return hipErrorInvalidValue;
     for (int i = 0; i < count; ++i) {
       if (wide_applies(K, N[i])) return hipErrorInvalidValue;
     }

@@ -717,12 +717,13 @@ def test_engine_path_operators(pkg):
 
 @pytest.mark.parametrize("K,N", [(8960, 1536), (6144, 256), (8992, 1000), (12288, 2048)])
 def test_decode_linear_split_over_k_and_the_launch_that_reads_its_parts(pkg, orc, K, N):
-    """A decode Linear with a long K and few output rows leaves its result as three partial rows (its k range
-    dealt to three workgroups per tile row); the next launch adds them up while it loads its row. The parts
-    must add up to the unsplit Linear's output (f32 rounding apart) and match the oracle; a reader given the
-    parts must produce, bit for bit, what it produces from the row added up beforehand in the same order."""
+    """A decode Linear with a long K and few output rows leaves its result as partial rows (its k range dealt
+    to several workgroups per tile row); the next launch adds them up while it loads its row. The parts must
+    add up to the unsplit Linear's output (f32 rounding apart) and match the oracle; a reader given partial
+    rows must produce, bit for bit, what it produces from the row added up beforehand in the same order."""
     L = pkg.lib()
-    assert L.w4a32_decode_kparts(K, N) == 3
+    P = L.w4a32_decode_kparts(K, N)
+    assert P == 2
     assert L.w4a32_decode_kparts(1536, 1536) == 1 and L.w4a32_decode_kparts(1536, 8960) == 1
     assert L.w4a32_decode_kparts(8960, 151936) == 1 and L.w4a32_decode_kparts(100, 16) == 0
     rng = np.random.default_rng(K + N)
@@ -731,38 +732,40 @@ def test_decode_linear_split_over_k_and_the_launch_that_reads_its_parts(pkg, orc
     x = rng.standard_normal((1, K)).astype(np.float32)
     u4, sc = orc.quant_rhs(w)
     packed = pkg.repack_native(dev(u4), dev(sc.view(np.int16)), dev(bias), N, K)
-    (parts,), _ = pkg.decode_linear(dev(x), [packed], [N], out_parts=3)
-    assert parts.shape == (3, N)
-    total = (parts[0] + parts[1]) + parts[2]
+    (parts,), _ = pkg.decode_linear(dev(x), [packed], [N], out_parts=P)
+    assert parts.shape == (P, N)
+    total = parts[0] + parts[1]
     whole = pkg.matmul(dev(x), packed, N)
     ref = orc.linear(x, u4, sc, bias=bias, threads=8)
     assert max_abs_rel(total.cpu().numpy()[None], whole.cpu().numpy()) < 1e-6
     assert max_abs_rel(total.cpu().numpy()[None], ref) <= 2e-5
-    assert float(parts[1].abs().max()) > 0 and float(parts[2].abs().max()) > 0
+    assert float(parts[1].abs().max()) > 0
+    with pytest.raises(pkg.W4A32Error):
+        pkg.decode_linear(dev(x), [packed], [N], out_parts=P + 1)        # not the library's split of this shape
 
     if N % 32:
         return
-    # readers: three Linears on the row that arrives in parts (K of the reader = N of the producer)
+    # readers: Linears on a row that arrives in two or three partial rows (K of the reader = N of the producer)
     ns = [256, 64, 48]
     rd = [pkg.quant_pack_rhs(dev((rng.standard_normal((n, N)) * 0.05).astype(np.float32)),
                              dev((rng.standard_normal(n) * 0.1).astype(np.float32))) for n in ns]
-    summed = total[None].contiguous()
-    for cnt in (3, 1):
-        got, _ = pkg.decode_linear(parts, rd[:cnt], ns[:cnt], in_parts=3)
-        want, _ = pkg.decode_linear(summed, rd[:cnt], ns[:cnt])
-        for a, b in zip(got, want):
-            assert torch.equal(a, b)
-    two = (parts[0] + parts[1])[None].contiguous()
-    got, _ = pkg.decode_linear(parts, rd, ns, in_parts=2)
-    want, _ = pkg.decode_linear(two, rd, ns)
-    assert all(torch.equal(a, b) for a, b in zip(got, want))
-    # ... and with the residual add + RMSNorm in front: the parts are the delta
+    three = torch.cat([parts, dev(rng.standard_normal((1, N)).astype(np.float32) * 0.3)]).contiguous()
     h = dev(rng.standard_normal((1, N)).astype(np.float32) * 2)
     nw = dev((1 + 0.1 * rng.standard_normal(N)).astype(np.float32))
-    got, sum_got = pkg.decode_linear(h, rd, ns, norm_weight=nw, delta=parts, want_sum=True, in_parts=3)
-    want, sum_want = pkg.decode_linear(h, rd, ns, norm_weight=nw, delta=summed, want_sum=True)
-    assert torch.equal(sum_got, sum_want) and torch.equal(sum_got, h + summed)
-    assert all(torch.equal(a, b) for a, b in zip(got, want))
+    for rows in (2, 3):
+        summed = three[0] + three[1]
+        if rows == 3:
+            summed = summed + three[2]
+        summed = summed[None].contiguous()
+        for cnt in (3, 1):
+            got, _ = pkg.decode_linear(three, rd[:cnt], ns[:cnt], in_parts=rows)
+            want, _ = pkg.decode_linear(summed, rd[:cnt], ns[:cnt])
+            assert all(torch.equal(a, b) for a, b in zip(got, want)), (rows, cnt)
+        # ... and with the residual add + RMSNorm in front: the partial rows are the delta
+        got, sum_got = pkg.decode_linear(h, rd, ns, norm_weight=nw, delta=three, want_sum=True, in_parts=rows)
+        want, sum_want = pkg.decode_linear(h, rd, ns, norm_weight=nw, delta=summed, want_sum=True)
+        assert torch.equal(sum_got, sum_want) and torch.equal(sum_got, h + summed)
+        assert all(torch.equal(a, b) for a, b in zip(got, want)), rows
 
 
 def test_decoder_refuses_to_run_past_its_cache(pkg):
