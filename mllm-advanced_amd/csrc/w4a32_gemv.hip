@@ -634,6 +634,10 @@ __global__ __launch_bounds__(1024) void gemv_kparts_kernel(const float* __restri
 #pragma unroll
     for (int e = 0; e < 8; ++e) xv[r][e] = f[e];
   }
+  // A compute unit's vector memory pipe returns loads in the order they were issued, over all its wavefronts: every
+  // wavefront puts its (small, cache-resident) row loads in before any of them queues its weight loads, or a late
+  // wavefront's row would wait behind the others' weight traffic.
+  __syncthreads();
   const uint8_t* tiles = packed + (size_t)nt * KC * kTileBytes;
   u32x4 wq[kCPW];
   u32x2 sc[kCPW];
