@@ -126,6 +126,20 @@ int w4a32_op_rope_attention_decode(const float* d_q, const float* d_k, const flo
                                    int head_dim, int max_seq, const int* d_pos0, int pos0,
                                    void* d_scratch, void* stream);
 
+/* The same decode step followed by the Linear that reads the attention output (o_proj: K = n_heads *
+ * head_dim inputs, N outputs, d_packed from w4a32_quant_pack_rhs), as the decoder's step issues the two:
+ * the attention launch leaves its key slices unmerged and the Linear merges them while it loads its input
+ * row, so no workgroup of the attention waits for another. d_y [N] receives what
+ * w4a32_op_rope_attention_decode followed by w4a32_matmul (M = 1) would, bit for bit; the attention output
+ * itself is not materialised. W4A32_ESHAPE when the Linear's shape has no such kernel (K > 3072, or an
+ * lm_head-sized N): then call the two operators.
+ * Reference: the attention block of modeling_ds_qwen2.hpp:126-153 followed by o_proj (:154). */
+int w4a32_op_rope_attention_decode_linear(const float* d_q, const float* d_k, const float* d_v,
+                                          const float* d_sin, const float* d_cos, float* d_kcache,
+                                          float* d_vcache, const void* d_packed, int N, float* d_y,
+                                          int n_heads, int n_kv_heads, int head_dim, int max_seq,
+                                          const int* d_pos0, int pos0, void* d_scratch, void* stream);
+
 /* *d_token = index of the first maximum of d_logits[0..n) (AutoLLM.hpp:70-88); when d_pos_to_advance
  * is not NULL, *d_pos_to_advance += 1 afterwards. */
 int w4a32_op_argmax(const float* d_logits, int n, void* d_scratch, int64_t* d_token,

@@ -68,6 +68,8 @@ ABI = {
                                          _vp]),
     "w4a32_op_rope_attention_decode": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci,
                                              _vp, _ci, _vp, _vp]),
+    "w4a32_op_rope_attention_decode_linear": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _vp, _ci, _ci,
+                                                    _ci, _ci, _vp, _ci, _vp, _vp]),
     "w4a32_op_argmax": (_ci, [_vp, _ci, _vp, _vp, _vp, _vp]),
     "w4a32_op_silu": (_ci, [_vp, _vp, _sz, _vp]),
     "w4a32_op_mul": (_ci, [_vp, _vp, _vp, _sz, _vp]),
@@ -548,6 +550,20 @@ def op_rope_attention_decode(q, k, v, sin, cos, kcache, vcache, n_heads, n_kv_he
                                                 _ptr(scratch), _stream()),
            "w4a32_op_rope_attention_decode")
     return out
+
+
+def op_rope_attention_decode_linear(q, k, v, sin, cos, kcache, vcache, packed, N, n_heads, n_kv_heads,
+                                    head_dim, pos0, scratch, d_pos0=None):
+    """op_rope_attention_decode followed by the Linear that reads it (o_proj), as the decoder's step issues
+    them: the attention's key slices are merged by the Linear's row load. Returns y [1][N]."""
+    import torch
+
+    y = torch.empty((1, N), dtype=torch.float32, device="cuda")
+    _check(lib().w4a32_op_rope_attention_decode_linear(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(sin), _ptr(cos), _ptr(kcache), _ptr(vcache), _ptr(packed), N, _ptr(y),
+        n_heads, n_kv_heads, head_dim, kcache.shape[1], _ptr(d_pos0), pos0, _ptr(scratch), _stream()),
+        "w4a32_op_rope_attention_decode_linear")
+    return y
 
 
 def op_argmax(logits, scratch, d_pos=None):

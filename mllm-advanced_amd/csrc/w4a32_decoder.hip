@@ -8,7 +8,10 @@
 
 namespace {
 
-constexpr int kAttnSplit = 16;    // wavefronts per head in the decode attention
+constexpr int kAttnSplit = 16;    // key slices (workgroups) per head group in the decode attention
+// ... when the slices are left to the Linear that follows: 16 measured better than 8 (0.794 ms per token against
+// 0.809 with the same 4 wavefronts, which then take two key blocks in sequence, and 0.810 with 8 wavefronts)
+constexpr int kAttnDeferSlices = 16;
 constexpr int kArgmaxBlocks = 64;
 
 inline int from_hip(hipError_t e) { return e == hipSuccess ? W4A32_OK : W4A32_ELAUNCH; }
@@ -174,7 +177,8 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
       W4_TRY(from_hip(w4::launch_attention_decode(
           q, kc, vc, attn, Hq, Hkv, c->max_seq, d_pos, 0, kAttnSplit,
           reinterpret_cast<float*>(scratch + sg.part_off),
-          reinterpret_cast<unsigned int*>(scratch + sg.counters_off), nullptr, nullptr, nullptr, nullptr, s)));
+          reinterpret_cast<unsigned int*>(scratch + sg.counters_off), nullptr, nullptr, nullptr, nullptr, false,
+          s)));
     } else {
       // the gate and up buffers are dead here: they hold the per-chunk results of long query blocks
       W4_TRY(from_hip(w4::launch_attention_prefill(q, kc, vc, attn, M, Hq, Hkv, c->max_seq, d_pos, 0, gate,
@@ -274,6 +278,9 @@ int run_decode_fused(const w4a32_decoder_config* c, const w4a32_decoder_weights*
   // layer's feeds the lm_head launch, which takes a single row, and runs unsplit.
   const int down_parts = w4::gemv_kparts(I, H);
   int delta_parts = 1;
+  // The attention's key slices are merged by o_proj while it loads its row, where its shape allows: the
+  // slices' workgroups then end without waiting for each other.
+  const bool attn_slices_to_o = w4::gemv_attn_rows_applies(qd, H, kAttnDeferSlices);
   for (int l = 0; l < c->n_layers; ++l) {
     const w4a32_layer_weights& lw = w->layers[l];
     float* kc = reinterpret_cast<float*>(st + g.kcache_off) + (size_t)l * g.cache_layer;
@@ -288,11 +295,16 @@ int run_decode_fused(const w4a32_decoder_config* c, const w4a32_decoder_weights*
                                              delta_parts, s)));
       if (l != 0) std::swap(hcur, hnext);
     }
+    float* attn_part = reinterpret_cast<float*>(scratch + sg.part_off);
     W4_TRY(from_hip(w4::launch_attention_decode(
-        q, kc, vc, attn, Hq, Hkv, c->max_seq, d_pos, 0, kAttnSplit,
-        reinterpret_cast<float*>(scratch + sg.part_off),
-        reinterpret_cast<unsigned int*>(scratch + sg.counters_off), k, v, sin_t, cos_t, s)));
-    W4_TRY(one(attn, lw.o, qd, H, delta));
+        q, kc, vc, attn, Hq, Hkv, c->max_seq, d_pos, 0, kAttnDeferSlices, attn_part,
+        reinterpret_cast<unsigned int*>(scratch + sg.counters_off), k, v, sin_t, cos_t, attn_slices_to_o, s)));
+    if (attn_slices_to_o) {
+      W4_TRY(from_hip(w4::launch_gemv_attn_rows(delta, attn_part, kAttnDeferSlices, static_cast<const uint8_t*>(lw.o),
+                                                qd, H, s)));
+    } else {
+      W4_TRY(one(attn, lw.o, qd, H, delta));
+    }
     {
       const uint8_t* pk[2] = {static_cast<const uint8_t*>(lw.gate), static_cast<const uint8_t*>(lw.up)};
       float* ys[2] = {act, nullptr};
@@ -454,7 +466,8 @@ int w4a32_op_attention(const float* d_q, const float* d_kcache, const float* d_v
     return from_hip(w4::launch_attention_decode(
         d_q, const_cast<float*>(d_kcache), const_cast<float*>(d_vcache), d_out, n_heads, n_kv_heads,
         max_seq, d_pos0, pos0, kAttnSplit, reinterpret_cast<float*>(sc + sg.part_off),
-        reinterpret_cast<unsigned int*>(sc + sg.counters_off), nullptr, nullptr, nullptr, nullptr, S(stream)));
+        reinterpret_cast<unsigned int*>(sc + sg.counters_off), nullptr, nullptr, nullptr, nullptr, false,
+        S(stream)));
   }
   return from_hip(w4::launch_attention_prefill(d_q, d_kcache, d_vcache, d_out, M, n_heads, n_kv_heads,
                                                max_seq, d_pos0, pos0, nullptr, 0, nullptr, S(stream)));
@@ -494,7 +507,29 @@ int w4a32_op_rope_attention_decode(const float* d_q, const float* d_k, const flo
   return from_hip(w4::launch_attention_decode(
       d_q, d_kcache, d_vcache, d_out, n_heads, n_kv_heads, max_seq, d_pos0, pos0, kAttnSplit,
       reinterpret_cast<float*>(sc + sg.part_off), reinterpret_cast<unsigned int*>(sc + sg.counters_off),
-      d_k, d_v, d_sin, d_cos, S(stream)));
+      d_k, d_v, d_sin, d_cos, false, S(stream)));
+}
+
+int w4a32_op_rope_attention_decode_linear(const float* d_q, const float* d_k, const float* d_v,
+                                          const float* d_sin, const float* d_cos, float* d_kcache,
+                                          float* d_vcache, const void* d_packed, int N, float* d_y,
+                                          int n_heads, int n_kv_heads, int head_dim, int max_seq,
+                                          const int* d_pos0, int pos0, void* d_scratch, void* stream) {
+  if (!d_q || !d_k || !d_v || !d_sin || !d_cos || !d_kcache || !d_vcache || !d_packed || !d_y || !d_scratch)
+    return W4A32_EINVAL;
+  if (n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0 || N <= 0) return W4A32_EINVAL;
+  if (head_dim != 128 || n_heads % n_kv_heads != 0) return W4A32_ESHAPE;
+  if (!d_pos0 && (pos0 < 0 || pos0 >= max_seq)) return W4A32_ESHAPE;
+  const int K = n_heads * head_dim;
+  if (!w4::gemv_attn_rows_applies(K, N, kAttnDeferSlices)) return W4A32_ESHAPE;
+  const ScratchGeom sg = scratch_geom(n_heads);
+  uint8_t* sc = static_cast<uint8_t*>(d_scratch);
+  float* part = reinterpret_cast<float*>(sc + sg.part_off);
+  W4_TRY(from_hip(w4::launch_attention_decode(
+      d_q, d_kcache, d_vcache, nullptr, n_heads, n_kv_heads, max_seq, d_pos0, pos0, kAttnDeferSlices, part,
+      reinterpret_cast<unsigned int*>(sc + sg.counters_off), d_k, d_v, d_sin, d_cos, true, S(stream))));
+  return from_hip(w4::launch_gemv_attn_rows(d_y, part, kAttnDeferSlices, static_cast<const uint8_t*>(d_packed), K, N,
+                                            S(stream)));
 }
 
 int w4a32_op_argmax(const float* d_logits, int n, void* d_scratch, int64_t* d_token,

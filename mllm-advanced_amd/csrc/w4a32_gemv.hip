@@ -716,6 +716,120 @@ __global__ __launch_bounds__(1024) void gemv_kparts_kernel(const float* __restri
   }
 }
 
+// One decode row through one Linear whose input is the output of the decode attention, left by
+// attention_decode_kernel<.., kDefer = true> as kS key slices per head (K = heads * 128):
+//   rows [kS][K]: sum over the slice's keys of exp(score - max_s) * v      hdr [kS][heads][2]: (max_s, sum_s)
+// behind each other. A thread owns 8 consecutive values of one head; it requests its piece of every slice and
+// the head's headers at once and merges them as the attention kernel's last workgroup would,
+//   x = (sum_s rows_s * exp(max_s - max)) / (sum_s sum_s * exp(max_s - max)),
+// then the kernel goes on as gemv_fused_kernel does for a single row (range, quantise, products, epilogue).
+// W wavefronts of three chunks each (KC <= 3 W), K <= 512 W.
+template <int kS>
+__global__ __launch_bounds__(512) void gemv_attn_rows_kernel(const float* __restrict__ part, int K, int KC, int W,
+                                                             const uint8_t* packed, int N, int NT, float* y) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  constexpr int kCPW = 3;
+  const int nt = (int)blockIdx.x;
+  const float* rsum = reinterpret_cast<const float*>(packed + (size_t)NT * KC * kTileBytes);
+  int8_t* s_a = reinterpret_cast<int8_t*>(smem);                            // [KC * 128]
+  float* s_red = reinterpret_cast<float*>(smem + (size_t)KC * kTileK);       // [W][16]
+  float2* s_mm = reinterpret_cast<float2*>(s_red + W * 16);                  // [W] (min, max)
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int g = lane >> 4, j = lane & 15;
+
+  const int groups = K >> 3, heads = K >> 7;
+  const int c = threadIdx.x;
+  const int cc = c < groups ? c : groups - 1;
+  const float* hdr = part + (size_t)kS * K + 2 * (cc >> 4);
+  float2 ml[kS];
+  float4 r0[kS], r1[kS];
+#pragma unroll
+  for (int sl = 0; sl < kS; ++sl) ml[sl] = *reinterpret_cast<const float2*>(hdr + (size_t)sl * heads * 2);
+#pragma unroll
+  for (int sl = 0; sl < kS; ++sl) {
+    r0[sl] = *reinterpret_cast<const float4*>(part + (size_t)sl * K + 8 * cc);
+    r1[sl] = *reinterpret_cast<const float4*>(part + (size_t)sl * K + 8 * cc + 4);
+  }
+  // every wavefront's row loads are queued before any weight load (the memory pipe returns in order)
+  __syncthreads();
+  const uint8_t* tiles = packed + (size_t)nt * KC * kTileBytes;
+  u32x4 wq[kCPW];
+  u32x2 sc[kCPW];
+#pragma unroll
+  for (int i = 0; i < kCPW; ++i) {
+    const int kc = wave + i * W < KC ? wave + i * W : KC - 1;  // masked where used
+    wq[i] = load_global<u32x4>(tiles + (size_t)kc * kTileBytes + 16 * lane);
+    sc[i] = load_global<u32x2>(tiles + (size_t)kc * kTileBytes + kTileQBytes + 8 * j);
+  }
+  float rs = 0.0f, bs = 0.0f;
+  const int n_out = kTileRows * nt + j;
+  if (threadIdx.x < 16 && n_out < N) {
+    rs = load_global<float>(rsum + n_out);
+    bs = load_global<float>(rsum + NT * kTileRows + n_out);
+  }
+
+  float xv[8];
+  {
+    float mm = -INFINITY;
+#pragma unroll
+    for (int sl = 0; sl < kS; ++sl) mm = fmaxf(mm, ml[sl].x);
+    float ll = 0.0f, a[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int sl = 0; sl < kS; ++sl) {
+      const float wt = ml[sl].x != -INFINITY ? __expf(ml[sl].x - mm) : 0.0f;  // a slice without keys holds zeros
+      ll += ml[sl].y * wt;
+      a[0] += r0[sl].x * wt; a[1] += r0[sl].y * wt; a[2] += r0[sl].z * wt; a[3] += r0[sl].w * wt;
+      a[4] += r1[sl].x * wt; a[5] += r1[sl].y * wt; a[6] += r1[sl].z * wt; a[7] += r1[sl].w * wt;
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) xv[e] = a[e] / ll;  // key 0 is always there: ll > 0
+  }
+
+  float lo = xv[0], hi = xv[0];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    lo = fminf(lo, xv[e]);
+    hi = fmaxf(hi, xv[e]);
+  }
+  wave_minmax_pair(lo, hi);
+  if (lane == 63) s_mm[wave] = make_float2(lo, hi);
+  __syncthreads();
+  float2 v = s_mm[j < W ? j : W - 1];
+  row16_minmax_pair(v.x, v.y);
+  const RowQuant par = row_quant_params(v.x, v.y);
+
+  const int grp_per_row = KC * (kTileK / 8);
+  if (c < grp_per_row) {
+    uint2 out = quant_group8(xv, par);
+    if (c >= groups) out = make_uint2(0, 0);  // the tile padding, k >= K
+    *reinterpret_cast<uint2*>(s_a + 8 * c) = out;
+  }
+  __syncthreads();
+
+  float acc[1] = {0.0f};
+#pragma unroll
+  for (int i = 0; i < kCPW; ++i) {
+    const bool valid = wave + i * W < KC;
+    const int kc = valid ? wave + i * W : KC - 1;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const int8_t* a_base = s_a + kTileK * kc + kBlockLen * d + 8 * g;
+      const uint32_t sw = sc[i][d >> 1];
+      const uint32_t sbits = valid ? ((d & 1) ? (sw & 0xFFFF0000u) : (sw << 16)) : 0u;
+      block_products<1>(wq[i][d], __uint_as_float(sbits), a_base, 0, j, acc);
+    }
+  }
+  store_row_sums<1>(acc, s_red + wave * 16, lane);
+  __syncthreads();
+  if (threadIdx.x < 16 && n_out < N) {
+    float sum = 0.0f;
+    for (int w = 0; w < W; ++w) sum += s_red[w * 16 + threadIdx.x];
+    float out = __fmaf_rn((float)(-par.zp), rs, sum * 0.0625f);
+    out = __fmaf_rn(out, par.recip, bs);
+    *(W4_GLOBAL float*)(y + n_out) = fminf(fmaxf(out, -3.402823466e+38f), 3.402823466e+38f);
+  }
+}
+
 static int pick_waves(int KC) { return KC < 16 ? KC : 16; }
 
 template <typename Kern>
@@ -1197,6 +1311,25 @@ bool gemv_decode_applies(int K, const int* N, int count, bool pair) {
     wide = wide || wide_applies(K, N[i]);
   }
   return !wide || (count == 1 && !pair);  // a wide layer goes alone
+}
+
+bool gemv_attn_rows_applies(int K, int N, int slices) {
+  if (K <= 0 || N <= 0 || K % kTileK != 0 || wide_applies(K, N)) return false;
+  const int KC = K / kTileK, W = (KC + 2) / 3;
+  return W <= 8 && K / 8 <= 64 * W && (slices == 8 || slices == 16);
+}
+
+hipError_t launch_gemv_attn_rows(float* y, const float* part, int slices, const uint8_t* packed, int K, int N,
+                                 hipStream_t s) {
+  if (!gemv_attn_rows_applies(K, N, slices)) return hipErrorInvalidValue;
+  const int KC = K / kTileK, NT = (N + kTileRows - 1) / kTileRows, W = (KC + 2) / 3;
+  const size_t lds = (size_t)KC * kTileK + (size_t)W * 16 * sizeof(float) + (size_t)W * sizeof(float2);
+  if (slices == 8) {
+    hipLaunchKernelGGL(gemv_attn_rows_kernel<8>, dim3(NT), dim3(64 * W), lds, s, part, K, KC, W, packed, N, NT, y);
+  } else {
+    hipLaunchKernelGGL(gemv_attn_rows_kernel<16>, dim3(NT), dim3(64 * W), lds, s, part, K, KC, W, packed, N, NT, y);
+  }
+  return hipGetLastError();
 }
 
 hipError_t launch_gemv_decode(float* const* y, const float* x, const uint8_t* const* packed,

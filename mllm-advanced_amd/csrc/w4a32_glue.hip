@@ -557,25 +557,28 @@ __global__ __launch_bounds__(64 * kPfWaves) void attention_prefill_mfma_kernel(
 constexpr int kDecWaves = 4;
 constexpr int kMaxAttnSplit = 16;  // key slices per head group, at most
 
-// v += the same register of the other 15 lanes of the row (all lanes get the row's sum). Callers
-// interleave several independent values per step so that no DPP read follows its write directly.
-#define W4_ROW_ADD(v, ctrl) asm volatile("v_add_f32_dpp %0, %0, %0 " ctrl " row_mask:0xf bank_mask:0xf" : "+v"(v))
-
+// d[g] += the same register of the other 15 lanes of the row (all lanes get the row's sum), for kGW
+// independent values at once. A DPP operand must not be read within two wait states of the VALU write
+// that produced it: the waits are part of the same asm statement as the instructions they protect (the
+// compiler is free to schedule other instructions, the producer of d included, around a statement, but
+// not into it), and with three values the other two adds of a step are the wait.
+#define W4_DPP_ADD(n, ctrl) "v_add_f32_dpp %" #n ", %" #n ", %" #n " " ctrl " row_mask:0xf bank_mask:0xf\n\t"
+#define W4_DPP_STEPS(ADDS, gap)                                                              \
+  "s_nop 1\n\t" ADDS("quad_perm:[1,0,3,2]") gap ADDS("quad_perm:[2,3,0,1]") gap ADDS("row_half_mirror") gap \
+      ADDS("row_mirror")
+#define W4_DPP_ADDS1(ctrl) W4_DPP_ADD(0, ctrl)
+#define W4_DPP_ADDS2(ctrl) W4_DPP_ADD(0, ctrl) W4_DPP_ADD(1, ctrl)
+#define W4_DPP_ADDS3(ctrl) W4_DPP_ADD(0, ctrl) W4_DPP_ADD(1, ctrl) W4_DPP_ADD(2, ctrl)
 template <int kGW>
 __device__ __forceinline__ void row16_sum(float (&d)[kGW]) {
-  asm volatile("s_nop 1");
-#pragma unroll
-  for (int g = 0; g < kGW; ++g) W4_ROW_ADD(d[g], "quad_perm:[1,0,3,2]");
-  if (kGW < 3) asm volatile("s_nop 1");
-#pragma unroll
-  for (int g = 0; g < kGW; ++g) W4_ROW_ADD(d[g], "quad_perm:[2,3,0,1]");
-  if (kGW < 3) asm volatile("s_nop 1");
-#pragma unroll
-  for (int g = 0; g < kGW; ++g) W4_ROW_ADD(d[g], "row_half_mirror");
-  if (kGW < 3) asm volatile("s_nop 1");
-#pragma unroll
-  for (int g = 0; g < kGW; ++g) W4_ROW_ADD(d[g], "row_mirror");
-  asm volatile("s_nop 1");
+  static_assert(kGW >= 1 && kGW <= 3, "one to three values");
+  if constexpr (kGW == 1) {
+    asm volatile(W4_DPP_STEPS(W4_DPP_ADDS1, "s_nop 1\n\t") : "+v"(d[0]));
+  } else if constexpr (kGW == 2) {
+    asm volatile(W4_DPP_STEPS(W4_DPP_ADDS2, "s_nop 0\n\t") : "+v"(d[0]), "+v"(d[1]));
+  } else {
+    asm volatile(W4_DPP_STEPS(W4_DPP_ADDS3, "") : "+v"(d[0]), "+v"(d[1]), "+v"(d[2]));
+  }
 }
 
 // kRope: q, k_new, v_new are the raw outputs of the q/k/v Linears for the token at position pos0.
@@ -583,7 +586,12 @@ __device__ __forceinline__ void row16_sum(float (&d)[kGW]) {
 // it and v_new in place of the (not yet written) cache row and - in the first head group of each KV
 // head - appends both to the cache. That is the RoPE + cache-append operator folded in.
 // A lane holds dims 8*dl..8*dl+7; its RoPE partner dims (d +- 64) are read with a second load.
-template <int kGW, bool kRope>
+// kDefer: the workgroups of a head group do not meet. Each leaves its key slice's share where the Linear
+// that reads the attention output (gemv_attn_rows_kernel) finds it and merges the slices while it loads
+// its input row:  part[slice][head * 128 + d] = sum of exp(score - max) * v,  then, ns * Hq * 128 floats
+// on,  [slice][head][2] = (max, sum of exp). That takes the hand-over (stores acknowledged, counter, reload)
+// out of the chain of dependent memory round trips a decode step consists of.
+template <int kGW, bool kRope, bool kDefer>
 __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
     const int* __restrict__ d_pos0, const float* __restrict__ q, const float* __restrict__ sin_t,
     const float* __restrict__ cos_t, float* __restrict__ kc, float* __restrict__ vc, int Hq, int Hkv,
@@ -766,6 +774,14 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
       ll += ls[w] * wt;
       a += as[w] * wt;
     }
+    if (kDefer) {
+      part[((size_t)blockIdx.y * Hq + h0 + g) * kHeadDim + d] = a;
+      if (d == 0) {
+        float* hdr = part + (size_t)ns * Hq * kHeadDim + ((size_t)blockIdx.y * Hq + h0 + g) * 2;
+        *reinterpret_cast<float2*>(hdr) = make_float2(mm, ll);
+      }
+      continue;
+    }
     float* mine = part + ((size_t)(h0 + g) * ns + blockIdx.y) * kPartStride;
     store_shared_across_wgs(mine + 2 + d, a);
     if (d == 0) {
@@ -773,6 +789,7 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
       store_shared_across_wgs(mine + 1, ll);
     }
   }
+  if (kDefer) return;
   stores_done();
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -1029,14 +1046,22 @@ hipError_t launch_attention_bshd(const float* q, const float* k, const float* v,
 hipError_t launch_attention_decode(const float* q, float* kc, float* vc, float* out, int Hq, int Hkv,
                                    int max_seq, const int* d_pos0, int pos0, int nsplit, float* part,
                                    unsigned int* counters, const float* k_new, const float* v_new,
-                                   const float* sin_t, const float* cos_t, hipStream_t s) {
+                                   const float* sin_t, const float* cos_t, bool defer, hipStream_t s) {
   const float scale = 1.0f / sqrtf((float)kHeadDim);
   const int G = Hq / Hkv;  // query heads per KV head; a workgroup takes 2 or 3 of them when it divides
   if (nsplit > kMaxAttnSplit) return hipErrorInvalidValue;
-#define W4_ATTN(gw, rope)                                                                              \
-  hipLaunchKernelGGL((attention_decode_kernel<gw, rope>), dim3(Hq / gw, nsplit), dim3(64 * kDecWaves), \
-                     0, s, d_pos0, q, sin_t, cos_t, kc, vc, Hq, Hkv, max_seq, pos0, nsplit, scale,     \
+#define W4_ATTN_D(gw, rope, df)                                                                            \
+  hipLaunchKernelGGL((attention_decode_kernel<gw, rope, df>), dim3(Hq / gw, nsplit), dim3(64 * kDecWaves), \
+                     0, s, d_pos0, q, sin_t, cos_t, kc, vc, Hq, Hkv, max_seq, pos0, nsplit, scale,         \
                      k_new, v_new, out, part, counters)
+#define W4_ATTN(gw, rope) W4_ATTN_D(gw, rope, false)
+  if (defer) {  // the slices are left for the Linear that follows: the folded RoPE form only
+    if (!k_new) return hipErrorInvalidValue;
+    if (G % 2 == 0) W4_ATTN_D(2, true, true);
+    else if (G % 3 == 0) W4_ATTN_D(3, true, true);
+    else W4_ATTN_D(1, true, true);
+    return hipGetLastError();
+  }
   if (G % 2 == 0) {
     if (k_new) W4_ATTN(2, true); else W4_ATTN(2, false);
   } else if (G % 3 == 0) {
@@ -1045,6 +1070,7 @@ hipError_t launch_attention_decode(const float* q, float* kc, float* vc, float* 
     if (k_new) W4_ATTN(1, true); else W4_ATTN(1, false);
   }
 #undef W4_ATTN
+#undef W4_ATTN_D
   return hipGetLastError();
 }
 

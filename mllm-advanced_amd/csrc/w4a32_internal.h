@@ -120,7 +120,12 @@ hipError_t launch_matmul_f32_nt(const float* a, const float* b, float* c, int M,
 hipError_t launch_attention_decode(const float* q, float* kc, float* vc, float* out, int Hq, int Hkv,
                                    int max_seq, const int* d_pos0, int pos0, int nsplit, float* part,
                                    unsigned int* counters, const float* k_new, const float* v_new,
-                                   const float* sin_t, const float* cos_t, hipStream_t s);
+                                   const float* sin_t, const float* cos_t, bool defer, hipStream_t s);
+// one decode row through one Linear whose input row is still in key slices, as the decode attention leaves it
+// with defer = true (`part`: the same pointer, `slices`: its nsplit)
+bool gemv_attn_rows_applies(int K, int N, int slices);
+hipError_t launch_gemv_attn_rows(float* y, const float* part, int slices, const uint8_t* packed, int K, int N,
+                                 hipStream_t s);
 hipError_t launch_argmax(const float* logits, int n, float* part_val, int* part_idx,
                          unsigned int* counter, int64_t* token_out, int* pos_to_advance, int blocks,
                          hipStream_t s);

@@ -224,6 +224,45 @@ def test_rope_attention_decode_equals_the_two_operators(pkg, Hq, Hkv):
         assert torch.equal(kc2, kc1) and torch.equal(vc2, vc1), pos
 
 
+@pytest.mark.parametrize("Hq,Hkv,N,bias", [(12, 2, 1536, False), (4, 4, 272, True), (3, 1, 40, True),
+                                            (24, 4, 3072, False)])
+def test_attention_slices_merged_by_the_linear_that_reads_them(pkg, Hq, Hkv, N, bias):
+    """Decode attention that leaves its key slices unmerged + the Linear whose row load merges them
+    == the attention operator followed by the Linear, bit for bit, and the same cache rows."""
+    g = torch.Generator(device="cuda").manual_seed(16)
+    D, S = 128, 1024
+    sin, cos = pkg.op_rope_table(S, D, 1e6)
+    scratch = pkg.op_scratch(Hq)
+    w = torch.randn((N, Hq * D), generator=g, device="cuda") * 0.05
+    b = torch.randn((N,), generator=g, device="cuda") if bias else None
+    packed = pkg.quant_pack_rhs(w, b)
+    for pos in [0, 3, 15, 16, 17, 100, 255, 640, 1023]:
+        kc = torch.randn((Hkv, S, D), generator=g, device="cuda")
+        vc = torch.randn((Hkv, S, D), generator=g, device="cuda")
+        kc[:, pos + 1:] = float("nan")       # rows past the position are never part of the result
+        vc[:, pos + 1:] = float("nan")
+        q = torch.randn((1, Hq * D), generator=g, device="cuda")
+        k = torch.randn((1, Hkv * D), generator=g, device="cuda")
+        v = torch.randn((1, Hkv * D), generator=g, device="cuda")
+        kc1, vc1 = kc.clone(), vc.clone()
+        attn = pkg.op_rope_attention_decode(q, k, v, sin, cos, kc1, vc1, Hq, Hkv, D, pos, scratch)
+        want = pkg.matmul(attn, packed, N)
+        kc2, vc2 = kc.clone(), vc.clone()
+        d_pos = torch.tensor([pos], dtype=torch.int32, device="cuda")
+        got = pkg.op_rope_attention_decode_linear(q, k, v, sin, cos, kc2, vc2, packed, N, Hq, Hkv, D, 0, scratch,
+                                                  d_pos0=d_pos)
+        assert torch.isfinite(got).all(), pos
+        assert torch.equal(got, want), (pos, float((got - want).abs().max()))
+        assert torch.equal(kc2[:, :pos + 1], kc1[:, :pos + 1]) and torch.equal(vc2[:, :pos + 1], vc1[:, :pos + 1]), pos
+    # a Linear too long for the merging kernel is refused, not mis-computed
+    wide = pkg.quant_pack_rhs(torch.randn((32, 28 * D), generator=g, device="cuda"), None)
+    kc = torch.zeros((4, S, D), device="cuda")
+    with pytest.raises(Exception):
+        pkg.op_rope_attention_decode_linear(torch.zeros((1, 28 * D), device="cuda"), torch.zeros((1, 4 * D), device="cuda"),
+                                            torch.zeros((1, 4 * D), device="cuda"), sin, cos, kc, kc.clone(), wide, 32,
+                                            28, 4, D, 0, pkg.op_scratch(28))
+
+
 def test_argmax_first_maximum(pkg):
     g = torch.Generator(device="cuda").manual_seed(3)
     scratch = pkg.op_scratch(12)
