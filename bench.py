@@ -31,7 +31,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the decode pass, measured with hardware counters (not re-measured by a
 # bench run: the counters need the profiler); algorithmic bytes per launch are 7,732,011.
-PASS_TRAFFIC_BYTES_PER_LAUNCH = 7_993_476
+PASS_TRAFFIC_BYTES_PER_LAUNCH = 8_004_915
 LAYERS = 28
 # name, K, N, bias, count per layer
 LAYER_LINEARS = [
@@ -62,6 +62,9 @@ def parse():
     ap.add_argument("--roofline-only", action="store_true",
                     help="only the decode passes (the run profiled under rocprofv3 --kernel-trace)")
     ap.add_argument("--no-decoder", action="store_true", help="skip the whole-decoder tokens/s leg")
+    ap.add_argument("--pass", dest="which_pass", choices=("auto", "split", "unsplit"), default="auto",
+                    help="decode pass to time: down_proj split over K, unsplit, or both and the faster one "
+                         "(auto); a profiled run names one so that its trace holds a single pass shape")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="a 256 MiB copy, then the decode kernel on gate_proj and lm_head and the "
                          "prefill kernel on gate_proj and down_proj (the run profiled under rocprofv3 --pmc)")
@@ -247,11 +250,13 @@ def main():
 
     # Every call is ONE kernel (row quantisation inside): gemv_fused_kernel for the decoder
     # Linears (q,k,v in one launch, gate,up in one launch), gemv_wide_kernel for lm_head.
-    ms_unsplit, wall_unsplit = timed(grouped_pass, args.steps, args.warmup, use_graph)
-    ms_step, wall_ms, split_down = ms_unsplit, wall_unsplit, False
-    if parts_calls:
+    ms_unsplit = ms_parts = None
+    if args.which_pass != "split" or not parts_calls:
+        ms_unsplit, wall_unsplit = timed(grouped_pass, args.steps, args.warmup, use_graph)
+        ms_step, wall_ms, split_down = ms_unsplit, wall_unsplit, False
+    if parts_calls and args.which_pass != "unsplit":
         ms_parts, wall_parts = timed(parts_pass, args.steps, args.warmup, use_graph)
-        if ms_parts < ms_unsplit:
+        if ms_unsplit is None or ms_parts < ms_unsplit:
             ms_step, wall_ms, split_down = ms_parts, wall_parts, True
     n_launch = len(grouped_calls)
     roof_avg_us = ms_step * 1e3 / n_launch
@@ -260,10 +265,11 @@ def main():
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": PASS_TRAFFIC_BYTES_PER_LAUNCH,
                 "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over this pass's 113 launches "
-                                  "(3889.3 / 27.6 KiB per dispatch), scaled x2.00 / x1.00 by the same counters' "
+                                  "(3894.1 / 29.1 KiB per dispatch), scaled x2.00 / x1.00 by the same counters' "
                                   "reading for a 256 MiB copy; profiles/traffic_fetch_write_decode_prefill.md",
-                "kernel": "gemv_fused_kernel<1,R> (R=1 for K=1536, R=2 for K=8960); lm_head runs "
-                          "gemv_wide_kernel<1,true>",
+                "kernel": "gemv_fused_kernel<1,1> for K=1536 (q,k,v grouped; o; gate,up grouped), "
+                          "gemv_kparts_kernel<2> for down_proj (K=8960 in two k-parts; gemv_fused_kernel<1,2> "
+                          "when the unsplit pass is the faster one), gemv_wide_kernel<1,true> for lm_head",
                 "launches_per_step": n_launch, "avg_launch_us": round(roof_avg_us, 3),
                 "algorithmic_bytes_per_launch": int(roof_bytes),
                 "note": "average over the step's 113 launches (28 x {qkv, o, gate+up, down} + lm_head), "
@@ -284,8 +290,8 @@ def main():
 
     extra = {"decode_linears_tokens_per_s": round(1e3 / ms_step, 1),
              "down_proj_split_over_k": {"used_for_value": split_down, "parts": kparts,
-                                        "ms_per_step_unsplit": round(ms_unsplit, 4),
-                                        "ms_per_step_split": round(ms_parts, 4) if parts_calls else None},
+                                        "ms_per_step_unsplit": None if ms_unsplit is None else round(ms_unsplit, 4),
+                                        "ms_per_step_split": None if ms_parts is None else round(ms_parts, 4)},
              "wall_ms_per_step": round(wall_ms, 4), "graph": use_graph,
              "one_launch_per_linear": {"launches": len(step_linears), "ms_per_step": round(ms_single, 4),
                                        "GBps": round(step_bytes / (ms_single * 1e-3) / 1e9, 1)},
