@@ -133,9 +133,10 @@ int w4a32_matmul_quantized(float* d_y, const void* d_ws, const void* d_packed, i
 /* The f16 kernel with one named tile shape, W4A32_KERNEL_GEMM_F16_TILE0 + i:
  * i = 0: 64 x 64, 1: 128 x 64, 2: 128 x 128, 3: 256 x 128 (rows x columns per workgroup),
  * 4: 128 x 64 with one barrier per two stages, 5: 128 x 160, 6: 128 x 128 with eight wavefronts (each
- * 32-k half of a stage has its own four). */
+ * 32-k half of a stage has its own four), 7: 256 x 96, 8: 256 x 96 with one barrier per two stages,
+ * 9: 256 x 128 with one barrier per two stages. */
 #define W4A32_KERNEL_GEMM_F16_TILE0 16
-#define W4A32_GEMM_F16_TILES 7
+#define W4A32_GEMM_F16_TILES 10
 int w4a32_matmul_quantized_ex(float* d_y, const void* d_ws, const void* d_packed, int M, int K,
                               int N, int kernel, void* stream);
 

@@ -19,7 +19,7 @@ GEMV_MAX_M = 8
 BF16_TRUNC = 0
 BF16_RNE = 1
 KERNEL_AUTO, KERNEL_GEMV, KERNEL_GEMM_I8, KERNEL_GEMM_F16 = 0, 1, 2, 3
-KERNEL_GEMM_F16_TILE0, GEMM_F16_TILES = 16, 7   # + i: the f16 kernel with tile shape i
+KERNEL_GEMM_F16_TILE0, GEMM_F16_TILES = 16, 10  # + i: the f16 kernel with tile shape i
 
 #: every symbol include/w4a32_hip.h declares, with (restype, argtypes)
 _vp, _ci, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t

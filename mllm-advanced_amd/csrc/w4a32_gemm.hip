@@ -198,7 +198,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
   static_assert(BE == 1 || (BE == 2 && D == 2), "two stages per barrier are built for a ring of two");
   constexpr int U = BE == 2 ? 4 : (D < 2 ? 2 : D);
   static_assert(U % (2 * BE) == 0, "the unrolled stages must cover whole pairs of LDS buffer sets");
-  static_assert(WK == 1 || (WK == 2 && WM == 1), "k-halves: built for one 32-row block per wavefront");
+  static_assert(WK == 1 || WK == 2, "one or two sets of wavefronts per stage");
   constexpr int NWAVES = WAVES_M * WAVES_N * WK;
   constexpr int BM = 32 * WM * WAVES_M;
   constexpr int BN32 = WN * WAVES_N;           // 32-column fragments per workgroup and k-slice
@@ -615,7 +615,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
     float* xmine = reinterpret_cast<float*>(sB) + wave * 1024 + 4 * lane;
     const float* xpeer = reinterpret_cast<const float*>(sB) + (wave ^ (NWAVES / 2)) * 1024 + 4 * lane;
 #pragma unroll
-    for (int r = 0; r < BH; ++r) {
+    for (int ra = 0; ra < BH * WM; ++ra) {
+      const int r = ra / WM, a = ra % WM;
       const int give0 = BH + r < WN ? BH + r : WN - 1;  // block the first half hands over in this round
       __syncthreads();  // the loop's (then the previous round's) reads of these bytes are over
       if (wk == 0) {
@@ -623,30 +624,30 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
 #pragma unroll
           for (int q = 0; q < 4; ++q)
             *reinterpret_cast<float4*>(xmine + 256 * q) = make_float4(
-                acc[0][give0][4 * q], acc[0][give0][4 * q + 1], acc[0][give0][4 * q + 2], acc[0][give0][4 * q + 3]);
+                acc[a][give0][4 * q], acc[a][give0][4 * q + 1], acc[a][give0][4 * q + 2], acc[a][give0][4 * q + 3]);
         }
       } else {
 #pragma unroll
         for (int q = 0; q < 4; ++q)
           *reinterpret_cast<float4*>(xmine + 256 * q) =
-              make_float4(acc[0][r][4 * q], acc[0][r][4 * q + 1], acc[0][r][4 * q + 2], acc[0][r][4 * q + 3]);
+              make_float4(acc[a][r][4 * q], acc[a][r][4 * q + 1], acc[a][r][4 * q + 2], acc[a][r][4 * q + 3]);
       }
       __syncthreads();
       if (wk == 0) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const float4 o = *reinterpret_cast<const float4*>(xpeer + 256 * q);
-          acc[0][r][4 * q] += o.x; acc[0][r][4 * q + 1] += o.y;
-          acc[0][r][4 * q + 2] += o.z; acc[0][r][4 * q + 3] += o.w;
+          acc[a][r][4 * q] += o.x; acc[a][r][4 * q + 1] += o.y;
+          acc[a][r][4 * q + 2] += o.z; acc[a][r][4 * q + 3] += o.w;
         }
       } else if (BH + r < WN) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const float4 o = *reinterpret_cast<const float4*>(xpeer + 256 * q);
-          acc[0][give0][4 * q] = o.x + acc[0][give0][4 * q];
-          acc[0][give0][4 * q + 1] = o.y + acc[0][give0][4 * q + 1];
-          acc[0][give0][4 * q + 2] = o.z + acc[0][give0][4 * q + 2];
-          acc[0][give0][4 * q + 3] = o.w + acc[0][give0][4 * q + 3];
+          acc[a][give0][4 * q] = o.x + acc[a][give0][4 * q];
+          acc[a][give0][4 * q + 1] = o.y + acc[a][give0][4 * q + 1];
+          acc[a][give0][4 * q + 2] = o.z + acc[a][give0][4 * q + 2];
+          acc[a][give0][4 * q + 3] = o.w + acc[a][give0][4 * q + 3];
         }
       }
     }
@@ -881,6 +882,15 @@ static hipError_t launch_gemm_i8(float* y, const uint8_t* ws, const uint8_t* pac
 //   6: 128 x 128, 8 wavefronts: 4 of 32 x 128 for each 32-k half of a stage (two wavefronts per SIMD from
 //      a single workgroup); for 129..256 tiles, where every workgroup has a CU to itself (7-19 % over
 //      shape 2). The same arrangement on the 128 x 160 tile measured 1-3 % behind shape 5.
+//   7: 256 x  96, 4 wavefronts of 64 x 96, two workgroups per CU: for problems whose 256 x 128 tiles come to
+//      a little more than one full round of the 512 resident workgroups (gate_proj at M = 2048: 560 tiles of
+//      256 x 128 leave 48 for a second round, 752 of these cost three quarters each: 62.8 -> 57.7 us)
+//   8: 256 x  96 with one barrier per two stages, one workgroup per CU: for 161..256 of these tiles, each
+//      alone on its CU (gate_proj at M = 512: 188 tiles, 24.1 -> 22.2 us; o_proj and down_proj at M = 3072:
+//      23.4 -> 21.4 and 96.9 -> 83.1 us; ViT fc1 and the merger at M = 1024: 20.5 -> 19.3, 62.5 -> 55.6 us).
+//      With two wavefronts per SIMD from the same workgroup (k-halves) it measured the same.
+//   9: 256 x 128 with one barrier per two stages: shape 3 for up to one tile per CU (3-6 % over shape 3 there:
+//      gate_proj at M = 640: 26.8 -> 25.5 us; behind it as soon as two workgroups share a CU)
 static hipError_t launch_f16_tile(int tile, float* y, const uint8_t* ws, const uint8_t* packed, int M,
                                   int K, int N, const GemmGroup* group, const int* group_N, int count,
                                   int ksplit, float* part, hipStream_t s) {
@@ -899,20 +909,31 @@ static hipError_t launch_f16_tile(int tile, float* y, const uint8_t* ws, const u
       return launch_f16<4, 1, 1, 5, 2, 2>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
     case 6:
       return launch_f16<4, 1, 1, 4, 2, 2, 1, 2>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
+    case 7:
+      return launch_f16<4, 1, 2, 3, 1, 2>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
+    case 8:
+      return launch_f16<4, 1, 2, 3, 2, 1, 2>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
+    case 9:
+      return launch_f16<4, 1, 2, 4, 2, 1, 2>(y, ws, packed, M, K, N, group, group_N, count, ksplit, part, s);
   }
   return hipErrorInvalidValue;
 }
 
-// tiles: 128 x 128 tiles of the problem; tiles160: 128 x 160 tiles; tiles256: 256 x 128 tiles.
-static int choose_f16_tile(long tiles, long tiles160, long tiles256, int K) {
+// tiles: 128 x 128 tiles of the problem; tiles160: 128 x 160 tiles; tiles256: 256 x 128 tiles; tiles96: 256 x 96.
+static int choose_f16_tile(long tiles, long tiles160, long tiles256, long tiles96, int K) {
   if (tiles <= 128) return 4;
   if (tiles <= 256) return 6;
+  // 256 x 96 tiles, one per CU on most CUs
+  if (tiles96 > 160 && tiles96 <= 256) return 8;
   // 128 x 160 tiles, two workgroups per CU: when they come to one or two per CU with few CUs left over
   const long slots = 256 * ((tiles160 + 255) / 256);
   if (tiles160 <= 512 && tiles160 * 100 >= slots * 85) return 5;
   // 256 x 128 tiles, two workgroups per CU: from three quarters of a full round on, for up to one per CU,
   // and on a long K
-  if (tiles256 >= 384 || (tiles256 >= 160 && tiles256 <= 256) || (K >= 4096 && tiles >= 320)) return 3;
+  if (tiles256 >= 160 && tiles256 <= 256) return 9;
+  // a second round of 256 x 128 tiles that would be nearly empty: the same rows in narrower tiles
+  if (tiles256 > 512 && tiles256 <= 640 && tiles96 <= 768) return 7;
+  if (tiles256 >= 384 || (K >= 4096 && tiles >= 320)) return 3;
   return 2;
 }
 
@@ -937,14 +958,15 @@ hipError_t launch_gemm(float* y, const uint8_t* ws, const uint8_t* packed, int M
   const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
   const long tiles160 = (long)((M + 127) / 128) * ((N + 159) / 160);
   const long tiles256 = (long)((M + 255) / 256) * ((N + 127) / 128);
-  return launch_f16_tile(choose_f16_tile(tiles, tiles160, tiles256, K), y, ws, packed, M, K, N, nullptr, nullptr, 0,
-                         1, nullptr, s);
+  const long tiles96 = (long)((M + 255) / 256) * ((N + 95) / 96);
+  return launch_f16_tile(choose_f16_tile(tiles, tiles160, tiles256, tiles96, K), y, ws, packed, M, K, N, nullptr,
+                         nullptr, 0, 1, nullptr, s);
 }
 
 hipError_t launch_gemm_group(float* const* y, const uint8_t* ws, const uint8_t* const* packed,
                              const int* N, int count, int M, int K, hipStream_t s) {
   GemmGroup g{};
-  long tiles = 0, tiles160 = 0, tiles256 = 0;
+  long tiles = 0, tiles160 = 0, tiles256 = 0, tiles96 = 0;
   for (int i = 0; i < count; ++i) {
     g.y[i] = y[i];
     g.packed[i] = packed[i];
@@ -952,9 +974,10 @@ hipError_t launch_gemm_group(float* const* y, const uint8_t* ws, const uint8_t* 
     tiles += (long)((M + 127) / 128) * ((N[i] + 127) / 128);
     tiles160 += (long)((M + 127) / 128) * ((N[i] + 159) / 160);
     tiles256 += (long)((M + 255) / 256) * ((N[i] + 127) / 128);
+    tiles96 += (long)((M + 255) / 256) * ((N[i] + 95) / 96);
   }
-  return launch_f16_tile(choose_f16_tile(tiles, tiles160, tiles256, K), nullptr, ws, nullptr, M, K, 0, &g, N, count, 1,
-                         nullptr, s);
+  return launch_f16_tile(choose_f16_tile(tiles, tiles160, tiles256, tiles96, K), nullptr, ws, nullptr, M, K, 0, &g, N,
+                         count, 1, nullptr, s);
 }
 
 // The MLP's gate and up Linears with silu(gate) * up as the only output. Tile shape as for the two Linears

@@ -291,7 +291,7 @@ def test_gemm_ragged_m(pkg, orc, m):
     assert max_abs_rel(y, ref) <= TIGHT
 
 
-@pytest.mark.parametrize("kernel", ["i8", "f16"] + [f"f16:{i}" for i in range(7)])
+@pytest.mark.parametrize("kernel", ["i8", "f16"] + [f"f16:{i}" for i in range(10)])
 @pytest.mark.parametrize("m,k,n", [(9, 32, 16), (40, 96, 50), (200, 160, 330), (128, 1536, 256),
                                    (300, 1280, 3840), (512, 8960, 1536), (1024, 5120, 1280),
                                    # a last 64-k stage that is half empty, behind whole and behind
