@@ -990,6 +990,11 @@ hipError_t launch_gemm_pair(float* act, const uint8_t* ws, const uint8_t* gate, 
   if (tiles256 >= 384 || (K >= 4096 && tiles >= 320)) {  // 256 x 128, as for a single Linear
     return launch_f16_pair<4, 4, 1, 2, 2>(act, ws, gate, up, M, K, N, s);
   }
+  // 128 x (96 + 96), loads one stage ahead, two workgroups per CU: up to about a round and a half of them it
+  // beats the 128 x (64 + 64) shape (N = 8960 at M = 256 / 512 / 1024: 27.2 -> 23.7, 40.6 -> 38.3, 66.3 -> 62.4 us;
+  // at M = 2048 it is behind, 122 -> 140 us)
+  const long tiles192 = (long)((M + 127) / 128) * ((N + 95) / 96);
+  if (tiles192 <= 768) return launch_f16_pair<4, 6, 1, 2>(act, ws, gate, up, M, K, N, s);
   return launch_f16_pair<4, 4, 2, 3>(act, ws, gate, up, M, K, N, s);
 }
 
