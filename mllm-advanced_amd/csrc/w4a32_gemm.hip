@@ -137,6 +137,15 @@ __device__ __forceinline__ uint4 dequant8(uint32_t w, h2 s, h2 s16) {
 
 constexpr int kF16BK = 64;    // k per stage (two scale blocks, half of a weight tile chunk)
 
+// Timing-only builds (make leaveout LEAVE_OUT=<mask>, read by mllm-advanced_amd/gemm_leave_out.py): the
+// steady-state loop without its barriers (1), without the weights' dequantisation and LDS writes (2), without
+// the packed weights' global loads (4), without the activation loads (8). The results are wrong; what such a
+// build shows is how much of a stage's time waits for that part.
+#ifndef W4A32_GEMM_LEAVE_OUT
+#define W4A32_GEMM_LEAVE_OUT 0
+#endif
+constexpr int kLeaveOut = W4A32_GEMM_LEAVE_OUT;
+
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 // v_mfma_f32_32x32x16_f16 (8 passes of 4 clocks; measured on MI355X: twice the rate of the
@@ -475,7 +484,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
             *reinterpret_cast<const h8*>(base + ((f / WN) * BN32 + wn * WN + f % WN) * 1024);
       };
       if (u % BE == 0) {
-        __syncthreads();
+        if (!((kLeaveOut & 1) && FORM == kSteady)) __syncthreads();
 #pragma unroll
         for (int f = 0; f < LA; ++f) fetch(f, bbuf);
         __builtin_amdgcn_sched_barrier(0);  // requested first: their latency covers what follows
@@ -499,9 +508,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
           dx[2 * q + 1] = breg[slot][q].y;
         }
       }
-      const bool dequantise = FORM != kLast || u + BE < U;  // (after unrolling: a constant)
+      const bool dequantise =  // (after unrolling: a constant)
+          (FORM != kLast || u + BE < U) && !((kLeaveOut & 2) && FORM == kSteady);
       if constexpr (FORM == kSteady) {
-        load_b_rel(u + BE + D, breg[slot], sreg[slot]);
+        if (!(kLeaveOut & 4)) load_b_rel(u + BE + D, breg[slot], sreg[slot]);
       } else {
         if (FORM != kLast || u + BE + D < U) load_b(s + BE + D, breg[slot], sreg[slot]);
       }
@@ -562,7 +572,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
           if constexpr (TAIL) {
             if (FORM != kLast || u + D < U) load_a_kb(s + D, sl >> 1, areg[slot]);
           } else {
-            load_a_kb_next(sl >> 1, areg[slot]);
+            if (!(kLeaveOut & 8)) load_a_kb_next(sl >> 1, areg[slot]);
           }
         }
       }
