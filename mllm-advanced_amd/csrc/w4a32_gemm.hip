@@ -139,8 +139,9 @@ constexpr int kF16BK = 64;    // k per stage (two scale blocks, half of a weight
 
 // Timing-only builds (make leaveout LEAVE_OUT=<mask>, read by mllm-advanced_amd/gemm_leave_out.py): the
 // steady-state loop without its barriers (1), without the weights' dequantisation and LDS writes (2), without
-// the packed weights' global loads (4), without the activation loads (8). The results are wrong; what such a
-// build shows is how much of a stage's time waits for that part.
+// the packed weights' global loads (4), without the activation loads (8), without the LDS reads of the weight
+// fragments (16), without the products (32). The results are wrong; what such a build shows is how much of a
+// stage's time waits for that part.
 #ifndef W4A32_GEMM_LEAVE_OUT
 #define W4A32_GEMM_LEAVE_OUT 0
 #endif
@@ -480,6 +481,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
       constexpr int LA = 2;
       static_assert(LA <= 2 * WN && LA < F, "a fragment would overwrite one that is still to be used");
       auto fetch = [&](int f, const uint8_t* base) {
+        if ((kLeaveOut & 16) && FORM == kSteady) return;
         bf[(f / WN) & 1][f % WN] =
             *reinterpret_cast<const h8*>(base + ((f / WN) * BN32 + wn * WN + f % WN) * 1024);
       };
@@ -549,9 +551,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
         for (int b = 0; b < WN; ++b) {
 #pragma unroll
           for (int a = 0; a < WM; ++a) {
-            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                __builtin_bit_cast(h8, areg[slot][sl >> 1][a][sl & 1]), bf[sl & 1][b], acc[a][b], 0,
-                0, 0);
+            if (!((kLeaveOut & 32) && FORM == kSteady)) {
+              acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                  __builtin_bit_cast(h8, areg[slot][sl >> 1][a][sl & 1]), bf[sl & 1][b], acc[a][b], 0, 0, 0);
+            }
             if (a == 0) {
               const int f = sl * WN + b + LA;
               if (f < F) {

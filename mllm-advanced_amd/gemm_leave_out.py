@@ -2,7 +2,8 @@
 M = 2048 on a library whose loop lacks one of its parts.
 
     make -C mllm-advanced_amd/csrc leaveout LEAVE_OUT=<mask>      # 1 barriers, 2 dequantisation + LDS writes,
-    python3 mllm-advanced_amd/gemm_leave_out.py <mask>            # 4 packed-weight loads, 8 activation loads
+    python3 mllm-advanced_amd/gemm_leave_out.py <mask>            # 4 packed-weight loads, 8 activation loads,
+                                                                  # 16 LDS fragment reads, 32 products (masks add)
 
 With mask 0 (or none) the product library is timed. A build with a part left out computes wrong results: the
 figures say how much of the launch waits for that part, nothing else. Run every mask in a process of its own
