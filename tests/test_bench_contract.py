@@ -31,3 +31,20 @@ def test_flags_and_algorithmic_bytes():
     finally:
         sys.argv = argv
     assert args.gpus == 1 and args.steps > 0 and args.warmup >= 0
+
+
+def test_traffic_constant_is_the_one_the_counter_profile_derives():
+    """roofline.traffic is typed into bench.py (a bench run cannot carry hardware counters): it must be the
+    figure the committed counter summary arrives at, so that a kernel change that re-measures the one without
+    updating the other is caught here."""
+    sys.path.insert(0, ROOT)
+    import bench
+    import re
+
+    text = open(os.path.join(ROOT, "profiles", "traffic_fetch_write_decode_prefill.md")).read()
+    m = re.search(r"Traffic per launch = ([\d,]+) \+ ([\d,]+) = ([\d,]+) bytes", text)
+    assert m, "the profile no longer states the traffic per launch"
+    fetch, write, total = (int(x.replace(",", "")) for x in m.groups())
+    assert fetch + write == total == bench.PASS_TRAFFIC_BYTES_PER_LAUNCH
+    # and the profiled command times the pass the bench line's value comes from
+    assert "--roofline-only --pass split" in text
