@@ -167,7 +167,8 @@ typedef struct {
   int silu_pair;
   int in_parts;   /* 0 or 1: a single row. 2 or 3: the row is given in that many partial rows, K floats apart, which
                      the launch adds up ((r0 + r1) + r2) before it does anything else - at d_delta when
-                     d_norm_weight is given (d_delta is then required), else at d_x. Not with silu_pair. */
+                     d_norm_weight is given (d_delta is then required), else at d_x. Not with silu_pair; for an
+                     lm_head-sized Linear (N >= 32768) only as a single Linear with a norm (W4A32_ENOTSUP else). */
   int out_parts;  /* 0 or 1: d_y holds the Linears' outputs. > 1 (count == 1, no norm, no pair, in_parts <= 1;
                      must equal w4a32_decode_kparts(K, N[0])): the Linear's k range is dealt to that many workgroups
                      per tile row and d_y[0] receives [out_parts][N[0]] partial rows whose sum is the output (bias

@@ -247,14 +247,14 @@ bool decode_fusable(const w4a32_decoder_config* c) {
 }
 
 int run_decode_fused(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, uint8_t* st,
-                     const StateGeom& g, int64_t* d_token_out, void* stream) {
+                     const StateGeom& g, const int64_t* d_token_in, int64_t* d_token_out, void* stream) {
   hipStream_t s = S(stream);
   const int H = c->hidden, I = c->intermediate, D = c->head_dim;
   const int Hq = c->n_heads, Hkv = c->n_kv_heads, qd = Hq * D, kvd = Hkv * D;
   int* d_pos = reinterpret_cast<int*>(st + g.pos_off);
   uint8_t* scratch = st + g.scratch_off;
   const ScratchGeom sg = scratch_geom(Hq);
-  float* hcur = reinterpret_cast<float*>(st + g.h_off);    // the embedding was written here
+  float* hcur = reinterpret_cast<float*>(st + g.h_off);    // the first launch copies the token's embedding here
   float* hnext = reinterpret_cast<float*>(st + g.xn_off);
   float* q = reinterpret_cast<float*>(st + g.q_off);
   float* k = reinterpret_cast<float*>(st + g.k_off);
@@ -274,8 +274,8 @@ int run_decode_fused(const w4a32_decoder_config* c, const w4a32_decoder_weights*
   };
 
   // down_proj (K = intermediate, few tile rows) runs with its k range dealt to two workgroups per tile row;
-  // its partial rows are added up by the launch that reads them, the next layer's [add+norm+q,k,v]. The last
-  // layer's feeds the lm_head launch, which takes a single row, and runs unsplit.
+  // its partial rows are added up by the launch that reads them: the next layer's [add+norm+q,k,v], after the
+  // last layer [add+norm+lm_head].
   const int down_parts = w4::gemv_kparts(I, H);
   int delta_parts = 1;
   // The attention's key slices are merged by o_proj while it loads its row, where its shape allows: the
@@ -290,10 +290,16 @@ int run_decode_fused(const w4a32_decoder_config* c, const w4a32_decoder_weights*
                               static_cast<const uint8_t*>(lw.v)};
       float* ys[3] = {q, k, v};
       const int ns[3] = {qd, kvd, kvd};
-      W4_TRY(from_hip(w4::launch_gemv_decode(ys, hcur, pk, ns, 3, H, l == 0 ? nullptr : delta,
-                                             l == 0 ? nullptr : hnext, lw.attn_norm, c->rms_eps, false,
-                                             delta_parts, s)));
-      if (l != 0) std::swap(hcur, hnext);
+      if (l == 0) {
+        // the token's row of the embedding table is gathered by this launch (and copied to hcur, where the
+        // residual stream starts), not by a launch of its own
+        W4_TRY(from_hip(w4::launch_gemv_decode(ys, w->embedding, pk, ns, 3, H, nullptr, hcur, lw.attn_norm,
+                                               c->rms_eps, false, 1, s, d_token_in, c->vocab)));
+      } else {
+        W4_TRY(from_hip(w4::launch_gemv_decode(ys, hcur, pk, ns, 3, H, delta, hnext, lw.attn_norm, c->rms_eps,
+                                               false, delta_parts, s)));
+        std::swap(hcur, hnext);
+      }
     }
     float* attn_part = reinterpret_cast<float*>(scratch + sg.part_off);
     W4_TRY(from_hip(w4::launch_attention_decode(
@@ -313,7 +319,7 @@ int run_decode_fused(const w4a32_decoder_config* c, const w4a32_decoder_weights*
                                              true, 1, s)));
       std::swap(hcur, hnext);
     }
-    if (down_parts > 1 && l + 1 < c->n_layers) {
+    if (down_parts > 1) {
       W4_TRY(from_hip(w4::launch_gemv_kparts(delta, act, static_cast<const uint8_t*>(lw.down), I, H, s)));
       delta_parts = down_parts;
     } else {
@@ -326,7 +332,7 @@ int run_decode_fused(const w4a32_decoder_config* c, const w4a32_decoder_weights*
     float* ys[1] = {logits};
     const int ns[1] = {c->vocab};
     W4_TRY(from_hip(w4::launch_gemv_decode(ys, hcur, pk, ns, 1, H, delta, nullptr, w->final_norm, c->rms_eps,
-                                           false, 1, s)));
+                                           false, delta_parts, s)));
   }
   return from_hip(w4::launch_argmax(logits, c->vocab, reinterpret_cast<float*>(scratch + sg.amax_val_off),
                                     reinterpret_cast<int*>(scratch + sg.amax_idx_off),
@@ -568,7 +574,8 @@ int w4a32_decode_linear(const w4a32_decode_linear_args* a, void* stream) {
   if (a->in_parts > 1) {
     if (a->in_parts > 3 || pair || (a->d_norm_weight && !a->d_delta)) return W4A32_EINVAL;
     for (int i = 0; i < a->count; ++i) {
-      if (a->N[i] >= 32768) return W4A32_ENOTSUP;  // the one-wavefront-per-tile-row kernel takes a single row
+      // the one-wavefront-per-tile-row kernel adds partial rows only in front of a norm, for a single Linear
+      if (a->N[i] >= 32768 && !(a->count == 1 && a->d_norm_weight)) return W4A32_ENOTSUP;
     }
   }
   return from_hip(w4::launch_gemv_decode(a->d_y, a->d_x, pk, a->N, a->count, a->K, a->d_delta,
@@ -634,9 +641,9 @@ int w4a32_decoder_step(const w4a32_decoder_config* cfg, const w4a32_decoder_weig
   if (!config_ok(cfg) || !w || !w->layers || !d_state || !d_token_in || !d_token_out) return W4A32_EINVAL;
   const StateGeom g = state_geom(cfg);
   uint8_t* st = static_cast<uint8_t*>(d_state);
+  if (decode_fusable(cfg)) return run_decode_fused(cfg, w, st, g, d_token_in, d_token_out, stream);
   W4_TRY(from_hip(w4::launch_embedding(d_token_in, w->embedding, 1, cfg->hidden, cfg->vocab,
                                        reinterpret_cast<float*>(st + g.h_off), S(stream))));
-  if (decode_fusable(cfg)) return run_decode_fused(cfg, w, st, g, d_token_out, stream);
   return run_layers(cfg, w, st, g, 1, d_token_out, true, stream);
 }
 

@@ -259,6 +259,7 @@ struct RowPrologue {
   float* sum_out;       // optional: receives x + delta (must not alias x)
   const float* norm_w;  // RMSNorm weight [K]
   float eps;
+  int delta_parts;      // gemv_wide_kernel: delta is the sum of that many rows, K floats apart (0 or 1: one row)
 };
 struct GroupArgs {
   const uint8_t* packed[kMaxGroup];
@@ -342,10 +343,26 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
   // run while the weights are on their way from HBM.
   const int groups = K >> 3;
   W4_TRACE(0, 0.0f);  // the workgroup has started
+  // kNorm at M = 1 with ldx < 0 (a row stride has no use at M = 1): x is a table of -ldx rows of K floats, the
+  // delta argument points to an int64 row number instead, and the input row is that row of the table (the number
+  // clamped to it); workgroup 0 copies the row to sum_out. The decoder's first launch of a token reads the
+  // token's embedding this way instead of behind a gather launch. Both arguments arrive preloaded, so a launch
+  // that gathers nothing does not wait for anything new.
+  const float* xin = x;
+  bool gathered = false;
+  if constexpr (kNorm && M == 1) {
+    if (ldx < 0) {
+      long id = load_global<int64_t>(pro_delta);
+      id = id < 0 ? 0 : (id >= -ldx ? -ldx - 1 : id);
+      xin = x + (size_t)id * K;
+      pro_delta = nullptr;
+      gathered = true;
+    }
+  }
   float xv[M][kFusedR][8];
 #pragma unroll
   for (int m = 0; m < M; ++m) {
-    const float* row = x + (size_t)m * ldx;
+    const float* row = xin + (size_t)m * ldx;
 #pragma unroll
     for (int r = 0; r < kFusedR; ++r) {
       const int c = threadIdx.x + r * nthreads;
@@ -457,6 +474,10 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
             *reinterpret_cast<float4*>(dst) = make_float4(xv[m][r][0], xv[m][r][1], xv[m][r][2], xv[m][r][3]);
             *reinterpret_cast<float4*>(dst + 4) = make_float4(xv[m][r][4], xv[m][r][5], xv[m][r][6], xv[m][r][7]);
           }
+        } else if (gathered && pro_sum_out && blockIdx.x == 0 && c < groups) {
+          float* dst = pro_sum_out + 8 * c;  // the row itself: the residual stream starts with it
+          *reinterpret_cast<float4*>(dst) = make_float4(xv[m][r][0], xv[m][r][1], xv[m][r][2], xv[m][r][3]);
+          *reinterpret_cast<float4*>(dst + 4) = make_float4(xv[m][r][4], xv[m][r][5], xv[m][r][6], xv[m][r][7]);
         }
         if (c < groups) {
 #pragma unroll
@@ -981,7 +1002,14 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
           const float* dsrc = pro.delta + (size_t)m * ldx + 8 * c;
           const float4 d0 = *reinterpret_cast<const float4*>(dsrc);
           const float4 d1 = *reinterpret_cast<const float4*>(dsrc + 4);
-          const float dd[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
+          float dd[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
+          // a producer that ran split over K left partial rows: ((r0 + r1) + r2), as gemv_fused_kernel adds them
+          for (int p = 1; p < pro.delta_parts; ++p) {
+            const float4 e0 = *reinterpret_cast<const float4*>(dsrc + (size_t)p * K);
+            const float4 e1 = *reinterpret_cast<const float4*>(dsrc + (size_t)p * K + 4);
+            dd[0] += e0.x; dd[1] += e0.y; dd[2] += e0.z; dd[3] += e0.w;
+            dd[4] += e1.x; dd[5] += e1.y; dd[6] += e1.z; dd[7] += e1.w;
+          }
 #pragma unroll
           for (int e = 0; e < 8; ++e) f[e] += dd[e];
           if (pro.sum_out && blockIdx.x == 0 && (int)threadIdx.x < groups) {
@@ -1348,13 +1376,24 @@ hipError_t launch_gemv_attn_rows(float* y, const float* part, int slices, const 
 
 hipError_t launch_gemv_decode(float* const* y, const float* x, const uint8_t* const* packed,
                               const int* N, int count, int K, const float* delta, float* sum_out,
-                              const float* norm_w, float eps, bool pair, int in_parts, hipStream_t s) {
-  const RowPrologue pro{delta, sum_out, norm_w, eps};
-  if (in_parts > 1) {
-    // partial rows are added up by the grouped kernels only: no pair, no wide layer, a delta when there is a norm
-    if (in_parts > kMaxInParts || pair || (norm_w && !delta)) return hipErrorInvalidValue;
+                              const float* norm_w, float eps, bool pair, int in_parts, hipStream_t s,
+                              const int64_t* x_row, int x_rows) {
+  RowPrologue pro{delta, sum_out, norm_w, eps, in_parts};
+  int ldx = K;
+  if (x_row) {  // a gathered row: through the norm prologue of the tile-row kernels only, no delta, no pair
+    if (!norm_w || delta || x_rows <= 0 || pair || in_parts > 1) return hipErrorInvalidValue;
     for (int i = 0; i < count; ++i) {
       if (wide_applies(K, N[i])) return hipErrorInvalidValue;
+    }
+    pro.delta = reinterpret_cast<const float*>(x_row);  // see gemv_fused_kernel: the row number, flagged by ldx < 0
+    ldx = -x_rows;
+  }
+  if (in_parts > 1) {
+    // partial rows are added up by the grouped kernels and, in front of a norm, by the wide kernel: no pair, a
+    // delta when there is a norm
+    if (in_parts > kMaxInParts || pair || (norm_w && !delta)) return hipErrorInvalidValue;
+    for (int i = 0; i < count; ++i) {
+      if (wide_applies(K, N[i]) && !(count == 1 && norm_w)) return hipErrorInvalidValue;
     }
   }
   if (count == 1 && wide_applies(K, N[0])) {
@@ -1371,7 +1410,7 @@ hipError_t launch_gemv_decode(float* const* y, const float* x, const uint8_t* co
   }
   ga.count = count;
   ga.in_parts = in_parts > 1 ? in_parts : 1;
-  return launch_fused_group(ga, x, K, 1, K, norm_w ? &pro : nullptr, pair, s);
+  return launch_fused_group(ga, x, ldx, 1, K, norm_w ? &pro : nullptr, pair, s);
 }
 
 }  // namespace w4

@@ -54,7 +54,8 @@ bool gemv_decode_applies(int K, const int* N, int count, bool pair);
 // in_parts > 1: the row (the delta row when there is a norm) is the sum of that many rows, K floats apart
 hipError_t launch_gemv_decode(float* const* y, const float* x, const uint8_t* const* packed,
                               const int* N, int count, int K, const float* delta, float* sum_out,
-                              const float* norm_w, float eps, bool pair, int in_parts, hipStream_t s);
+                              const float* norm_w, float eps, bool pair, int in_parts, hipStream_t s,
+                              const int64_t* x_row = nullptr, int x_rows = 0);
 // one decode row through one Linear with its k range dealt to gemv_kparts(K, N) workgroups per tile row, the
 // result left as that many partial rows y_parts[p][N] for the reader to add up (1: the shape is not split)
 int gemv_kparts(int K, int N);

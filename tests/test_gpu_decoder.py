@@ -805,6 +805,19 @@ def test_decode_linear_split_over_k_and_the_launch_that_reads_its_parts(pkg, orc
         want, sum_want = pkg.decode_linear(h, rd, ns, norm_weight=nw, delta=summed, want_sum=True)
         assert torch.equal(sum_got, sum_want) and torch.equal(sum_got, h + summed)
         assert all(torch.equal(a, b) for a, b in zip(got, want)), rows
+    # ... and an lm_head-sized reader (one wavefront per tile row): partial rows only as the delta in front of a norm
+    nv = 32768 + 48
+    wide = pkg.quant_pack_rhs(dev((rng.standard_normal((nv, N)) * 0.05).astype(np.float32)), None)
+    for rows in (2, 3):
+        summed = three[0] + three[1]
+        if rows == 3:
+            summed = summed + three[2]
+        summed = summed[None].contiguous()
+        (got,), _ = pkg.decode_linear(h, [wide], [nv], norm_weight=nw, delta=three, in_parts=rows)
+        (want,), _ = pkg.decode_linear(h, [wide], [nv], norm_weight=nw, delta=summed)
+        assert torch.equal(got, want), rows
+    with pytest.raises(pkg.W4A32Error):
+        pkg.decode_linear(three, [wide], [nv], in_parts=2)               # no norm: that kernel takes one row
 
 
 def test_decoder_refuses_to_run_past_its_cache(pkg):
