@@ -13,6 +13,7 @@ constexpr int kAttnSplit = 16;    // key slices (workgroups) per head group in t
 // 0.809 with the same 4 wavefronts, which then take two key blocks in sequence, and 0.810 with 8 wavefronts)
 constexpr int kAttnDeferSlices = 16;
 constexpr int kArgmaxBlocks = 64;
+constexpr int kArgmaxParts = 4096;  // partial results an lm_head launch can leave (one per wavefront)
 
 inline int from_hip(hipError_t e) { return e == hipSuccess ? W4A32_OK : W4A32_ELAUNCH; }
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -22,8 +23,8 @@ inline hipStream_t S(void* stream) { return static_cast<hipStream_t>(stream); }
 struct ScratchGeom {
   size_t counters_off;  // u32 [n_heads + 1]
   size_t part_off;      // f32 [n_heads][kAttnSplit][130]
-  size_t amax_val_off;  // f32 [kArgmaxBlocks]
-  size_t amax_idx_off;  // i32 [kArgmaxBlocks]
+  size_t amax_val_off;  // f32 [kArgmaxParts]
+  size_t amax_idx_off;  // i32 [kArgmaxParts]
   size_t total;
 };
 
@@ -35,9 +36,9 @@ ScratchGeom scratch_geom(int n_heads) {
   g.part_off = o;
   o = align_up(o + sizeof(float) * (size_t)n_heads * kAttnSplit * 130, 256);
   g.amax_val_off = o;
-  o = align_up(o + sizeof(float) * kArgmaxBlocks, 256);
+  o = align_up(o + sizeof(float) * kArgmaxParts, 256);
   g.amax_idx_off = o;
-  o = align_up(o + sizeof(int) * kArgmaxBlocks, 256);
+  o = align_up(o + sizeof(int) * kArgmaxParts, 256);
   g.total = o;
   return g;
 }
@@ -331,6 +332,16 @@ int run_decode_fused(const w4a32_decoder_config* c, const w4a32_decoder_weights*
     const uint8_t* pk[1] = {static_cast<const uint8_t*>(w->lm_head)};
     float* ys[1] = {logits};
     const int ns[1] = {c->vocab};
+    // an lm_head-sized launch leaves the first maximum of every wavefront's outputs beside the logits: the
+    // greedy choice then reads a few thousand pairs instead of the whole row
+    const int parts = w4::gemv_wide_applies(H, c->vocab) ? w4::wide_partials(c->vocab) : 0;
+    float* amax_val = reinterpret_cast<float*>(scratch + sg.amax_val_off);
+    int* amax_idx = reinterpret_cast<int*>(scratch + sg.amax_idx_off);
+    if (parts > 0 && parts <= kArgmaxParts) {
+      W4_TRY(from_hip(w4::launch_gemv_decode(ys, hcur, pk, ns, 1, H, delta, nullptr, w->final_norm, c->rms_eps,
+                                             false, delta_parts, s, nullptr, 0, amax_val, amax_idx)));
+      return from_hip(w4::launch_argmax_parts(amax_val, amax_idx, parts, d_token_out, d_pos, s));
+    }
     W4_TRY(from_hip(w4::launch_gemv_decode(ys, hcur, pk, ns, 1, H, delta, nullptr, w->final_norm, c->rms_eps,
                                            false, delta_parts, s)));
   }

@@ -260,6 +260,11 @@ struct RowPrologue {
   const float* norm_w;  // RMSNorm weight [K]
   float eps;
   int delta_parts;      // gemv_wide_kernel: delta is the sum of that many rows, K floats apart (0 or 1: one row)
+  // gemv_wide_kernel at M = 1: when given, wavefront w of the launch also leaves the largest of the outputs it
+  // stored and its column (the first such column; -inf and 0x7fffffff when it stored none) in amax_val[w],
+  // amax_idx[w], for a greedy sampler that then looks at wide_partials() pairs instead of N outputs
+  float* amax_val;
+  int* amax_idx;
 };
 struct GroupArgs {
   const uint8_t* packed[kMaxGroup];
@@ -1075,6 +1080,8 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
   }
   __syncthreads();
 
+  float best_v = -INFINITY;
+  int best_n = 0x7fffffff;
   for (int nt = wave_global; nt < NT; nt += wave_stride) {
     const int n = kTileRows * nt + j;
     float rs = 0.0f, bs = 0.0f;
@@ -1154,10 +1161,38 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
           v = __fmaf_rn(v, recip_m[m], bs);
           v = fminf(fmaxf(v, -3.402823466e+38f), 3.402823466e+38f);
           y[(size_t)m * N + n] = v;
+          if (M == 1 && (v > best_v || (v == best_v && n < best_n))) {  // columns rise: the first maximum stays
+            best_v = v;
+            best_n = n;
+          }
         }
       }
     }
   }
+  if constexpr (M == 1) {
+    if (pro.amax_val) {
+      // lanes 0..15 hold the candidates of their columns: the largest value, the lowest column among equals
+#pragma unroll
+      for (int off = 8; off >= 1; off >>= 1) {
+        const float ov = __shfl_xor(best_v, off, 64);
+        const int on = __shfl_xor(best_n, off, 64);
+        if (ov > best_v || (ov == best_v && on < best_n)) {
+          best_v = ov;
+          best_n = on;
+        }
+      }
+      if (lane == 0) {
+        pro.amax_val[wave_global] = best_v;
+        pro.amax_idx[wave_global] = best_n;
+      }
+    }
+  }
+}
+
+// wavefronts (= partial results) of a wide launch for N outputs
+int wide_partials(int N) {
+  const int NT = (N + kTileRows - 1) / kTileRows;
+  return std::min((NT + kWideWaves - 1) / kWideWaves, 1024) * kWideWaves;
 }
 
 template <int M, bool kFused, bool kNorm>
@@ -1184,6 +1219,7 @@ static bool wide_applies(int K, int N) {
   (void)K;
   return (N + kTileRows - 1) / kTileRows >= kWideMinTiles;
 }
+bool gemv_wide_applies(int K, int N) { return wide_applies(K, N); }
 
 #define W4_DISPATCH_M(CALL)   \
   switch (M) {               \
@@ -1377,8 +1413,9 @@ hipError_t launch_gemv_attn_rows(float* y, const float* part, int slices, const 
 hipError_t launch_gemv_decode(float* const* y, const float* x, const uint8_t* const* packed,
                               const int* N, int count, int K, const float* delta, float* sum_out,
                               const float* norm_w, float eps, bool pair, int in_parts, hipStream_t s,
-                              const int64_t* x_row, int x_rows) {
-  RowPrologue pro{delta, sum_out, norm_w, eps, in_parts};
+                              const int64_t* x_row, int x_rows, float* amax_val, int* amax_idx) {
+  RowPrologue pro{delta, sum_out, norm_w, eps, in_parts, amax_val, amax_idx};
+  if (amax_val && !(count == 1 && wide_applies(K, N[0]) && amax_idx)) return hipErrorInvalidValue;
   int ldx = K;
   if (x_row) {  // a gathered row: through the norm prologue of the tile-row kernels only, no delta, no pair
     if (!norm_w || delta || x_rows <= 0 || pair || in_parts > 1) return hipErrorInvalidValue;

@@ -900,6 +900,54 @@ __global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ l
   }
 }
 
+// The same decision from partial results: (value, index) pairs, each the first maximum of a disjoint set of
+// logits, as the lm_head launch leaves them (one pair per wavefront; n <= 4096). One workgroup of 1024 threads:
+// every thread requests its four pairs at once, wavefronts reduce with shuffles, the first one finishes.
+__global__ __launch_bounds__(1024) void argmax_parts_kernel(const float* __restrict__ val,
+                                                            const int* __restrict__ idx, int n,
+                                                            int64_t* __restrict__ token_out, int* pos_to_advance) {
+  __shared__ float s_val[16];
+  __shared__ int s_idx[16];
+  float v[4];
+  int ix[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int i = (int)threadIdx.x + 1024 * k;
+    const int ic = i < n ? i : n - 1;  // a duplicate of a real pair: harmless
+    v[k] = val[ic];
+    ix[k] = idx[ic];
+  }
+  float bv = v[0];
+  int bi = ix[0];
+#pragma unroll
+  for (int k = 1; k < 4; ++k) argmax_merge(bv, bi, v[k], ix[k]);
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, 64);
+    const int oi = __shfl_xor(bi, off, 64);
+    argmax_merge(bv, bi, ov, oi);
+  }
+  if ((threadIdx.x & 63) == 0) {
+    s_val[threadIdx.x >> 6] = bv;
+    s_idx[threadIdx.x >> 6] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x < 64) {
+    bv = s_val[threadIdx.x & 15];
+    bi = s_idx[threadIdx.x & 15];
+#pragma unroll
+    for (int off = 8; off >= 1; off >>= 1) {
+      const float ov = __shfl_xor(bv, off, 64);
+      const int oi = __shfl_xor(bi, off, 64);
+      argmax_merge(bv, bi, ov, oi);
+    }
+    if (threadIdx.x == 0) {
+      *token_out = bi == 0x7fffffff ? 0 : bi;  // all -inf / NaN: token 0, as the reference's scan
+      if (pos_to_advance) *pos_to_advance += 1;
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // im2col for a Conv3D without padding and dilation (the vision patch embedding), so that the
 // convolution becomes the same quantized Linear: row = (b, ot, oh, ow), column = (c, kt, kh, kw),
@@ -1079,6 +1127,13 @@ hipError_t launch_argmax(const float* logits, int n, float* part_val, int* part_
                          hipStream_t s) {
   hipLaunchKernelGGL(argmax_kernel, dim3(blocks), dim3(256), 0, s, logits, n, part_val, part_idx,
                      counter, token_out, pos_to_advance);
+  return hipGetLastError();
+}
+
+hipError_t launch_argmax_parts(const float* val, const int* idx, int n, int64_t* token_out, int* pos_to_advance,
+                               hipStream_t s) {
+  if (n <= 0 || n > 4096) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(argmax_parts_kernel, dim3(1), dim3(1024), 0, s, val, idx, n, token_out, pos_to_advance);
   return hipGetLastError();
 }
 

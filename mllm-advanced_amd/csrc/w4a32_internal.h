@@ -55,7 +55,12 @@ bool gemv_decode_applies(int K, const int* N, int count, bool pair);
 hipError_t launch_gemv_decode(float* const* y, const float* x, const uint8_t* const* packed,
                               const int* N, int count, int K, const float* delta, float* sum_out,
                               const float* norm_w, float eps, bool pair, int in_parts, hipStream_t s,
-                              const int64_t* x_row = nullptr, int x_rows = 0);
+                              const int64_t* x_row = nullptr, int x_rows = 0, float* amax_val = nullptr,
+                              int* amax_idx = nullptr);
+// lm_head-sized Linears (one wavefront per tile row): does that kernel take [N][K], and how many wavefronts
+// (partial argmax results, see launch_gemv_decode's amax_val / amax_idx) does its launch have
+bool gemv_wide_applies(int K, int N);
+int wide_partials(int N);
 // one decode row through one Linear with its k range dealt to gemv_kparts(K, N) workgroups per tile row, the
 // result left as that many partial rows y_parts[p][N] for the reader to add up (1: the shape is not split)
 int gemv_kparts(int K, int N);
@@ -130,6 +135,8 @@ hipError_t launch_gemv_attn_rows(float* y, const float* part, int slices, const 
 hipError_t launch_argmax(const float* logits, int n, float* part_val, int* part_idx,
                          unsigned int* counter, int64_t* token_out, int* pos_to_advance, int blocks,
                          hipStream_t s);
+hipError_t launch_argmax_parts(const float* val, const int* idx, int n, int64_t* token_out, int* pos_to_advance,
+                               hipStream_t s);
 hipError_t launch_im2col_conv3d(const float* a, float* z, int B, int C, int T, int H, int W, int kt,
                                 int kh, int kw, int st, int sh, int sw, int ld, hipStream_t s);
 hipError_t launch_set_int(int* p, int value, hipStream_t s);
