@@ -379,7 +379,7 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
       for (int e = 0; e < 8; ++e) xv[m][r][e] = f[e];
     }
   }
-  float dv[kNorm ? M : 1][kNorm ? kFusedR : 1][8];  // delta, then the norm weight
+  float dv[kNorm ? M : 1][kNorm ? kFusedR : 1][8];  // delta
   if (kNorm && pro_delta) {
 #pragma unroll
     for (int m = 0; m < M; ++m) {
@@ -394,6 +394,21 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
 #pragma unroll
         for (int e = 0; e < 8; ++e) dv[m][r][e] = f[e];
       }
+    }
+  }
+  // The norm weight is requested here, before the weights: a CU's memory pipe returns loads in issue order, and
+  // behind this workgroup's weight loads it would arrive after all of them, with the normalisation waiting for it.
+  float nwv[kNorm ? kFusedR : 1][8];
+  if constexpr (kNorm) {
+#pragma unroll
+    for (int r = 0; r < kFusedR; ++r) {
+      const int c = threadIdx.x + r * nthreads;
+      const int cc = c < groups ? c : groups - 1;
+      const float4 v0 = *reinterpret_cast<const float4*>(pro_norm_w + 8 * cc);
+      const float4 v1 = *reinterpret_cast<const float4*>(pro_norm_w + 8 * cc + 4);
+      const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) nwv[r][e] = f[e];
     }
   }
   // A producer that ran split over K (gemv_kparts_kernel) leaves its result as up to three partial rows:
@@ -492,17 +507,6 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
       ss = wave_sum_to_lane63(ss);
       if (lane == 63) s_ss[wave * M + m] = ss;
     }
-    // the norm weight travels while the partial sums meet
-#pragma unroll
-    for (int r = 0; r < kFusedR; ++r) {
-      const int c = threadIdx.x + r * nthreads;
-      const int cc = c < groups ? c : groups - 1;
-      const float4 v0 = *reinterpret_cast<const float4*>(pro_norm_w + 8 * cc);
-      const float4 v1 = *reinterpret_cast<const float4*>(pro_norm_w + 8 * cc + 4);
-      const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-#pragma unroll
-      for (int e = 0; e < 8; ++e) dv[0][r][e] = f[e];
-    }
     __syncthreads();
 #pragma unroll
     for (int m = 0; m < M; ++m) {
@@ -512,7 +516,7 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
 #pragma unroll
       for (int r = 0; r < kFusedR; ++r) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) xv[m][r][e] = xv[m][r][e] * (dv[0][r][e] * rstd);
+        for (int e = 0; e < 8; ++e) xv[m][r][e] = xv[m][r][e] * (nwv[r][e] * rstd);
       }
     }
   }
