@@ -605,7 +605,33 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
   const int hk = h0 / G;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int kq = lane >> 4, dl = lane & 15;
-  if (d_pos0) pos0 = *d_pos0;
+  const int pdl = dl ^ 8;                      // the lane position that holds the RoPE partner dims
+  if (d_pos0) pos0 = *d_pos0;                  // (a scalar load: nothing waits for it before its first use below)
+
+  auto load8 = [](const float* src, float (&dst)[8]) {
+    const float4 a = *reinterpret_cast<const float4*>(src);
+    const float4 b = *reinterpret_cast<const float4*>(src + 4);
+    dst[0] = a.x; dst[1] = a.y; dst[2] = a.z; dst[3] = a.w;
+    dst[4] = b.x; dst[5] = b.y; dst[6] = b.z; dst[7] = b.w;
+  };
+  // What does not depend on the position is requested while the position is on its way: q and (kRope) the new
+  // token's k and v, each lane's own dims and, for the rotation, its partner's. Every wavefront asks for the
+  // new k and v (three cached rows); only the one whose keys include the position uses them.
+  float q_own[kGW][8], q_oth[kRope ? kGW : 1][8];
+#pragma unroll
+  for (int g = 0; g < kGW; ++g) {
+    const float* src = q + (size_t)(h0 + g) * kHeadDim;
+    load8(src + 8 * dl, q_own[g]);
+    if (kRope) load8(src + 8 * pdl, q_oth[g]);
+  }
+  float kn_own[8], kn_oth[8], vnew[8];
+  if (kRope) {
+    load8(k_new + (size_t)hk * kHeadDim + 8 * dl, kn_own);
+    load8(k_new + (size_t)hk * kHeadDim + 8 * pdl, kn_oth);
+    load8(v_new + (size_t)hk * kHeadDim + 8 * dl, vnew);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
   if (pos0 >= max_seq) pos0 = max_seq - 1;     // the caller keeps the position inside the cache
   const int len = pos0 + 1;
   // keys of this workgroup, then of this wavefront (multiples of 4 so that slots stay aligned)
@@ -614,31 +640,20 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
   const int begin = min((int)blockIdx.y * per_wg + wave * per_wave, len);
   const int end = min(begin + per_wave, len);
 
-  auto load8 = [](const float* src, float (&dst)[8]) {
-    const float4 a = *reinterpret_cast<const float4*>(src);
-    const float4 b = *reinterpret_cast<const float4*>(src + 4);
-    dst[0] = a.x; dst[1] = a.y; dst[2] = a.z; dst[3] = a.w;
-    dst[4] = b.x; dst[5] = b.y; dst[6] = b.z; dst[7] = b.w;
-  };
   // y0 = x0 c - x1 s (first half of the head), y1 = x0 s + x1 c (second half)
-  const int pdl = dl ^ 8;                      // the lane position that holds the partner dims
   float sn[8], cs[8];
   if (kRope) {
     load8(sin_t + (size_t)pos0 * (kHeadDim / 2) + 8 * (dl & 7), sn);
     load8(cos_t + (size_t)pos0 * (kHeadDim / 2) + 8 * (dl & 7), cs);
   }
-  auto rotate = [&](const float* vec, float (&dst)[8]) {
-    float own[8], oth[8];
-    load8(vec + 8 * dl, own);
-    load8(vec + 8 * pdl, oth);
+  auto rotate = [&](const float (&own)[8], const float (&oth)[8], float (&dst)[8]) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       dst[i] = dl < 8 ? own[i] * cs[i] - oth[i] * sn[i] : oth[i] * sn[i] + own[i] * cs[i];
     }
   };
 
-  // The first block of K and V rows depends only on the position: it is requested before q, the
-  // RoPE factors and the new token's k, v, whose latency it then shares instead of following.
+  // The first block of K and V rows depends only on the position: it is requested as soon as that is known.
   const float* kbase = kc + (size_t)hk * max_seq * kHeadDim + 8 * dl;
   const float* vbase = vc + (size_t)hk * max_seq * kHeadDim + 8 * dl;
   float kk[4][8], vv[4][8];
@@ -657,18 +672,17 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
   float qr[kGW][8];
 #pragma unroll
   for (int g = 0; g < kGW; ++g) {
-    const float* src = q + (size_t)(h0 + g) * kHeadDim;
     if (kRope) {
-      rotate(src, qr[g]);
+      rotate(q_own[g], q_oth[g], qr[g]);
     } else {
-      load8(src + 8 * dl, qr[g]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) qr[g][i] = q_own[g][i];
     }
   }
-  float knew[8], vnew[8];
+  float knew[8];
   const bool has_new = kRope && begin <= pos0 && pos0 < end;   // wavefront-uniform
   if (has_new) {
-    rotate(k_new + (size_t)hk * kHeadDim, knew);
-    load8(v_new + (size_t)hk * kHeadDim + 8 * dl, vnew);
+    rotate(kn_own, kn_oth, knew);
     if (h0 % G == 0 && blockIdx.x * kGW == (unsigned)h0 && kq == 0) {
       float* kd = kc + ((size_t)hk * max_seq + pos0) * kHeadDim + 8 * dl;
       float* vd = vc + ((size_t)hk * max_seq + pos0) * kHeadDim + 8 * dl;
