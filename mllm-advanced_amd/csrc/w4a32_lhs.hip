@@ -123,11 +123,23 @@ __global__ __launch_bounds__(kLhsThreads) void quant_rows_kernel(
           if (nparts > 0) {
             // b = the parts of a split-K product, [nparts][M][K] with the row and column factors applied:
             // delta = ((part 0 + part 1) + ...) + bias, clamped like every Linear output
-            for (int p = 1; p < nparts; ++p) {
-              const float4 e0 = *reinterpret_cast<const float4*>(b + p * part_stride + row + i);
-              const float4 e1 = *reinterpret_cast<const float4*>(b + p * part_stride + row + i + 4);
-              d0.x += e0.x; d0.y += e0.y; d0.z += e0.z; d0.w += e0.w;
-              d1.x += e1.x; d1.y += e1.y; d1.z += e1.z; d1.w += e1.w;
+            // four parts are requested at a time (one memory round trip, not four) and added in their order;
+            // a part past the last one is read from part 0's place again and not added
+            for (int p0 = 1; p0 < nparts; p0 += 4) {
+              float4 e0[4], e1[4];
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                const size_t off = (size_t)(p0 + q < nparts ? p0 + q : 0) * part_stride + row + i;
+                e0[q] = *reinterpret_cast<const float4*>(b + off);
+                e1[q] = *reinterpret_cast<const float4*>(b + off + 4);
+              }
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                if (p0 + q < nparts) {
+                  d0.x += e0[q].x; d0.y += e0[q].y; d0.z += e0[q].z; d0.w += e0[q].w;
+                  d1.x += e1[q].x; d1.y += e1[q].y; d1.z += e1[q].z; d1.w += e1[q].w;
+                }
+              }
             }
             const float4 b0 = *reinterpret_cast<const float4*>(part_bias + i);
             const float4 b1 = *reinterpret_cast<const float4*>(part_bias + i + 4);
