@@ -594,9 +594,10 @@ def main():
             "decode_ms_per_token": round(decode_ms / n_new, 4),
             "decode_tokens_per_s": round(n_new / (decode_ms * 1e-3), 1),
             "decode_weight_GBps": round(step_bytes / (decode_ms / n_new * 1e-3) / 1e9, 1),
-            "note": "one decode step = 143 launches (embedding, 28 x [add+norm+qkv, rope+cache+attention, o, "
-                    "add+norm+gate/up+silu*mul, down], add+norm+lm_head, argmax), captured once and replayed; "
-                    "positions and cache lengths are read from device memory",
+            "note": "one decode step = 142 launches (28 x [add+norm+qkv (layer 0: on the token's embedding row, "
+                    "gathered), rope+cache+attention slices, o merging the slices, add+norm+gate/up+silu*mul, down "
+                    "in two k-parts], add+norm+lm_head, argmax over lm_head's partial results), captured once and "
+                    "replayed; positions and cache lengths are read from device memory",
         }
         # config 5, language side: prefill of the 256 merged vision tokens through the same decoder
         with torch.cuda.stream(stream):
