@@ -368,6 +368,33 @@ def test_decoder_ignores_what_its_state_memory_held(pkg):
         assert torch.equal(a, b)
 
 
+def test_decoder_step_gathers_the_token_s_embedding_row_itself(pkg):
+    # The first launch of a step reads row `token` of the embedding table (no gather launch in front of it):
+    # a step on token t must equal a one-token prefill of [t] bit for bit in what it leaves as the residual
+    # stream's start and in its logits' token, and ids outside the table are clamped to it as the embedding
+    # operator clamps them (LLMEmbeddingTokenOp.cpp:24-50 reads the row; out-of-range ids are undefined there).
+    rng = np.random.default_rng(11)
+    H, Hq, Hkv, I, V, L = 256, 2, 1, 384, 640, 2
+    weights = tiny_model(rng, H, Hq, Hkv, I, V, L)
+    emb = weights["embedding"]
+    outs = {}
+    for tok in (0, 5, V - 1, V + 7, -3):
+        dec = to_device_model(pkg, weights, Hq, Hkv, max_seq=32, max_batch_tokens=16, rope_theta=1e6)
+        dec.token.fill_(tok)
+        dec.step()
+        torch.cuda.synchronize()
+        outs[tok] = (dec.logits.clone(), int(dec.token))
+        row = min(max(tok, 0), V - 1)
+        ref = to_device_model(pkg, weights, Hq, Hkv, max_seq=32, max_batch_tokens=16, rope_theta=1e6)
+        ref.prefill(dev(np.array([row], dtype=np.int64)))
+        torch.cuda.synchronize()
+        assert int(ref.token) == outs[tok][1], tok
+        assert max_abs_rel(outs[tok][0].cpu().numpy(), ref.logits.cpu().numpy()) < 2e-3, tok
+        assert np.isfinite(outs[tok][0].cpu().numpy()).all()
+    assert torch.equal(outs[V + 7][0], outs[V - 1][0]) and torch.equal(outs[-3][0], outs[0][0])
+    assert not torch.equal(outs[0][0], outs[5][0]) and emb.shape == (V, H)
+
+
 @pytest.mark.parametrize("prompt_len", [300, 520])
 def test_decoder_runner_at_the_model_s_widths(pkg, prompt_len):
     # hidden 1536, 12 / 2 heads, MLP 8960 (two layers, small vocabulary): the prefill runs the kernels the
