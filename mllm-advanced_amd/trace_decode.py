@@ -27,7 +27,7 @@ POINTS = ["workgroup starts", "row arrived, range known", "quantisation paramete
           "weights arrived, products done", "sums in LDS", "outputs stored"]
 
 
-def trace(label, K, Ns, sets):
+def trace(label, K, Ns, sets, nwg=None):
     g = torch.Generator(device="cuda").manual_seed(0)
     packs = [[pkg.quant_pack_rhs(torch.randn((n, K), generator=g, device="cuda") * 0.02) for n in Ns]
              for _ in range(sets)]                     # more weight sets than the 256 MB cache holds: cold every time
@@ -35,7 +35,9 @@ def trace(label, K, Ns, sets):
     ys = [torch.empty((1, n), device="cuda") for n in Ns]
     ws = torch.empty(pkg.workspace_bytes(1, K), dtype=torch.uint8, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
-    cnt, nwg = len(Ns), sum((n + 15) // 16 for n in Ns)
+    cnt = len(Ns)
+    if nwg is None:
+        nwg = sum((n + 15) // 16 for n in Ns)           # one workgroup per 16-row tile row of every Linear
     ya = (ctypes.c_void_p * cnt)(*[t.data_ptr() for t in ys])
     na = (ctypes.c_int * cnt)(*Ns)
     for _ in range(3):
@@ -57,7 +59,8 @@ def trace(label, K, Ns, sets):
 
 
 if __name__ == "__main__":
-    trace("gate,up grouped (K 1536, N 2 x 8960)", 1536, [8960, 8960], 20)
+    # two Linears of equal N on one row run as a pair: a workgroup takes tile row nt of both
+    trace("gate,up as a pair (K 1536, N 2 x 8960)", 1536, [8960, 8960], 20, nwg=8960 // 16)
     trace("o_proj (K 1536, N 1536)", 1536, [1536], 28)
     trace("q,k,v grouped (K 1536, N 1536 + 256 + 256)", 1536, [1536, 256, 256], 28)
     trace("down_proj unsplit, as w4a32_matmul runs it (K 8960, N 1536)", 8960, [1536], 28)
