@@ -140,7 +140,7 @@ constexpr int kF16BK = 64;    // k per stage (two scale blocks, half of a weight
 // Timing-only builds (make leaveout LEAVE_OUT=<mask>, read by mllm-advanced_amd/gemm_leave_out.py): the
 // steady-state loop without its barriers (1), without the weights' dequantisation and LDS writes (2), without
 // the packed weights' global loads (4), without the activation loads (8), without the LDS reads of the weight
-// fragments (16), without the products (32). The results are wrong; what such a build shows is how much of a
+// fragments (16), without the products (32), with half of each lane's activation loads (64). The results are wrong; what such a build shows is how much of a
 // stage's time waits for that part.
 #ifndef W4A32_GEMM_LEAVE_OUT
 #define W4A32_GEMM_LEAVE_OUT 0
@@ -356,7 +356,11 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
 #pragma unroll
     for (int a = 0; a < WM; ++a) {
       dst[kbl][a][0] = *reinterpret_cast<const uint4*>(a_ptr[a] + kbl * 2048);
-      dst[kbl][a][1] = *reinterpret_cast<const uint4*>(a_ptr[a] + kbl * 2048 + 16);
+      if (kLeaveOut & 64) {  // half the activation bytes: what a one-byte activation copy would load
+        dst[kbl][a][1] = dst[kbl][a][0];
+      } else {
+        dst[kbl][a][1] = *reinterpret_cast<const uint4*>(a_ptr[a] + kbl * 2048 + 16);
+      }
     }
   };
 
