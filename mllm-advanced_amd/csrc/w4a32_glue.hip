@@ -658,13 +658,17 @@ __global__ __launch_bounds__(64 * kDecWaves) void attention_decode_kernel(
   const float* vbase = vc + (size_t)hk * max_seq * kHeadDim + 8 * dl;
   float kk[4][8], vv[4][8];
   auto load_block = [&](int blk) {
+    // all K rows before the V rows: loads return in issue order and the scores need K only
+    const int last = end > begin ? end - 1 : 0;
 #pragma unroll
     for (int it = 0; it < 4; ++it) {
       const int key = blk + 4 * it + kq;
-      const int last = end > begin ? end - 1 : 0;
-      const size_t row = (size_t)(key < end ? key : last) * kHeadDim;
-      load8(kbase + row, kk[it]);
-      load8(vbase + row, vv[it]);
+      load8(kbase + (size_t)(key < end ? key : last) * kHeadDim, kk[it]);
+    }
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int key = blk + 4 * it + kq;
+      load8(vbase + (size_t)(key < end ? key : last) * kHeadDim, vv[it]);
     }
   };
   load_block(begin);
