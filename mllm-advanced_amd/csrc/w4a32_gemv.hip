@@ -1286,6 +1286,12 @@ static hipError_t launch_fused_group(const GroupArgs& ga, const float* x, int ld
   const FusedPlan p = fused_plan(M, K);
   if (p.W == 0) return hipErrorInvalidValue;
   const RowPrologue none{nullptr, nullptr, nullptr, 0.0f};
+  if (pair && !pro && M > 1) {  // two Linears of equal N on the same M rows, both outputs stored (ga.pair_both)
+    if (p.R != 1 || !ga.pair_both) return hipErrorInvalidValue;
+#define W4_CALL(m) (launch_fused_cpw<m, 1, false, true>(ga, x, ldx, K, p, none, s))
+    W4_DISPATCH_M(W4_CALL)
+#undef W4_CALL
+  }
   if (pro || pair) {
     if (M != 1) return hipErrorInvalidValue;
     const RowPrologue& pr = pro ? *pro : none;
@@ -1344,9 +1350,10 @@ hipError_t launch_gemv_group(float* const* y, const float* x, int ldx, const uin
   }
   ga.count = count;
   // one row through two Linears of equal N: the pair kernel with both outputs stored
-  if (M == 1 && count == 2 && N[0] == N[1] && fused_plan(1, K).W != 0 && fused_plan(1, K).CPW <= 3) {
+  const FusedPlan fp = fused_plan(M, K);
+  if (count == 2 && N[0] == N[1] && fp.W != 0 && fp.CPW <= 3 && fp.R == 1) {
     ga.pair_both = 1;
-    return launch_fused_group(ga, x, ldx, 1, K, nullptr, true, s);
+    return launch_fused_group(ga, x, ldx, M, K, nullptr, true, s);
   }
   return launch_fused_group(ga, x, ldx, M, K, nullptr, false, s);
 }
