@@ -199,7 +199,10 @@ def test_fused_decode_kernel_equals_two_step_path(pkg, orc, m, k, n):
 
 
 @pytest.mark.parametrize("m,k,ns", [(1, 1536, [1536, 256, 256]), (8, 1536, [1536, 256, 256]),
-                                    (1, 1536, [8960, 8960]), (4, 1536, [8960, 8960]),
+                                    (1, 1536, [8960, 8960]), (4, 1536, [8960, 8960]), (8, 1536, [8960, 8960]),
+                                    # two Linears of equal N: one workgroup per tile row of both (M <= 8)
+                                    (3, 256, [48, 48]), (2, 64, [40, 40]), (5, 1280, [1280, 1280]),
+                                    (1, 8960, [1536, 1536]),
                                     (1, 8960, [1536]), (4, 8960, [1536, 50]), (12, 256, [64, 48, 16, 100]),
                                     (2, 64, [40, 16]), (40, 256, [64, 48, 16, 100]),
                                     (130, 96, [50, 16]), (300, 1536, [1536, 256, 256]),
