@@ -137,16 +137,6 @@ __device__ __forceinline__ uint4 dequant8(uint32_t w, h2 s, h2 s16) {
 
 constexpr int kF16BK = 64;    // k per stage (two scale blocks, half of a weight tile chunk)
 
-// Timing-only builds (make leaveout LEAVE_OUT=<mask>, read by mllm-advanced_amd/gemm_leave_out.py): the
-// steady-state loop without its barriers (1), without the weights' dequantisation and LDS writes (2), without
-// the packed weights' global loads (4), without the activation loads (8), without the LDS reads of the weight
-// fragments (16), without the products (32), with half of each lane's activation loads (64). The results are wrong; what such a build shows is how much of a
-// stage's time waits for that part.
-#ifndef W4A32_GEMM_LEAVE_OUT
-#define W4A32_GEMM_LEAVE_OUT 0
-#endif
-constexpr int kLeaveOut = W4A32_GEMM_LEAVE_OUT;
-
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 // v_mfma_f32_32x32x16_f16 (8 passes of 4 clocks; measured on MI355X: twice the rate of the
@@ -356,11 +346,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
 #pragma unroll
     for (int a = 0; a < WM; ++a) {
       dst[kbl][a][0] = *reinterpret_cast<const uint4*>(a_ptr[a] + kbl * 2048);
-      if (kLeaveOut & 64) {  // half the activation bytes: what a one-byte activation copy would load
-        dst[kbl][a][1] = dst[kbl][a][0];
-      } else {
-        dst[kbl][a][1] = *reinterpret_cast<const uint4*>(a_ptr[a] + kbl * 2048 + 16);
-      }
+      dst[kbl][a][1] = *reinterpret_cast<const uint4*>(a_ptr[a] + kbl * 2048 + 16);
     }
   };
 
@@ -485,12 +471,11 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
       constexpr int LA = 2;
       static_assert(LA <= 2 * WN && LA < F, "a fragment would overwrite one that is still to be used");
       auto fetch = [&](int f, const uint8_t* base) {
-        if ((kLeaveOut & 16) && FORM == kSteady) return;
         bf[(f / WN) & 1][f % WN] =
             *reinterpret_cast<const h8*>(base + ((f / WN) * BN32 + wn * WN + f % WN) * 1024);
       };
       if (u % BE == 0) {
-        if (!((kLeaveOut & 1) && FORM == kSteady)) __syncthreads();
+        __syncthreads();
 #pragma unroll
         for (int f = 0; f < LA; ++f) fetch(f, bbuf);
         __builtin_amdgcn_sched_barrier(0);  // requested first: their latency covers what follows
@@ -514,10 +499,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
           dx[2 * q + 1] = breg[slot][q].y;
         }
       }
-      const bool dequantise =  // (after unrolling: a constant)
-          (FORM != kLast || u + BE < U) && !((kLeaveOut & 2) && FORM == kSteady);
+      const bool dequantise = FORM != kLast || u + BE < U;  // (after unrolling: a constant)
       if constexpr (FORM == kSteady) {
-        if (!(kLeaveOut & 4)) load_b_rel(u + BE + D, breg[slot], sreg[slot]);
+        load_b_rel(u + BE + D, breg[slot], sreg[slot]);
       } else {
         if (FORM != kLast || u + BE + D < U) load_b(s + BE + D, breg[slot], sreg[slot]);
       }
@@ -555,10 +539,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
         for (int b = 0; b < WN; ++b) {
 #pragma unroll
           for (int a = 0; a < WM; ++a) {
-            if (!((kLeaveOut & 32) && FORM == kSteady)) {
-              acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                  __builtin_bit_cast(h8, areg[slot][sl >> 1][a][sl & 1]), bf[sl & 1][b], acc[a][b], 0, 0, 0);
-            }
+            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                __builtin_bit_cast(h8, areg[slot][sl >> 1][a][sl & 1]), bf[sl & 1][b], acc[a][b], 0, 0, 0);
             if (a == 0) {
               const int f = sl * WN + b + LA;
               if (f < F) {
@@ -579,7 +561,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
           if constexpr (TAIL) {
             if (FORM != kLast || u + D < U) load_a_kb(s + D, sl >> 1, areg[slot]);
           } else {
-            if (!(kLeaveOut & 8)) load_a_kb_next(sl >> 1, areg[slot]);
+            load_a_kb_next(sl >> 1, areg[slot]);
           }
         }
       }

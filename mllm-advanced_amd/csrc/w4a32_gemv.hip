@@ -41,24 +41,6 @@
 
 namespace w4 {
 
-// Optional timestamps (make trace: -DW4A32_TRACE, a library of its own): thread 0 of every workgroup of
-// gemv_fused_kernel records the wall clock (100 MHz) at seven points of its life; w4a32_trace_dump() copies them
-// out. `dep` makes the point wait for the value it names (a loaded row, the products), so that the stamp is taken
-// when that value exists. The product build compiles the macro to nothing.
-#ifdef W4A32_TRACE
-constexpr int kTraceWorkgroups = 8192, kTracePoints = 8;
-__device__ unsigned long long g_trace[kTraceWorkgroups * kTracePoints];
-__device__ __forceinline__ void trace_point(int i, float dep) {
-  asm volatile("" ::"v"(dep) : "memory");
-  const unsigned long long t = wall_clock64();
-  if (threadIdx.x == 0 && blockIdx.x < kTraceWorkgroups) g_trace[blockIdx.x * kTracePoints + i] = t;
-  asm volatile("" ::: "memory");
-}
-#define W4_TRACE(i, dep) trace_point((i), (dep))
-#else
-#define W4_TRACE(i, dep) ((void)0)
-#endif
-
 typedef int v4i_t __attribute__((ext_vector_type(4)));
 constexpr int kDecodeMfmaMinM = 3;
 constexpr bool decode_mfma(int M) { return M >= kDecodeMfmaMinM; }
@@ -347,7 +329,6 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
   // x first (a few KB, normally in L2), then the weights, so that the min/max and quantise passes
   // run while the weights are on their way from HBM.
   const int groups = K >> 3;
-  W4_TRACE(0, 0.0f);  // the workgroup has started
   // kNorm at M = 1 with ldx < 0 (a row stride has no use at M = 1): x is a table of -ldx rows of K floats, the
   // delta argument points to an int64 row number instead, and the input row is that row of the table (the number
   // clamped to it); workgroup 0 copies the row to sum_out. The decoder's first launch of a token reads the
@@ -533,7 +514,6 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
       }
     }
     wave_minmax_pair(lo, hi);
-    if (m == 0) W4_TRACE(1, lo);  // the row has arrived and this wavefront's range is known
     if (lane == 63) s_mm[wave * M + m] = make_float2(lo, hi);
   }
   __syncthreads();
@@ -547,7 +527,6 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
     par[m] = row_quant_params(v.x, v.y);
   }
 
-  W4_TRACE(2, par[0].recip);  // quantisation parameters
   // Quantise into the LDS copy; the tile padding (k >= K) is 0.
   const int grp_per_row = Kp >> 3;
 #pragma unroll
@@ -563,7 +542,6 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
     }
   }
   __syncthreads();
-  W4_TRACE(3, 0.0f);  // the int8 row is in LDS
 
   float acc[kSets][decode_acc(M)];
 #pragma unroll
@@ -585,12 +563,10 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
       }
     }
   }
-  W4_TRACE(4, acc[0][0]);  // the weights have arrived and this wavefront's products are done
   // The sums of the four k-groups of a row, then across wavefronts via LDS.
 #pragma unroll
   for (int st = 0; st < kSets; ++st) store_row_sums<M>(acc[st], s_red + (wave * kSets + st) * M * 16, lane);
   __syncthreads();
-  W4_TRACE(5, 0.0f);  // every wavefront's sums are in LDS
 
   //   y = (sum/16 + off * rsum[n]) * lhs_scale + bias[n], clamped to the finite f32 range
   const bool prefetched = nthreads >= kOutputs;
@@ -631,7 +607,6 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
       *(W4_GLOBAL float*)(y + (size_t)m * N + n) = v;
     }
   }
-  W4_TRACE(6, 0.0f);  // outputs stored
 }
 
 // One decode row through ONE Linear with a long K, the k range dealt to kDecodeParts workgroups per tile row
@@ -1462,11 +1437,3 @@ hipError_t launch_gemv_decode(float* const* y, const float* x, const uint8_t* co
 }
 
 }  // namespace w4
-
-#ifdef W4A32_TRACE
-// [workgroup][point] wall-clock ticks (10 ns) of the last gemv_fused_kernel launch; n = entries of `host`.
-extern "C" int w4a32_trace_dump(unsigned long long* host, size_t n) {
-  const size_t have = (size_t)w4::kTraceWorkgroups * w4::kTracePoints;
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(w4::g_trace), (n < have ? n : have) * sizeof(unsigned long long));
-}
-#endif
