@@ -208,6 +208,21 @@ int w4a32_op_attention_bshd(const float* d_q, const float* d_k, const float* d_v
  * how the reference applies lm_head, modeling_ds_qwen2.hpp:209-213). K % 4 == 0. M <= 8 streams B once. */
 int w4a32_op_matmul_f32_nt(const float* d_a, const float* d_b, float* d_c, int M, int N, int K, void* stream);
 
+/* Element types of a dense (unquantised) operand. The reference's W4A32 quantizer configuration stores lm_head
+ * and the three RMSNorm weights as Fp16 (scripts/QuantCfg/ds_qwen2/1.5B-W4A32-KAI.json:33-45). */
+#define W4A32_DENSE_F32 1
+#define W4A32_DENSE_F16 2
+
+/* The same product with B [N][K] held as f32 or f16 (b_dtype = W4A32_DENSE_*): an f16 element widens to f32
+ * exactly, every product and sum is f32. With K % 8 == 0 and M <= 8, B is streamed once and the f16 and the f32
+ * form of the same values give identical bits. K % 4 == 0. */
+int w4a32_op_matmul_nt(const float* d_a, const void* d_b, int b_dtype, float* d_c, int M, int N, int K,
+                       void* stream);
+
+/* d_out[i] = (float)d_in[i] for n IEEE half values (exact): Fp16 parameters of a model file are widened once at
+ * load and the f32 operators run on the result. */
+int w4a32_op_f16_to_f32(const void* d_in, float* d_out, size_t n, void* stream);
+
 /* ---- decoder runner -------------------------------------------------------------------- */
 
 typedef struct {
@@ -223,11 +238,17 @@ typedef struct {
   const float *attn_norm, *ffn_norm;
 } w4a32_layer_weights;
 
+/* Zero-initialise the struct before filling it (fields may be added at its end). */
 typedef struct {
   const float* embedding;             /* [vocab][hidden] f32 */
   const float* final_norm;            /* [hidden] */
-  const void* lm_head;                /* W4 blob [vocab][hidden] */
+  const void* lm_head;                /* W4 blob [vocab][hidden]; may be NULL when lm_head_dense is given */
   const w4a32_layer_weights* layers;  /* HOST array of n_layers entries */
+  /* lm_head as the reference applies it (a dense matmul with transpose_b, modeling_ds_qwen2.hpp:209-213):
+   * [vocab][hidden] of lm_head_dense_dtype (W4A32_DENSE_F16 as the reference's quantizer stores it, or
+   * W4A32_DENSE_F32). When not NULL it is used instead of lm_head; hidden % 8 == 0. */
+  const void* lm_head_dense;
+  int lm_head_dense_dtype;
 } w4a32_decoder_weights;
 
 /* Bytes of the decoder state (KV caches, activations, tables, counters), 256-byte aligned base. */

@@ -20,6 +20,7 @@ BF16_TRUNC = 0
 BF16_RNE = 1
 KERNEL_AUTO, KERNEL_GEMV, KERNEL_GEMM_I8, KERNEL_GEMM_F16 = 0, 1, 2, 3
 KERNEL_GEMM_F16_TILE0, GEMM_F16_TILES = 16, 10  # + i: the f16 kernel with tile shape i
+DENSE_F32, DENSE_F16 = 1, 2  # element types of a dense (unquantised) operand
 
 #: every symbol include/w4a32_hip.h declares, with (restype, argtypes)
 _vp, _ci, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
@@ -76,6 +77,8 @@ ABI = {
     "w4a32_op_rope": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp]),
     "w4a32_op_attention_bshd": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _vp]),
     "w4a32_op_matmul_f32_nt": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp]),
+    "w4a32_op_matmul_nt": (_ci, [_vp, _vp, _ci, _vp, _ci, _ci, _ci, _vp]),
+    "w4a32_op_f16_to_f32": (_ci, [_vp, _vp, _sz, _vp]),
     "w4a32_decode_linear": (_ci, [_vp, _vp]),
     "w4a32_decode_kparts": (_ci, [_ci, _ci]),
     "w4a32_decoder_state_bytes": (_sz, [_vp]),
@@ -111,7 +114,8 @@ class LayerWeights(ctypes.Structure):
 class DecoderWeights(ctypes.Structure):
     """w4a32_decoder_weights"""
     _fields_ = [("embedding", ctypes.c_void_p), ("final_norm", ctypes.c_void_p),
-                ("lm_head", ctypes.c_void_p), ("layers", ctypes.POINTER(LayerWeights))]
+                ("lm_head", ctypes.c_void_p), ("layers", ctypes.POINTER(LayerWeights)),
+                ("lm_head_dense", ctypes.c_void_p), ("lm_head_dense_dtype", ctypes.c_int)]
 
 
 class W4A32Error(RuntimeError):
@@ -504,6 +508,35 @@ def op_matmul_f32_nt(a, b):
     return out
 
 
+def _dense_dtype(b):
+    import torch
+
+    if b.dtype == torch.float16:
+        return DENSE_F16
+    if b.dtype == torch.float32:
+        return DENSE_F32
+    raise W4A32Error(f"a dense operand is f16 or f32, not {b.dtype}")
+
+
+def op_matmul_nt(a, b):
+    """a f32 [M][K] x b [N][K]^T with b held as f16 or f32; products and sums in f32."""
+    import torch
+
+    (M, K), N = a.shape, b.shape[0]
+    out = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    _check(lib().w4a32_op_matmul_nt(_ptr(a), _ptr(b), _dense_dtype(b), _ptr(out), M, N, K, _stream()),
+           "w4a32_op_matmul_nt")
+    return out
+
+
+def op_f16_to_f32(x):
+    import torch
+
+    out = torch.empty(x.shape, dtype=torch.float32, device="cuda")
+    _check(lib().w4a32_op_f16_to_f32(_ptr(x), _ptr(out), x.numel(), _stream()), "w4a32_op_f16_to_f32")
+    return out
+
+
 def op_scratch(n_heads):
     sc = _dev_empty(int(lib().w4a32_op_scratch_bytes(n_heads)))
     _check(lib().w4a32_op_scratch_init(_ptr(sc), n_heads, _stream()), "w4a32_op_scratch_init")
@@ -603,10 +636,12 @@ class Decoder:
     """Plumbing around the decoder runner: owns the state buffer and the argument structs.
 
     `layers` is a list of dicts with the packed blobs q,k,v,o,gate,up,down and the f32 norm weights
-    attn_norm, ffn_norm (cuda tensors); embedding f32 [vocab][hidden]; lm_head a packed blob."""
+    attn_norm, ffn_norm (cuda tensors); embedding f32 [vocab][hidden]; lm_head a packed blob, or (with
+    lm_head_dense=True) a dense f16 / f32 [vocab][hidden] tensor applied as the reference applies it."""
 
     def __init__(self, hidden, n_heads, n_kv_heads, intermediate, vocab, layers, embedding, final_norm,
-                 lm_head, max_seq=1024, max_batch_tokens=512, rope_theta=1e6, rms_eps=1e-6, head_dim=128):
+                 lm_head, max_seq=1024, max_batch_tokens=512, rope_theta=1e6, rms_eps=1e-6, head_dim=128,
+                 lm_head_dense=False):
         import torch
 
         self.cfg = DecoderConfig(hidden, n_heads, n_kv_heads, head_dim, intermediate, len(layers), vocab,
@@ -617,7 +652,12 @@ class Decoder:
             for name, _ in LayerWeights._fields_:
                 setattr(arr[i], name, lw[name].data_ptr())
         self._layers = arr
-        self.weights = DecoderWeights(embedding.data_ptr(), final_norm.data_ptr(), lm_head.data_ptr(), arr)
+        if lm_head_dense:
+            self.weights = DecoderWeights(embedding.data_ptr(), final_norm.data_ptr(), None, arr,
+                                          lm_head.data_ptr(), _dense_dtype(lm_head))
+        else:
+            self.weights = DecoderWeights(embedding.data_ptr(), final_norm.data_ptr(), lm_head.data_ptr(), arr,
+                                          None, 0)
         nbytes = int(lib().w4a32_decoder_state_bytes(ctypes.byref(self.cfg)))
         if nbytes == 0:
             raise W4A32Error("w4a32_decoder_state_bytes: invalid configuration")

@@ -226,7 +226,12 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
   const size_t last = (size_t)(M - 1) * H;
   W4_TRY(from_hip(w4::launch_rmsnorm(h + last, delta + last, w->final_norm, 1, H, c->rms_eps, h + last,
                                      xn + last, s)));
-  W4_TRY(w4a32_matmul(logits, xn + last, w->lm_head, ws, 1, H, c->vocab, stream));
+  if (w->lm_head_dense) {
+    W4_TRY(from_hip(w4::launch_dense_rows(xn + last, H, w->lm_head_dense, w->lm_head_dense_dtype, logits, 1,
+                                          c->vocab, H, s)));
+  } else {
+    W4_TRY(w4a32_matmul(logits, xn + last, w->lm_head, ws, 1, H, c->vocab, stream));
+  }
   W4_TRY(from_hip(w4::launch_argmax(logits, c->vocab, reinterpret_cast<float*>(scratch + sg.amax_val_off),
                                     reinterpret_cast<int*>(scratch + sg.amax_idx_off),
                                     reinterpret_cast<unsigned int*>(scratch + sg.counters_off) + Hq,
@@ -234,17 +239,25 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
   return W4A32_OK;
 }
 
+// lm_head is given, as a W4 blob or as a dense operand of a known element type that the dense kernel takes
+int head_ok(const w4a32_decoder_config* c, const w4a32_decoder_weights* w) {
+  if (!w->lm_head_dense) return w->lm_head ? W4A32_OK : W4A32_EINVAL;
+  if (w->lm_head_dense_dtype != W4A32_DENSE_F32 && w->lm_head_dense_dtype != W4A32_DENSE_F16) return W4A32_EINVAL;
+  if ((reinterpret_cast<uintptr_t>(w->lm_head_dense) & 15) != 0) return W4A32_EINVAL;
+  return w4::dense_rows_applies(1, c->hidden) ? W4A32_OK : W4A32_ESHAPE;
+}
+
 // One decode row with the operators between the Linears folded into them: 5 launches per layer
 // ([add+norm+q,k,v] [rope+cache+attention] [o] [add+norm+gate,up+silu*mul] [down]) instead of 9.
 // The residual stream alternates between two buffers because the launch that completes a row
 // (x + delta) is read by every workgroup while one of them stores the sum.
-bool decode_fusable(const w4a32_decoder_config* c) {
+bool decode_fusable(const w4a32_decoder_config* c, bool dense_head) {
   const int qd = c->n_heads * c->head_dim, kvd = c->n_kv_heads * c->head_dim;
   const int qkv[3] = {qd, kvd, kvd}, gu[2] = {c->intermediate, c->intermediate};
   const int o[1] = {c->hidden}, head[1] = {c->vocab};
   return w4::gemv_decode_applies(c->hidden, qkv, 3, false) && w4::gemv_decode_applies(c->hidden, gu, 2, true) &&
          w4::gemv_decode_applies(qd, o, 1, false) && w4::gemv_decode_applies(c->intermediate, o, 1, false) &&
-         w4::gemv_decode_applies(c->hidden, head, 1, false);
+         (dense_head ? w4::dense_rows_applies(1, c->hidden) : w4::gemv_decode_applies(c->hidden, head, 1, false));
 }
 
 int run_decode_fused(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, uint8_t* st,
@@ -328,7 +341,18 @@ int run_decode_fused(const w4a32_decoder_config* c, const w4a32_decoder_weights*
       delta_parts = 1;
     }
   }
-  {
+  if (w->lm_head_dense) {
+    // the reference's dense lm_head: residual add + final norm + the f16 / f32 rows in one launch, which also
+    // leaves one (max, first column) pair per wavefront where the pairs fit
+    const int parts = w4::dense_rows_partials(c->vocab);
+    float* amax_val = reinterpret_cast<float*>(scratch + sg.amax_val_off);
+    int* amax_idx = reinterpret_cast<int*>(scratch + sg.amax_idx_off);
+    const bool pairs = parts <= kArgmaxParts;
+    W4_TRY(from_hip(w4::launch_dense_head(hcur, delta, delta_parts, w->final_norm, c->rms_eps, w->lm_head_dense,
+                                          w->lm_head_dense_dtype, logits, c->vocab, H, pairs ? amax_val : nullptr,
+                                          pairs ? amax_idx : nullptr, s)));
+    if (pairs) return from_hip(w4::launch_argmax_parts(amax_val, amax_idx, parts, d_token_out, d_pos, s));
+  } else {
     const uint8_t* pk[1] = {static_cast<const uint8_t*>(w->lm_head)};
     float* ys[1] = {logits};
     const int ns[1] = {c->vocab};
@@ -634,6 +658,7 @@ int w4a32_decoder_prefill(const w4a32_decoder_config* cfg, const w4a32_decoder_w
                           void* d_state, const int64_t* d_tokens, int n_tokens, int pos0,
                           int64_t* d_next_token, void* stream) {
   if (!config_ok(cfg) || !w || !w->layers || !d_state || !d_tokens || !d_next_token) return W4A32_EINVAL;
+  W4_TRY(head_ok(cfg, w));
   if (n_tokens <= 0 || n_tokens > cfg->max_batch_tokens) return W4A32_ESHAPE;
   if (pos0 < 0 || pos0 + n_tokens > cfg->max_seq) return W4A32_ESHAPE;
   const StateGeom g = state_geom(cfg);
@@ -650,9 +675,10 @@ int w4a32_decoder_prefill(const w4a32_decoder_config* cfg, const w4a32_decoder_w
 int w4a32_decoder_step(const w4a32_decoder_config* cfg, const w4a32_decoder_weights* w, void* d_state,
                        const int64_t* d_token_in, int64_t* d_token_out, void* stream) {
   if (!config_ok(cfg) || !w || !w->layers || !d_state || !d_token_in || !d_token_out) return W4A32_EINVAL;
+  W4_TRY(head_ok(cfg, w));
   const StateGeom g = state_geom(cfg);
   uint8_t* st = static_cast<uint8_t*>(d_state);
-  if (decode_fusable(cfg)) return run_decode_fused(cfg, w, st, g, d_token_in, d_token_out, stream);
+  if (decode_fusable(cfg, w->lm_head_dense != nullptr)) return run_decode_fused(cfg, w, st, g, d_token_in, d_token_out, stream);
   W4_TRY(from_hip(w4::launch_embedding(d_token_in, w->embedding, 1, cfg->hidden, cfg->vocab,
                                        reinterpret_cast<float*>(st + g.h_off), S(stream))));
   return run_layers(cfg, w, st, g, 1, d_token_out, true, stream);

@@ -112,9 +112,17 @@ __global__ __launch_bounds__(256) void dense_gemv_kernel(const float* __restrict
 // wavefronts owns a 64 x 64 tile of C, each wavefront a 32 x 32 quarter; A and B tiles of 16 k go through
 // LDS ([row][16 + 1] floats, the pad keeps the operand reads off one bank). A plain kernel for an operator
 // the decoder runner does not use: every row's logits of a prompt are computed, as the reference does.
+// B may be held as f16 (BT = _Float16): its elements widen to f32 exactly on the way into LDS.
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
 constexpr int kMmTile = 64, kMmK = 16, kMmLd = kMmK + 1;
-__global__ __launch_bounds__(256) void dense_gemm_kernel(const float* __restrict__ a, const float* __restrict__ b,
+__device__ __forceinline__ float4 load4_as_f32(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load4_as_f32(const _Float16* p) {
+  const h4_t h = *reinterpret_cast<const h4_t*>(p);
+  return make_float4((float)h[0], (float)h[1], (float)h[2], (float)h[3]);
+}
+template <typename BT>
+__global__ __launch_bounds__(256) void dense_gemm_kernel(const float* __restrict__ a, const BT* __restrict__ b,
                                                          float* __restrict__ c, int M, int N, int K) {
   __shared__ float s_a[kMmTile * kMmLd], s_b[kMmTile * kMmLd];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -123,13 +131,13 @@ __global__ __launch_bounds__(256) void dense_gemm_kernel(const float* __restrict
   // loader: thread t brings A[m0 + t/4][k0 + 4*(t%4) ..+3] and the same of B (K % 4 == 0)
   const int lr = threadIdx.x >> 2, lk = 4 * (threadIdx.x & 3);
   const float* ap = a + (size_t)(m0 + lr < M ? m0 + lr : M - 1) * K + lk;
-  const float* bp = b + (size_t)(n0 + lr < N ? n0 + lr : N - 1) * K + lk;
+  const BT* bp = b + (size_t)(n0 + lr < N ? n0 + lr : N - 1) * K + lk;
   v16f acc = {0};
   for (int k0 = 0; k0 < K; k0 += kMmK) {
     float4 av = make_float4(0, 0, 0, 0), bv = make_float4(0, 0, 0, 0);
     if (k0 + lk < K) {
       av = *reinterpret_cast<const float4*>(ap + k0);
-      bv = *reinterpret_cast<const float4*>(bp + k0);
+      bv = load4_as_f32(bp + k0);
     }
     __syncthreads();  // the previous step's reads are done
     s_a[lr * kMmLd + lk + 0] = av.x; s_a[lr * kMmLd + lk + 1] = av.y;
@@ -174,7 +182,22 @@ hipError_t launch_rope_rows(const float* x, float* y, const float* sin_t, const 
   return hipGetLastError();
 }
 
+hipError_t launch_matmul_nt(const float* a, const void* b, int b_dtype, float* c, int M, int N, int K,
+                            hipStream_t s) {
+  // few rows: a stream over B (f16 or f32), 16 lanes per row of B
+  if (dense_rows_applies(M, K)) return launch_dense_rows(a, K, b, b_dtype, c, M, N, K, s);
+  const dim3 tiles((N + kMmTile - 1) / kMmTile, (M + kMmTile - 1) / kMmTile);
+  if (b_dtype == W4A32_DENSE_F16) {
+    hipLaunchKernelGGL(dense_gemm_kernel<_Float16>, tiles, dim3(256), 0, s, a, static_cast<const _Float16*>(b), c, M,
+                       N, K);
+    return hipGetLastError();
+  }
+  if (b_dtype != W4A32_DENSE_F32) return hipErrorInvalidValue;
+  return launch_matmul_f32_nt(a, static_cast<const float*>(b), c, M, N, K, s);
+}
+
 hipError_t launch_matmul_f32_nt(const float* a, const float* b, float* c, int M, int N, int K, hipStream_t s) {
+  if (dense_rows_applies(M, K)) return launch_dense_rows(a, K, b, W4A32_DENSE_F32, c, M, N, K, s);
   if (M <= 8) {
     const dim3 grid((N + 4 * kGemvRows - 1) / (4 * kGemvRows));
 #define W4_DENSE_GEMV(MM) \
@@ -186,8 +209,8 @@ hipError_t launch_matmul_f32_nt(const float* a, const float* b, float* c, int M,
 #undef W4_DENSE_GEMV
     return hipGetLastError();
   }
-  hipLaunchKernelGGL(dense_gemm_kernel, dim3((N + kMmTile - 1) / kMmTile, (M + kMmTile - 1) / kMmTile), dim3(256),
-                     0, s, a, b, c, M, N, K);
+  hipLaunchKernelGGL(dense_gemm_kernel<float>, dim3((N + kMmTile - 1) / kMmTile, (M + kMmTile - 1) / kMmTile),
+                     dim3(256), 0, s, a, b, c, M, N, K);
   return hipGetLastError();
 }
 
@@ -235,6 +258,21 @@ int w4a32_op_matmul_f32_nt(const float* d_a, const float* d_b, float* d_c, int M
   if (K % 4 != 0) return W4A32_ESHAPE;
   if (!aligned16(d_a) || !aligned16(d_b)) return W4A32_EINVAL;
   return from_hip(w4::launch_matmul_f32_nt(d_a, d_b, d_c, M, N, K, S(stream)));
+}
+
+int w4a32_op_matmul_nt(const float* d_a, const void* d_b, int b_dtype, float* d_c, int M, int N, int K,
+                       void* stream) {
+  if (!d_a || !d_b || !d_c || M <= 0 || N <= 0 || K <= 0) return W4A32_EINVAL;
+  if (b_dtype != W4A32_DENSE_F32 && b_dtype != W4A32_DENSE_F16) return W4A32_EINVAL;
+  if (K % 4 != 0) return W4A32_ESHAPE;
+  if (!aligned16(d_a) || !aligned16(d_b)) return W4A32_EINVAL;
+  return from_hip(w4::launch_matmul_nt(d_a, d_b, b_dtype, d_c, M, N, K, S(stream)));
+}
+
+int w4a32_op_f16_to_f32(const void* d_in, float* d_out, size_t n, void* stream) {
+  if (!d_in || !d_out || n == 0) return W4A32_EINVAL;
+  if ((reinterpret_cast<uintptr_t>(d_in) & 1) != 0 || (reinterpret_cast<uintptr_t>(d_out) & 3) != 0) return W4A32_EINVAL;
+  return from_hip(w4::launch_f16_to_f32(d_in, d_out, n, S(stream)));
 }
 
 }  // extern "C"

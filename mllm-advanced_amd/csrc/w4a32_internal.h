@@ -123,6 +123,18 @@ hipError_t launch_mul(const float* a, const float* b, float* out, size_t n, hipS
 hipError_t launch_rope_rows(const float* x, float* y, const float* sin_t, const float* cos_t, int M, int H,
                             int D, int pos0, hipStream_t s);
 hipError_t launch_matmul_f32_nt(const float* a, const float* b, float* c, int M, int N, int K, hipStream_t s);
+// dense [N][K] operands held as f16 or f32 (b_dtype: W4A32_DENSE_*), w4a32_dense.hip
+hipError_t launch_matmul_nt(const float* a, const void* b, int b_dtype, float* c, int M, int N, int K, hipStream_t s);
+hipError_t launch_f16_to_f32(const void* in, float* out, size_t n, hipStream_t s);
+bool dense_rows_applies(int M, int K);  // M <= 8 rows against a streamed B
+int dense_rows_partials(int N);         // wavefronts (= partial argmax results) of such a launch at M = 1
+hipError_t launch_dense_rows(const float* x, int ldx, const void* b, int b_dtype, float* c, int M, int N, int K,
+                             hipStream_t s);
+// one decode row through a dense lm_head with the residual add (delta_parts partial rows, or none) and the
+// RMSNorm in front; optionally one (max, first column) pair per wavefront to amax_val / amax_idx
+hipError_t launch_dense_head(const float* h, const float* delta, int delta_parts, const float* norm_w, float eps,
+                             const void* b, int b_dtype, float* logits, int N, int K, float* amax_val,
+                             int* amax_idx, hipStream_t s);
 hipError_t launch_attention_decode(const float* q, float* kc, float* vc, float* out, int Hq, int Hkv,
                                    int max_seq, const int* d_pos0, int pos0, int nsplit, float* part,
                                    unsigned int* counters, const float* k_new, const float* v_new,

@@ -140,6 +140,21 @@ Tensor toDevice(const Tensor& host) {
   return d;
 }
 
+Tensor toDeviceF32(const Tensor& host) {
+  if (host.dtype() == kFp32) return toDevice(host);
+  if (host.dtype() != kFp16) {
+    MLLM_ERROR_EXIT(kError, "{}: expected an Fp32 or Fp16 parameter, got {}", host.name(), dataTypes2Str(host.dtype()));
+  }
+  Tensor half = toDevice(host);
+  Tensor d = Tensor::empty(host.shape(), kFp32, kHIP).alloc();
+  d.setName(host.name());
+  auto& hb = currentHipBackend();
+  const int rc = w4a32_op_f16_to_f32(half.ptr<void>(), d.ptr<float>(), host.numel(), hb.stream());
+  if (rc != W4A32_OK) { MLLM_ERROR_EXIT(kHipRuntimeError, "w4a32_op_f16_to_f32 failed: {}", w4a32_error_string(rc)); }
+  hb.synchronize();  // `half` is released on return
+  return d;
+}
+
 Tensor toHost(const Tensor& device) {
   MLLM_RT_ASSERT(device.device() == kHIP);
   Tensor h = Tensor::empty(device.shape(), device.dtype(), kCPU).alloc();

@@ -98,4 +98,9 @@ HipBackend& currentHipBackend();
 Tensor toDevice(const Tensor& host);
 Tensor toHost(const Tensor& device);
 
+// A host parameter as an f32 device tensor of the same shape: Fp32 is copied, Fp16 (how the reference's W4A32
+// quantizer configuration stores the RMSNorm weights, scripts/QuantCfg/ds_qwen2/1.5B-W4A32-KAI.json:33-42) is
+// widened on the device, exactly. Any other dtype exits.
+Tensor toDeviceF32(const Tensor& host);
+
 }  // namespace mllm::hip

@@ -36,8 +36,9 @@ HipRMSNormOp::HipRMSNormOp(const RMSNormOpCargo& cargo) : RMSNormOp(cargo) {}
 
 void HipRMSNormOp::load(const std::shared_ptr<ParameterLoader>& ploader) {
   RMSNormOp::load(ploader);
-  if (weight_.dtype() != kFp32) { MLLM_ERROR_EXIT(kError, "{}.weight must be f32", name()); }
-  if (weight_.device() != kHIP) weight_ = toDevice(weight_);
+  // Fp32, or Fp16 as the reference's W4A32 quantizer configuration stores it: widened once, here
+  if (weight_.device() != kHIP) weight_ = toDeviceF32(weight_);
+  if (weight_.dtype() != kFp32) { MLLM_ERROR_EXIT(kError, "{}.weight must be f32 or f16", name()); }
 }
 
 void HipRMSNormOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
@@ -164,16 +165,21 @@ HipMatMulOp::HipMatMulOp(const MatMulOpCargo& cargo) : MatMulOp(cargo) {}
 
 void HipMatMulOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
   wantF32OnHip(inputs[0], name(), "A");
-  wantF32OnHip(inputs[1], name(), "B (move a host parameter to the device once, with hip::toDevice)");
+  // B: f32, or f16 as the reference's quantizer stores lm_head (its elements widen exactly inside the kernel)
+  const auto& B = inputs[1];
+  if (B.device() != kHIP || (B.dtype() != kFp32 && B.dtype() != kFp16)) {
+    MLLM_ERROR_EXIT(kError, "{}: B must be an f32 or f16 tensor on the HIP device (move a host parameter there "
+                    "once, with hip::toDevice)", name());
+  }
   const auto bs = inputs[1].shape();
   if (cargo_.transpose_a || !cargo_.transpose_b || bs.size() != 2) {
     MLLM_ERROR_EXIT(kError, "{}: the HIP backend implements A [.., M, K] x B [N, K]^T (transpose_b) only", name());
   }
   const int N = bs[0], K = bs[1];
   const int M = static_cast<int>(inputs[0].numel() / static_cast<size_t>(K));
-  check(w4a32_op_matmul_f32_nt(inputs[0].ptr<float>(), inputs[1].ptr<float>(), outputs[0].ptr<float>(), M, N, K,
-                               currentHipBackend().stream()),
-        "w4a32_op_matmul_f32_nt");
+  check(w4a32_op_matmul_nt(inputs[0].ptr<float>(), B.ptr<void>(), B.dtype() == kFp16 ? W4A32_DENSE_F16 : W4A32_DENSE_F32,
+                           outputs[0].ptr<float>(), M, N, K, currentHipBackend().stream()),
+        "w4a32_op_matmul_nt");
 }
 
 // ---------------------------------------------------------------------------- element-wise
@@ -210,10 +216,11 @@ HipLLMEmbeddingTokenOp::HipLLMEmbeddingTokenOp(const LLMEmbeddingTokenOpCargo& c
 
 void HipLLMEmbeddingTokenOp::load(const std::shared_ptr<ParameterLoader>& ploader) {
   LLMEmbeddingTokenOp::load(ploader);
-  if (weight_.dtype() != kFp32 || weight_.numel() != static_cast<size_t>(cargo_.vocab_size) * cargo_.hidden_size) {
-    MLLM_ERROR_EXIT(kError, "{}.weight must be f32 [{}, {}]", name(), cargo_.vocab_size, cargo_.hidden_size);
+  if ((weight_.dtype() != kFp32 && weight_.dtype() != kFp16) ||
+      weight_.numel() != static_cast<size_t>(cargo_.vocab_size) * cargo_.hidden_size) {
+    MLLM_ERROR_EXIT(kError, "{}.weight must be f32 or f16 [{}, {}]", name(), cargo_.vocab_size, cargo_.hidden_size);
   }
-  if (weight_.device() != kHIP) weight_ = toDevice(weight_);
+  if (weight_.device() != kHIP) weight_ = toDeviceF32(weight_);
 }
 
 void HipLLMEmbeddingTokenOp::reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {

@@ -70,16 +70,17 @@ void HipLinearOp::load(const std::shared_ptr<ParameterLoader>& ploader) {
   void* stream = hb.stream();
   Tensor packed = Tensor::empty({static_cast<int32_t>(packed_bytes)}, kInt8, kHIP).alloc();
 
-  if (weight_.dtype() == kFp32 && weight_.shape().size() == 2 && weight_.shape()[0] == N &&
-      weight_.shape()[1] == K) {
-    Tensor w_dev = toDevice(weight_);
+  if ((weight_.dtype() == kFp32 || weight_.dtype() == kFp16) && weight_.shape().size() == 2 &&
+      weight_.shape()[0] == N && weight_.shape()[1] == K) {
+    // an unquantised weight (f32, or f16 widened exactly): quantised here, as the reference's offline pass would
+    Tensor w_dev = toDeviceF32(weight_);
     Tensor b_dev;
     if (cargo_.bias) {
-      if (bias_.dtype() != kFp32 || static_cast<int>(bias_.numel()) != N) {
-        MLLM_ERROR_EXIT(kError, "{}.bias must be f32 [{}]", name(), N);
+      if ((bias_.dtype() != kFp32 && bias_.dtype() != kFp16) || static_cast<int>(bias_.numel()) != N) {
+        MLLM_ERROR_EXIT(kError, "{}.bias must be f32 or f16 [{}]", name(), N);
         return;
       }
-      b_dev = toDevice(bias_);
+      b_dev = toDeviceF32(bias_);
     }
     const size_t tmp_bytes = w4a32_native_u4_bytes(N, K) + w4a32_native_scale_bytes(N, K);
     Tensor tmp = Tensor::empty({static_cast<int32_t>(tmp_bytes)}, kInt8, kHIP).alloc();
@@ -117,7 +118,7 @@ void HipLinearOp::load(const std::shared_ptr<ParameterLoader>& ploader) {
     check(w4a32_repack_native(u4, sc, bias, N, K, packed.ptr<void>(), stream), "w4a32_repack_native");
     hb.synchronize();
   } else {
-    MLLM_ERROR_EXIT(kError, "{}.weight: expected f32 [{},{}] or an int8 W4 blob of {} bytes, "
+    MLLM_ERROR_EXIT(kError, "{}.weight: expected f32 / f16 [{},{}] or an int8 W4 blob of {} bytes, "
                     "got {} with {} elements", name(), N, K, nativeBlobBytes(N, K),
                     dataTypes2Str(weight_.dtype()), weight_.numel());
     return;

@@ -64,12 +64,13 @@ void HipQWenForCausalLM::load(const std::shared_ptr<ParameterLoader>& ploader) {
     return op->weight().ptr<void>();
   };
   auto f32 = [&](const std::string& name, size_t numel) -> const float* {
+    // Fp32, or Fp16 (the dtype the reference's W4A32 quantizer configuration gives the norm weights), widened once
     Tensor host((*ploader)[name]);
-    if (host.dtype() != kFp32 || host.numel() != numel) {
-      MLLM_ERROR_EXIT(kError, "{}: expected {} f32 values, got {} x {}", name, numel,
+    if ((host.dtype() != kFp32 && host.dtype() != kFp16) || host.numel() != numel) {
+      MLLM_ERROR_EXIT(kError, "{}: expected {} f32 or f16 values, got {} x {}", name, numel,
                       dataTypes2Str(host.dtype()), host.numel());
     }
-    Tensor dev = hip::toDevice(host);
+    Tensor dev = hip::toDeviceF32(host);
     f32_params_.push_back(dev);
     return dev.ptr<float>();
   };
@@ -90,7 +91,22 @@ void HipQWenForCausalLM::load(const std::shared_ptr<ParameterLoader>& ploader) {
   }
   weights_.embedding = f32("model.embed_tokens.weight", (size_t)cfg_.vocab_size * H);
   weights_.final_norm = f32("model.norm.weight", H);
-  weights_.lm_head = linear("lm_head", H, cfg_.vocab_size, false);
+  {
+    Tensor head((*ploader)["lm_head.weight"]);
+    const bool unquantised = head.dtype() == kFp32 || head.dtype() == kFp16;
+    if (unquantised && !cfg_.lm_head_w4a32) {
+      // the reference's form: x [S, D] times lm_head [V, D] transposed, on the tensor as the file holds it
+      if (head.numel() != (size_t)cfg_.vocab_size * H) {
+        MLLM_ERROR_EXIT(kError, "lm_head.weight: expected [{}, {}], got {} elements", cfg_.vocab_size, H, head.numel());
+      }
+      lm_head_dense_ = hip::toDevice(head);
+      weights_.lm_head = nullptr;
+      weights_.lm_head_dense = lm_head_dense_.ptr<void>();
+      weights_.lm_head_dense_dtype = head.dtype() == kFp16 ? W4A32_DENSE_F16 : W4A32_DENSE_F32;
+    } else {
+      weights_.lm_head = linear("lm_head", H, cfg_.vocab_size, false);
+    }
+  }
   weights_.layers = layer_weights_.data();
 
   const size_t bytes = w4a32_decoder_state_bytes(&dcfg_);

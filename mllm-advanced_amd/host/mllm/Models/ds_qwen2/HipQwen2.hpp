@@ -10,9 +10,13 @@
 //   model.layers.<i>.post_attention_layernorm.weight
 //   model.layers.<i>.mlp.{gate,up,down}_proj.weight
 //   model.norm.weight, lm_head.weight
-// Linear weights may be f32 [out, in] (quantised on load) or this build's int8 W4 file blob, as
-// HipLinearOp::load accepts them. lm_head is loaded like any other Linear: the reference multiplies
-// by a dense f32 lm_head (modeling_ds_qwen2.hpp:209-213), this model quantises it to W4A32.
+// Linear weights may be f32 / f16 [out, in] (quantised on load), this build's int8 W4 file blob or the Arm
+// quantizer's blob, as HipLinearOp::load accepts them. The norm weights and the embedding may be Fp32 or Fp16
+// (widened once at load). lm_head.weight is applied as the reference applies it, a dense matmul with
+// transpose_b (modeling_ds_qwen2.hpp:209-213), on the tensor as the file holds it: Fp16 [vocab, hidden] (what
+// the reference's W4A32 quantizer configuration writes, scripts/QuantCfg/ds_qwen2/1.5B-W4A32-KAI.json:33-45)
+// or Fp32. With HipQWenConfig::lm_head_w4a32 it is quantised to a W4A32 Linear instead (the benchmark's
+// lm_head shape); an int8 W4 blob under that name is always a W4A32 Linear.
 #pragma once
 
 #include <cstdint>
@@ -45,6 +49,7 @@ struct HipQWenConfig {
   LinearOpImplType linear_impl_type =
       LinearOpImplType::kKaiLinear_f32_qai8dxp_qsi4c32p_mxk_nxk_qai8dxp4x8_qsi4c32p4x8_8x4x32;
   int32_t max_prompt_chunk = 512;  // longest prompt slice one prefill call takes (not in the reference)
+  bool lm_head_w4a32 = false;      // quantise an Fp32 / Fp16 lm_head to W4A32 instead of the dense matmul (not in the reference)
 };
 
 class HipQWenForCausalLM {
@@ -75,6 +80,7 @@ class HipQWenForCausalLM {
   w4a32_decoder_config dcfg_{};
   std::vector<std::shared_ptr<hip::HipLinearOp>> linears_;  // keep the device blobs alive
   std::vector<Tensor> f32_params_;
+  Tensor lm_head_dense_;  // [vocab, hidden] f16 or f32 on the device, when lm_head is applied densely
   std::vector<w4a32_layer_weights> layer_weights_;
   w4a32_decoder_weights weights_{};
   Tensor state_, token_;

@@ -119,9 +119,16 @@ struct OpByOpModel {
       reg(OpType::kSiLU, SiLUOpCargo{}, b + "mlp.act", p);
     }
     norm("model.norm");
-    // the runner applies a W4A32 lm_head; so does this model, so that the two can be compared token by token
-    linear("lm_head", c.hidden_size, c.vocab_size, false);
+    if (c.lm_head_w4a32) {
+      // the runner was asked for a W4A32 lm_head; so does this model, so that the two can be compared token by token
+      linear("lm_head", c.hidden_size, c.vocab_size, false);
+    } else {
+      // the reference's form (modeling_ds_qwen2.hpp:209-213): the parameter itself, f32 or f16, moved to the
+      // device once, then x [1, S, D] times lm_head [V, D] transposed
+      lm_head = hip::toDevice(Tensor((*p)["lm_head.weight"]));
+    }
   }
+  Tensor lm_head;
 
   // QWenForCausalLM::forward: ids [1, S] on the host -> logits [1, S, V] on the device
   Tensor forward(const std::vector<int64_t>& ids) {
@@ -155,7 +162,10 @@ struct OpByOpModel {
       x = ctx.dispatch(OpType::kAdd, AddOpCargo{}, {g, tmp})[0];
     }
     x = ctx.dispatch("model.norm", {x})[0];
-    return ctx.dispatch("lm_head", {x})[0];
+    if (lm_head.isNil()) return ctx.dispatch("lm_head", {x})[0];
+    MatMulOpCargo mm;
+    mm.transpose_b = true;
+    return ctx.dispatch(OpType::kMatMul, mm, {x, lm_head})[0];
   }
 };
 
@@ -280,6 +290,7 @@ int main(int argc, char** argv) {
     cfg.max_cache_length = 1024;
     cfg.rope_theta = 1e6f;
     cfg.eos_token_id = -1;
+    cfg.lm_head_w4a32 = true;  // the benchmark's lm_head (a dense f32 one would add 933 MB per token to both sides)
     distinct = 7;
   } else {
     cfg.num_attention_heads = 2;

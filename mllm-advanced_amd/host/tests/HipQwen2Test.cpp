@@ -5,6 +5,10 @@
 // operators on all rows) predicts, and generation must be reproducible. The Python test that runs
 // this binary reads the same file and compares the printed tokens with the CPU oracle's.
 // Needs a GPU. Usage: hip_qwen2_test <directory>
+//        hip_qwen2_test <directory> --load <file.mllm>   loads that file instead (same tiny configuration),
+//            generates, prints the tokens and writes the last step's logits to <file.mllm>.logits (raw f32):
+//            for the Python test that writes one model twice, once with the dtypes of the reference's W4A32
+//            quantizer configuration (Fp16 norm weights and lm_head, int8 W4 blobs) and once all in f32
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -55,6 +59,29 @@ int main(int argc, char** argv) {
   cfg.rope_theta = 1e6f;
   cfg.eos_token_id = -1;  // never produced: generation runs to max_length
   cfg.max_prompt_chunk = 8;  // the 11-token prompt below goes in as two slices
+
+  const bool load_only = argc > 3 && std::string(argv[2]) == "--load";
+  if (load_only) {
+    std::printf("[ RUN      ] load %s, generate\n", argv[3]);
+    auto file = load(argv[3]);
+    models::HipQWenForCausalLM m(cfg);
+    m.load(file);
+    const std::vector<int64_t> prompt = {3, 17, 100, 42, 7, 250, 611, 5, 98, 301, 77};
+    std::vector<int64_t> gen = m.generate(prompt, 24);
+    std::printf("TOKENS:");
+    for (auto t : gen) std::printf(" %lld", (long long)t);
+    std::printf("\n");
+    const std::vector<float> logits = m.lastLogits();
+    const std::string out = std::string(argv[3]) + ".logits";
+    std::FILE* f = std::fopen(out.c_str(), "wb");
+    EXPECT(f != nullptr);
+    if (f) {
+      EXPECT(std::fwrite(logits.data(), sizeof(float), logits.size(), f) == logits.size());
+      std::fclose(f);
+    }
+    std::printf(g_failed ? "[  FAILED  ]\n" : "[ PASSED ]\n");
+    return g_failed ? 1 : 0;
+  }
 
   // ---- write the model file under the reference's parameter names
   std::printf("[ RUN      ] write + load .mllm\n");

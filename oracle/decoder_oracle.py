@@ -15,8 +15,9 @@ Follows (reference tree):
 
 Every operator here is a textbook routine in float32 numpy; the parity tests compare the HIP
 operators one by one against torch's own float32 operators as well. Linears go through the scalar
-oracle (w4a32_oracle.linear), lm_head included (the reference multiplies by a dense lm_head; the
-benchmark configuration quantises it like the other Linears).
+oracle (w4a32_oracle.linear). lm_head is either quantised like the other Linears (the benchmark
+configuration) or, with lm_head_dense=True, applied as the reference applies it: a dense matmul with
+transpose_b on the f32 / f16 tensor (modeling_ds_qwen2.hpp:209-213), here numpy's float64 product.
 """
 import numpy as np
 
@@ -91,7 +92,8 @@ class Decoder:
     """weights: dict with embedding [V][H], final_norm [H], lm_head [V][H] and layers = list of dicts
     (q,k,v,o,gate,up,down f32 [out][in]; q_bias,k_bias,v_bias optional; attn_norm, ffn_norm)."""
 
-    def __init__(self, weights, n_heads, n_kv_heads, head_dim=128, rope_theta=1e6, rms_eps=1e-6, max_seq=1024):
+    def __init__(self, weights, n_heads, n_kv_heads, head_dim=128, rope_theta=1e6, rms_eps=1e-6, max_seq=1024,
+                 lm_head_dense=False):
         self.w = weights
         self.Hq, self.Hkv, self.D = n_heads, n_kv_heads, head_dim
         self.eps = rms_eps
@@ -104,7 +106,11 @@ class Decoder:
                 "gate": Linear(lw["gate"]), "up": Linear(lw["up"]), "down": Linear(lw["down"]),
                 "attn_norm": lw["attn_norm"], "ffn_norm": lw["ffn_norm"],
             })
-        self.lm_head = Linear(weights["lm_head"])
+        if lm_head_dense:
+            dense = np.asarray(weights["lm_head"]).astype(np.float64)   # f16 or f32 values, widened exactly
+            self.lm_head = lambda x: (x.astype(np.float64) @ dense.T).astype(F)
+        else:
+            self.lm_head = Linear(weights["lm_head"])
         self.kc = [np.zeros((n_kv_heads, max_seq, head_dim), dtype=F) for _ in self.layers]
         self.vc = [np.zeros((n_kv_heads, max_seq, head_dim), dtype=F) for _ in self.layers]
         self.pos = 0
