@@ -35,6 +35,7 @@
 // the same f32 expression in the same order as on the dot4 path. The instruction count per chunk
 // no longer grows with M (M = 8: 130 -> 45 per wavefront).
 #include <algorithm>
+#include <cstdlib>
 
 #include "w4a32_internal.h"
 #include "w4a32_quant_math.h"
@@ -48,8 +49,8 @@ constexpr bool decode_mfma(int M) { return M >= kDecodeMfmaMinM; }
 // rows 4g..4g+3 of column j
 constexpr int decode_acc(int M) { return decode_mfma(M) ? 4 : M; }
 
-// One scale block (tile dword wv, scale sv) against the M int8 rows at a_base (+ m * Kp); a_base
-// already points at this lane's k-group.
+// One scale block (tile dword wv, scale sv) against the M int8 rows at a_base (+ m * Kp, the row stride of
+// the caller's layout); a_base already points at this lane's k-group.
 template <int M>
 __device__ __forceinline__ void block_products(uint32_t wv, float sv, const int8_t* a_base, int Kp,
                                                int j, float (&acc)[decode_acc(M)]) {
@@ -609,6 +610,294 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
   }
 }
 
+// Several decode rows (M >= kBatchedMinM) through 1..kMaxGroup Linears that share them: the whole op in one
+// launch, like gemv_fused_kernel, with the rows' quantisation shared by more weights. With one tile row per
+// workgroup every workgroup loads and quantises all M rows for 14 KB of weights (K = 1536): at M = 8 the row
+// reads of a gate,up launch (560 workgroups x 48 KB from L2) exceed its weight bytes, and a thread quantises 48
+// values before its first product. Here a workgroup is kWaves wavefronts: all of them load and quantise the
+// rows ((row, 64 groups of 8) segments dealt to wavefronts), then every Wt of them take one tile row exactly as
+// a workgroup of gemv_fused_kernel does (wavefront wl of a tile row holds chunks wl, wl + Wt, ...; same f32
+// expression per output in the same order, so the results are bit-identical). Tile rows are numbered through
+// the Linears of the group (ga.first). Eight wavefronts (two tile rows at K = 1536) measured best: gate,up at
+// M = 8 13.8 -> 10.3 us, q,k,v 6.5 -> 5.1; sixteen cost more than they save (11.8 / 6.0).
+//
+// kR = 0: the rows arrive quantised (workspace of w4a32_quant_lhs: aq [M][K], recip, negzp) and are only
+// copied into LDS; this form serves a long K (down_proj), whose f32 rows are too many to quantise per workgroup.
+//
+// The int8 rows lie in LDS as [32-k block][row][32 bytes]: the M rows of a block behind each other, so the 64
+// lanes of a product's operand read (row lane % 16, 8 bytes at 8 * (lane / 16)) cover one contiguous M * 32
+// bytes. As [row][Kp], with Kp a multiple of 256 bytes, every row of a block starts in the same LDS bank
+// (q,k,v at M = 8: 7.6 against 6.1 us).
+constexpr int kBatchedMinM = 3;
+constexpr int kBatchedStageMax = 10;  // 16-byte units of quantised rows a thread copies (kR = 0)
+
+// min and max of kR independent pairs across the wavefront, totals in lane 63: the chains of the pairs are
+// interleaved, so each DPP read finds its register at least two issue slots after its write without a wait.
+#define W4_MM2(c) \
+  "v_min_f32_dpp %0, %0, %0 " c "\n\tv_max_f32_dpp %1, %1, %1 " c "\n\t" \
+  "v_min_f32_dpp %2, %2, %2 " c "\n\tv_max_f32_dpp %3, %3, %3 " c "\n\t"
+#define W4_MM3(c) W4_MM2(c) "v_min_f32_dpp %4, %4, %4 " c "\n\tv_max_f32_dpp %5, %5, %5 " c "\n\t"
+#define W4_MM_STEPS(S)                                                                         \
+  "s_nop 1\n\t" S("quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf")                            \
+  S("quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf") S("row_half_mirror row_mask:0xf bank_mask:0xf") \
+  S("row_mirror row_mask:0xf bank_mask:0xf") S("row_bcast:15 row_mask:0xa bank_mask:0xf")      \
+  S("row_bcast:31 row_mask:0xc bank_mask:0xf") "s_nop 1"
+template <int kR>
+__device__ __forceinline__ void wave_minmax_pairs(float (&lo)[kR], float (&hi)[kR]) {
+  if constexpr (kR >= 3) {
+#pragma unroll
+    for (int b = 0; b + 3 <= kR; b += 3) {
+      asm volatile(W4_MM_STEPS(W4_MM3)
+                   : "+v"(lo[b]), "+v"(hi[b]), "+v"(lo[b + 1]), "+v"(hi[b + 1]), "+v"(lo[b + 2]), "+v"(hi[b + 2]));
+    }
+  }
+  constexpr int kDone = kR / 3 * 3;
+  if constexpr (kR - kDone == 2) {
+    asm volatile(W4_MM_STEPS(W4_MM2) : "+v"(lo[kDone]), "+v"(hi[kDone]), "+v"(lo[kDone + 1]), "+v"(hi[kDone + 1]));
+  } else if constexpr (kR - kDone == 1) {
+    wave_minmax_pair(lo[kDone], hi[kDone]);
+  }
+}
+#undef W4_MM_STEPS
+#undef W4_MM3
+#undef W4_MM2
+
+// min and max within every 8 consecutive lanes; all 8 end up with the totals
+__device__ __forceinline__ void octet_minmax_pair(float& lo, float& hi) {
+  asm volatile(
+      "s_nop 1\n\t"
+      "v_min_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 0\n\t"
+      "v_min_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 0\n\t"
+      "v_min_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 1"
+      : "+v"(lo), "+v"(hi));
+}
+
+// The row quantiser of the kernels that serve several rows, on (row, segment of 64 groups of 8) tasks dealt to
+// the workgroup's kWaves wavefronts: wavefront w owns tasks w, w + kWaves, ... (kR of them; xv[r] holds lane's
+// group of task r, loaded by load_row_tasks). Ranges of the segments (all chains of a wavefront interleaved),
+// a barrier, then the ranges and parameters of all M rows at once: lanes 8 m .. 8 m + 7 hold row m's segment
+// ranges (at most 8 segments: K <= 4096), reduce them and compute the row's parameters with the standalone
+// quantiser's arithmetic; a task reads its row's from lane 8 m. The int8 rows go to s_a in the
+// [32-k block][row][32 bytes] layout, recip / -zp of the rows to s_par ([M] f32, [M] i32). The caller
+// synchronises afterwards.
+template <int M, int kR>
+__device__ __forceinline__ void load_row_tasks(const float* __restrict__ x, int ldx, int K, int Kp, int kWaves,
+                                               int wave, int lane, float (&xv)[kR][8]) {
+  const int grp_per_row = Kp >> 3, groups = K >> 3;
+  const int nseg = (grp_per_row + 63) >> 6, ntask = M * nseg;
+#pragma unroll
+  for (int r = 0; r < kR; ++r) {
+    const int t = wave + r * kWaves;
+    const int tt = t < ntask ? t : ntask - 1;     // a wavefront without a task repeats the last one (not stored)
+    const int m = tt / nseg, c = (tt - m * nseg) * 64 + lane;
+    const int cc = c < groups ? c : groups - 1;   // a duplicate of a real element: harmless for min / max
+    const float* row = x + (size_t)m * ldx + 8 * cc;
+    const float4 v0 = *reinterpret_cast<const float4*>(row);
+    const float4 v1 = *reinterpret_cast<const float4*>(row + 4);
+    const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) xv[r][e] = f[e];
+  }
+}
+template <int M, int kR, int kWaves>
+__device__ __forceinline__ void quantise_row_tasks(const float (&xv)[kR][8], int K, int Kp, int8_t* s_a,
+                                                   float2* s_mm, float* s_par, int wave, int lane) {
+  const int grp_per_row = Kp >> 3, groups = K >> 3;
+  const int nseg = (grp_per_row + 63) >> 6, ntask = M * nseg;
+  float lo[kR], hi[kR];
+#pragma unroll
+  for (int r = 0; r < kR; ++r) {
+    lo[r] = xv[r][0];
+    hi[r] = xv[r][0];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      lo[r] = fminf(lo[r], xv[r][e]);
+      hi[r] = fmaxf(hi[r], xv[r][e]);
+    }
+  }
+  wave_minmax_pairs<kR>(lo, hi);
+#pragma unroll
+  for (int r = 0; r < kR; ++r) {
+    const int t = wave + r * kWaves;
+    if (lane == 63 && t < ntask) s_mm[t] = make_float2(lo[r], hi[r]);
+  }
+  __syncthreads();
+  const int pm = (lane >> 3) < M ? (lane >> 3) : M - 1, ps = (lane & 7) < nseg ? (lane & 7) : nseg - 1;
+  float2 v = s_mm[pm * nseg + ps];
+  octet_minmax_pair(v.x, v.y);
+  const RowQuant par = row_quant_params(v.x, v.y);
+  if (wave == 0 && (lane & 7) == 0 && (lane >> 3) < M) {
+    s_par[lane >> 3] = par.recip;
+    reinterpret_cast<int*>(s_par)[M + (lane >> 3)] = -par.zp;
+  }
+#pragma unroll
+  for (int r = 0; r < kR; ++r) {
+    const int t = wave + r * kWaves;
+    if (t < ntask) {  // wavefront-uniform
+      const int m = t / nseg, c = (t - m * nseg) * 64 + lane;
+      RowQuant pr;
+      pr.scale = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(par.scale), 8 * m));
+      pr.recip = 0.0f;  // not used by the quantiser
+      pr.zp = __builtin_amdgcn_readlane(par.zp, 8 * m);
+      if (c < grp_per_row) {
+        uint2 out = quant_group8(xv[r], pr);
+        if (c >= groups) out = make_uint2(0, 0);   // the tile padding, k >= K
+        *reinterpret_cast<uint2*>(s_a + ((size_t)(c >> 2) * M + m) * kBlockLen + 8 * (c & 3)) = out;
+      }
+    }
+  }
+}
+
+template <int M, int kCPW, int kR, int kWaves>
+__global__ __launch_bounds__(64 * kWaves) void gemv_batched_kernel(
+    const float* __restrict__ x, int ldx, const int8_t* __restrict__ aq, const float* __restrict__ recip,
+    const int32_t* __restrict__ negzp, int K, int KC, int Wt, const GroupArgs ga) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  constexpr bool kPreq = kR == 0;
+  constexpr int kTasks = kPreq ? 1 : kR;
+  const int Kp = KC * kTileK;
+  const int grp_per_row = Kp >> 3, groups = K >> 3;
+  const int nseg = (grp_per_row + 63) >> 6;       // 64-group segments per row (at most 8 when quantising here)
+  const int ntask = M * nseg;
+  int8_t* s_a = reinterpret_cast<int8_t*>(smem);                               // [Kp / 32][M][32]
+  float* s_red = reinterpret_cast<float*>(smem + (size_t)M * Kp);               // [kWaves][M][16]
+  float2* s_mm = reinterpret_cast<float2*>(s_red + kWaves * M * 16);            // [ntask] (min, max)
+  float* s_par = reinterpret_cast<float*>(s_mm + (kPreq ? 0 : ntask));          // [M] recip, [M] -zp
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int g = lane >> 4, j = lane & 15;
+  const int T = kWaves / Wt;                      // tile rows per workgroup
+  const int tg = wave / Wt, wl = wave - tg * Wt;  // this wavefront's tile row and its place in it
+  const int total = ga.first[ga.count];
+
+  // the rows first (a few KB, normally in L2), then the weights: loads return in issue order
+  float xv[kTasks][8];
+  uint4 staged[kPreq ? kBatchedStageMax : 1];
+  const int units_per_row = Kp >> 4, units = M * units_per_row;
+  if constexpr (kPreq) {
+#pragma unroll
+    for (int r = 0; r < kBatchedStageMax; ++r) {
+      const int u = threadIdx.x + r * 64 * kWaves;
+      staged[r] = make_uint4(0, 0, 0, 0);
+      if (u < units) {
+        const int m = u / units_per_row, c = u - m * units_per_row;
+        if (16 * c < K) staged[r] = *reinterpret_cast<const uint4*>(aq + (size_t)m * K + 16 * c);
+      }
+    }
+    if (threadIdx.x < M) {
+      s_par[threadIdx.x] = recip[threadIdx.x];
+      reinterpret_cast<int*>(s_par)[M + threadIdx.x] = negzp[threadIdx.x];
+    }
+  } else {
+    load_row_tasks<M, kTasks>(x, ldx, K, Kp, kWaves, wave, lane, xv);
+  }
+  // which Linear this wavefront's tile row belongs to
+  const int gt = (int)blockIdx.x * T + tg;
+  const uint8_t* packed = ga.packed[0];
+  int nt_first = 0;
+#pragma unroll
+  for (int i = 1; i < kMaxGroup; ++i) {
+    if (i < ga.count && gt >= ga.first[i]) {
+      packed = ga.packed[i];
+      nt_first = ga.first[i];
+    }
+  }
+  const int nt = gt < total ? gt - nt_first : 0;   // a wavefront past the last tile row repeats one (not stored)
+  const uint8_t* tiles = packed + (size_t)nt * KC * kTileBytes;
+  u32x4 wq[kCPW];
+  u32x2 sc[kCPW];
+#pragma unroll
+  for (int i = 0; i < kCPW; ++i) {
+    const int kc = wl + i * Wt < KC ? wl + i * Wt : KC - 1;  // masked where used
+    wq[i] = load_global<u32x4>(tiles + (size_t)kc * kTileBytes + 16 * lane);
+    sc[i] = load_global<u32x2>(tiles + (size_t)kc * kTileBytes + kTileQBytes + 8 * j);
+  }
+  // Output (tile row `to` of the workgroup, row m, column jj) belongs to thread (to * M + m) * 16 + jj; its
+  // rsum / bias are requested now.
+  const int outputs = T * M * 16;
+  float rs = 0.0f, bs = 0.0f, *oy = nullptr;
+  int on = 0, oN = 0;
+  bool owns = false;
+  {
+    const int o = threadIdx.x;
+    const int to = o / (M * 16), ogt = (int)blockIdx.x * T + to;
+    if (o < outputs && ogt < total) {
+      const uint8_t* opk = ga.packed[0];
+      int ofirst = 0;
+      oN = ga.N[0];
+      oy = ga.y[0];
+#pragma unroll
+      for (int i = 1; i < kMaxGroup; ++i) {
+        if (i < ga.count && ogt >= ga.first[i]) {
+          opk = ga.packed[i];
+          oN = ga.N[i];
+          oy = ga.y[i];
+          ofirst = ga.first[i];
+        }
+      }
+      const int oNT = (oN + kTileRows - 1) / kTileRows;
+      on = kTileRows * (ogt - ofirst) + (o & 15);
+      owns = on < oN;
+      if (owns) {
+        const float* rsp = reinterpret_cast<const float*>(opk + (size_t)oNT * KC * kTileBytes);
+        rs = load_global<float>(rsp + on);
+        bs = load_global<float>(rsp + oNT * kTileRows + on);
+      }
+    }
+  }
+
+  if constexpr (kPreq) {
+#pragma unroll
+    for (int r = 0; r < kBatchedStageMax; ++r) {
+      const int u = threadIdx.x + r * 64 * kWaves;
+      if (u < units) {
+        const int m = u / units_per_row, c = u - m * units_per_row;
+        *reinterpret_cast<uint4*>(s_a + ((size_t)(c >> 1) * M + m) * kBlockLen + 16 * (c & 1)) = staged[r];
+      }
+    }
+  } else {
+    quantise_row_tasks<M, kTasks, kWaves>(xv, K, Kp, s_a, s_mm, s_par, wave, lane);
+  }
+  __syncthreads();
+
+  float acc[decode_acc(M)];
+#pragma unroll
+  for (int m = 0; m < decode_acc(M); ++m) acc[m] = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kCPW; ++i) {
+    const bool valid = wl + i * Wt < KC;
+    const int kc = valid ? wl + i * Wt : KC - 1;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const int8_t* a_base = s_a + (size_t)(4 * kc + d) * (M * kBlockLen) + 8 * g;
+      const uint32_t sw = sc[i][d >> 1];
+      const uint32_t sbits = valid ? ((d & 1) ? (sw & 0xFFFF0000u) : (sw << 16)) : 0u;
+      block_products<M>(wq[i][d], __uint_as_float(sbits), a_base, kBlockLen, j, acc);
+    }
+  }
+  store_row_sums<M>(acc, s_red + wave * M * 16, lane);
+  __syncthreads();
+
+  //   y = (sum/16 + off * rsum[n]) * lhs_scale + bias[n], clamped to the finite f32 range
+  if (owns) {
+    const int o = threadIdx.x;
+    const int to = o / (M * 16), rem = o - to * (M * 16), m = rem >> 4;
+    float sum = 0.0f;
+    for (int w = 0; w < Wt; ++w) sum += s_red[(to * Wt + w) * (M * 16) + rem];
+    const float rcp = s_par[m];
+    const int off = reinterpret_cast<const int*>(s_par)[M + m];
+    float v = __fmaf_rn((float)off, rs, sum * 0.0625f);
+    v = __fmaf_rn(v, rcp, bs);
+    v = fminf(fmaxf(v, -3.402823466e+38f), 3.402823466e+38f);
+    *(W4_GLOBAL float*)(oy + (size_t)m * oN + on) = v;
+  }
+}
+
 // One decode row through ONE Linear with a long K, the k range dealt to kDecodeParts workgroups per tile row
 // (down_proj: 96 tile rows would otherwise occupy 96 of 256 CUs with 14 wavefronts each). Workgroup
 // (part p, tile row nt) quantises the row as gemv_fused_kernel does (the range needs the whole row; only
@@ -925,6 +1214,95 @@ static hipError_t launch_fused_m(const GroupArgs& ga, const float* x, int ldx, i
   return hipGetLastError();
 }
 
+// Launch shape of gemv_batched_kernel: `waves` wavefronts per workgroup, Wt of them per tile row (a divisor of
+// waves), each holding CPW chunks; a wavefront owns R (row, segment) quantisation tasks (R = 0: the rows arrive
+// quantised).
+struct BatchedPlan {
+  int waves, Wt, CPW, R;
+};
+static int batched_env(const char* name, int dflt) {
+  const char* e = getenv(name);
+  return e ? atoi(e) : dflt;
+}
+// whole op: the kernel quantises the rows itself
+static BatchedPlan batched_plan(int M, int K) {
+  const BatchedPlan none{0, 0, 0, 0};
+  static const int off = batched_env("W4A32_BATCHED_OFF", 0);
+  if (off || M < kBatchedMinM || M > kGemvMaxM) return none;
+  const int KC = (K + kTileK - 1) / kTileK;
+  const int nseg = (KC * (kTileK / 8) + 63) / 64;
+  if (nseg > 8) return none;                        // a row's segment ranges meet in one 8-lane reduction
+  const int waves = 8;
+  const int R = (M * nseg + waves - 1) / waves;
+  if (R > 3) return none;
+  for (int Wt = 1; Wt <= waves; Wt *= 2) {
+    const int cpw = (KC + Wt - 1) / Wt;
+    if (cpw <= 3) return BatchedPlan{waves, Wt, cpw, R};  // about three chunks per wavefront, as in gemv_fused_kernel
+  }
+  return none;
+}
+// rows already quantised
+static BatchedPlan batched_preq_plan(int M, int K) {
+  const BatchedPlan none{0, 0, 0, 0};
+  static const int off = batched_env("W4A32_BATCHED_PREQ_OFF", 0);
+  if (off || M < kBatchedMinM || M > kGemvMaxM) return none;
+  const int KC = (K + kTileK - 1) / kTileK;
+  const int waves = KC > 24 ? 16 : 8, cpw_max = KC > 24 ? 5 : 3;
+  if ((M * KC * (kTileK / 16) + 64 * waves - 1) / (64 * waves) > kBatchedStageMax) return none;
+  if ((size_t)M * KC * kTileK > 150 * 1024) return none;
+  for (int Wt = 1; Wt <= waves; Wt *= 2) {
+    const int cpw = (KC + Wt - 1) / Wt;
+    if (cpw <= cpw_max) return BatchedPlan{waves, Wt, cpw, 0};
+  }
+  return none;
+}
+
+template <int M, int kWaves, int kCPW, int kR>
+static hipError_t launch_batched_k(const GroupArgs& ga, const float* x, int ldx, const uint8_t* ws, int K,
+                                   const BatchedPlan& p, hipStream_t s) {
+  const int KC = (K + kTileK - 1) / kTileK, Kp = KC * kTileK;
+  const int nseg = (Kp / 8 + 63) / 64;
+  const int T = kWaves / p.Wt;
+  const size_t lds = (size_t)M * Kp + (size_t)kWaves * M * 16 * sizeof(float) +
+                     (kR ? (size_t)M * nseg * sizeof(float2) : 0) + (size_t)2 * M * sizeof(float);
+  const dim3 grid((ga.first[ga.count] + T - 1) / T), block(64 * kWaves);
+  const WsGeom w = ws_geom(M, K);
+  auto kern = gemv_batched_kernel<M, kCPW, kR, kWaves>;
+  static LdsLimitOnce raised;
+  if (hipError_t e = raise_lds_limit(kern, lds, &raised); e != hipSuccess) return e;
+  hipLaunchKernelGGL(kern, grid, block, lds, s, x, ldx, ws ? reinterpret_cast<const int8_t*>(ws + w.aq_off) : nullptr,
+                     ws ? reinterpret_cast<const float*>(ws + w.scale_off) : nullptr,
+                     ws ? reinterpret_cast<const int32_t*>(ws + w.off_off) : nullptr, K, KC, p.Wt, ga);
+  return hipGetLastError();
+}
+
+template <int M>
+static hipError_t launch_batched_m(const GroupArgs& ga, const float* x, int ldx, const uint8_t* ws, int K,
+                                   const BatchedPlan& p, hipStream_t s) {
+#define W4_BATCHED(w, c, r) \
+  if (p.waves == w && p.CPW == c && p.R == r) return launch_batched_k<M, w, c, r>(ga, x, ldx, ws, K, p, s);
+  W4_BATCHED(8, 1, 1) W4_BATCHED(8, 2, 1) W4_BATCHED(8, 3, 1)
+  W4_BATCHED(8, 1, 2) W4_BATCHED(8, 2, 2) W4_BATCHED(8, 3, 2)
+  W4_BATCHED(8, 1, 3) W4_BATCHED(8, 2, 3) W4_BATCHED(8, 3, 3)
+  W4_BATCHED(8, 1, 0) W4_BATCHED(8, 2, 0) W4_BATCHED(8, 3, 0)
+  W4_BATCHED(16, 2, 0) W4_BATCHED(16, 3, 0) W4_BATCHED(16, 4, 0) W4_BATCHED(16, 5, 0)
+#undef W4_BATCHED
+  return hipErrorInvalidValue;
+}
+
+static hipError_t launch_batched(const GroupArgs& ga, const float* x, int ldx, const uint8_t* ws, int M, int K,
+                                 const BatchedPlan& p, hipStream_t s) {
+  switch (M) {
+    case 3: return launch_batched_m<3>(ga, x, ldx, ws, K, p, s);
+    case 4: return launch_batched_m<4>(ga, x, ldx, ws, K, p, s);
+    case 5: return launch_batched_m<5>(ga, x, ldx, ws, K, p, s);
+    case 6: return launch_batched_m<6>(ga, x, ldx, ws, K, p, s);
+    case 7: return launch_batched_m<7>(ga, x, ldx, ws, K, p, s);
+    case 8: return launch_batched_m<8>(ga, x, ldx, ws, K, p, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
 // ----------------------------------------------------------------------------------------
 // Wide layers: one wavefront per tile row.
 // ----------------------------------------------------------------------------------------
@@ -943,10 +1321,13 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
     const float* __restrict__ bias, const RowPrologue pro) {
   extern __shared__ __align__(16) uint8_t smem[];
   const int Kp = KC * kTileK;
-  int8_t* s_a = reinterpret_cast<int8_t*>(smem);                   // [M][Kp]
+  // From three rows on (the MFMA form of the products) the int8 rows lie as [32-k block][row][32 bytes], see
+  // gemv_batched_kernel: an operand read then covers contiguous bytes instead of M rows in one bank.
+  constexpr bool kInterleaved = decode_mfma(M);
+  int8_t* s_a = reinterpret_cast<int8_t*>(smem);                   // [M][Kp], or [Kp / 32][M][32]
   float* s_mm = reinterpret_cast<float*>(smem + (size_t)M * Kp);   // [kWideWaves][M][2] or params
 
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int g = lane >> 4, j = lane & 15;
   const int wave_global = blockIdx.x * kWideWaves + wave;
   const int wave_stride = gridDim.x * kWideWaves;
@@ -970,7 +1351,21 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
 
   float recip_m[M];
   int negzp_m[M];
-  if (kFused) {
+  if constexpr (kFused && kInterleaved && !kNorm) {
+    // the rows' quantisation on (row, segment) tasks dealt to the four wavefronts
+    constexpr int kR = M;  // K <= 2048 here: at most four segments per row, 4 M tasks for four wavefronts
+    float xv[kR][8];
+    load_row_tasks<M, kR>(x, ldx, K, Kp, kWideWaves, wave, lane, xv);
+    float2* s_seg = reinterpret_cast<float2*>(s_mm);            // [M * nseg]
+    float* s_par = reinterpret_cast<float*>(s_seg + M * 4);     // [M] recip, [M] -zp
+    quantise_row_tasks<M, kR, kWideWaves>(xv, K, Kp, s_a, s_seg, s_par, wave, lane);
+    __syncthreads();
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      recip_m[m] = s_par[m];
+      negzp_m[m] = reinterpret_cast<const int*>(s_par)[M + m];
+    }
+  } else if (kFused) {
     const int groups = K >> 3;
     float xv[M][8];
     float2* s_mm2 = reinterpret_cast<float2*>(s_mm);
@@ -1049,7 +1444,9 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
       const int m = v / vec_per_row, c = v % vec_per_row;
       uint4 val = make_uint4(0, 0, 0, 0);
       if (16 * c < K) val = *reinterpret_cast<const uint4*>(aq + (size_t)m * K + 16 * c);
-      *reinterpret_cast<uint4*>(s_a + (size_t)m * Kp + 16 * c) = val;
+      int8_t* dst = kInterleaved ? s_a + ((size_t)(c >> 1) * M + m) * kBlockLen + 16 * (c & 1)
+                                 : s_a + (size_t)m * Kp + 16 * c;
+      *reinterpret_cast<uint4*>(dst) = val;
     }
 #pragma unroll
     for (int m = 0; m < M; ++m) {
@@ -1100,7 +1497,12 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
                                __uint_as_float(sc_cur[i].y & 0xFFFF0000u)};
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
-            block_products<M>(wv[d], sv[d], s_a + kTileK * kc + kBlockLen * d + 8 * g, Kp, j, acc);
+            if constexpr (kInterleaved) {
+              block_products<M>(wv[d], sv[d], s_a + (size_t)(4 * kc + d) * (M * kBlockLen) + 8 * g, kBlockLen, j,
+                                acc);
+            } else {
+              block_products<M>(wv[d], sv[d], s_a + kTileK * kc + kBlockLen * d + 8 * g, Kp, j, acc);
+            }
           }
         }
       }
@@ -1220,6 +1622,16 @@ hipError_t launch_gemv(float* y, const uint8_t* ws, const uint8_t* packed, int M
     W4_DISPATCH_M(W4_CALL)
 #undef W4_CALL
   }
+  if (const BatchedPlan bp = batched_preq_plan(M, K); bp.Wt != 0) {
+    GroupArgs ga{};
+    ga.packed[0] = packed;
+    ga.y[0] = y;
+    ga.N[0] = N;
+    ga.first[0] = 0;
+    ga.first[1] = (N + kTileRows - 1) / kTileRows;
+    ga.count = 1;
+    return launch_batched(ga, nullptr, 0, ws, M, K, bp, s);
+  }
 #define W4_CALL(m) (launch_gemv_m<m>(y, ws, packed, K, N, s))
   W4_DISPATCH_M(W4_CALL)
 #undef W4_CALL
@@ -1302,6 +1714,7 @@ hipError_t launch_gemv_fused(float* y, const float* x, int ldx, const uint8_t* p
   ga.first[0] = 0;
   ga.first[1] = (N + kTileRows - 1) / kTileRows;
   ga.count = 1;
+  if (const BatchedPlan bp = batched_plan(M, K); bp.Wt != 0) return launch_batched(ga, x, ldx, nullptr, M, K, bp, s);
   return launch_fused_group(ga, x, ldx, M, K, nullptr, false, s);
 }
 
@@ -1324,6 +1737,7 @@ hipError_t launch_gemv_group(float* const* y, const float* x, int ldx, const uin
     ga.first[i + 1] = ga.first[i] + (N[i] + kTileRows - 1) / kTileRows;
   }
   ga.count = count;
+  if (const BatchedPlan bp = batched_plan(M, K); bp.Wt != 0) return launch_batched(ga, x, ldx, nullptr, M, K, bp, s);
   // one row through two Linears of equal N: the pair kernel with both outputs stored
   const FusedPlan fp = fused_plan(M, K);
   if (count == 2 && N[0] == N[1] && fp.W != 0 && fp.CPW <= 3 && fp.R == 1) {
