@@ -155,6 +155,18 @@ int w4a32_matmul_quantized_splitk(float* d_y, const void* d_ws, const void* d_pa
 int w4a32_matmul(float* d_y, const float* d_x, const void* d_packed, void* d_ws, int M, int K,
                  int N, void* stream);
 
+/* The whole op for a caller that says how large its workspace is: with at least w4a32_workspace_bytes_n(M, K, N)
+ * bytes at d_ws (the activation workspace plus, behind it, room for the partial sums of a product whose k range
+ * the library deals to several workgroups: down_proj at prefill sizes) the call takes that faster form itself;
+ * with at least w4a32_workspace_bytes(M, K) it is w4a32_matmul; with less, W4A32_EINVAL. One call per Linear,
+ * as ...::matmul (kai_linear.cpp:350-398) is called from ArmLinearOp::forward
+ * (mllm/Backends/Arm/Ops/LinearOp.cpp:67-83), whose workspace_size() this pair replaces. Results equal
+ * w4a32_matmul_quantized_splitk's where the k range is split (f32 rounding of the parts' sum apart from
+ * w4a32_matmul's), else w4a32_matmul's bit for bit. */
+size_t w4a32_workspace_bytes_n(int M, int K, int N);
+int w4a32_matmul_ws(float* d_y, const float* d_x, const void* d_packed, void* d_ws, size_t ws_bytes, int M,
+                    int K, int N, void* stream);
+
 /* w4a32_matmul without a workspace argument, for callers that cannot allocate device memory (code under
  * HIP graph capture, serving loops and harnesses that forbid hipMalloc). It has no counterpart in the
  * reference, whose forward allocates its workspace on every call (mllm/Backends/Arm/Ops/LinearOp.cpp:74-78).

@@ -52,6 +52,8 @@ ABI = {
     "w4a32_matmul": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a32_matmul_grouped": (_ci, [_vp, _vp, _vp, _vp, _ci, _vp, _ci, _ci, _vp]),
     "w4a32_matmul_static_ws": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp]),
+    "w4a32_workspace_bytes_n": (_sz, [_ci, _ci, _ci]),
+    "w4a32_matmul_ws": (_ci, [_vp, _vp, _vp, _vp, _sz, _ci, _ci, _ci, _vp]),
     # include/w4a32_decoder.h
     "w4a32_op_embedding": (_ci, [_vp, _vp, _ci, _ci, _ci, _vp, _vp]),
     "w4a32_op_rmsnorm": (_ci, [_vp, _vp, _vp, _ci, _ci, ctypes.c_float, _vp, _vp, _vp]),
@@ -367,6 +369,21 @@ def matmul(x, packed, N, ws=None, out=None):
     _check(lib().w4a32_matmul(_ptr(y), _ptr(x), _ptr(packed), _ptr(ws), M, K, N, _stream()),
            "w4a32_matmul")
     return y
+
+
+def matmul_ws(x, packed, N, ws=None, out=None):
+    """The whole op with a workspace of stated size (w4a32_workspace_bytes_n by default: the library may then
+    deal a long k range to several workgroups, as for down_proj at prefill sizes)."""
+    import torch
+
+    M, K = x.shape
+    if ws is None:
+        ws = _dev_empty(int(lib().w4a32_workspace_bytes_n(M, K, N)))
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    _check(lib().w4a32_matmul_ws(_ptr(out), _ptr(x), _ptr(packed), _ptr(ws), ws.numel() * ws.element_size(), M, K, N,
+                                 _stream()), "w4a32_matmul_ws")
+    return out
 
 
 def matmul_grouped(x, packed_list, n_list, ws=None):

@@ -238,6 +238,27 @@ int w4a32_matmul(float* d_y, const float* d_x, const void* d_packed, void* d_ws,
   return w4a32_matmul_quantized(d_y, d_ws, d_packed, M, K, N, stream);
 }
 
+size_t w4a32_workspace_bytes_n(int M, int K, int N) {
+  const size_t ws = w4a32_workspace_bytes(M, K);
+  if (ws == 0 || shape_ok(N, K)) return 0;
+  return w4::round_up_sz(ws, 256) + w4a32_splitk_scratch_bytes(M, K, N);
+}
+
+int w4a32_matmul_ws(float* d_y, const float* d_x, const void* d_packed, void* d_ws, size_t ws_bytes, int M,
+                    int K, int N, void* stream) {
+  if (M <= 0) return W4A32_EINVAL;
+  if (int e = shape_ok(N, K)) return e;
+  const size_t ws = w4a32_workspace_bytes(M, K);
+  if (!d_ws || ws_bytes < ws) return W4A32_EINVAL;
+  const size_t parts = w4a32_splitk_scratch_bytes(M, K, N), parts_off = w4::round_up_sz(ws, 256);
+  if (parts != 0 && ws_bytes >= parts_off + parts && aligned(d_y, 16)) {
+    if (int e = w4a32_quant_lhs(d_x, M, K, K, d_ws, stream)) return e;
+    return w4a32_matmul_quantized_splitk(d_y, d_ws, d_packed, M, K, N, static_cast<uint8_t*>(d_ws) + parts_off,
+                                         parts, stream);
+  }
+  return w4a32_matmul(d_y, d_x, d_packed, d_ws, M, K, N, stream);
+}
+
 int w4a32_matmul_static_ws(float* d_y, const float* d_x, const void* d_packed, int M, int K, int N,
                            void* stream) {
   if (M <= 0) return W4A32_EINVAL;

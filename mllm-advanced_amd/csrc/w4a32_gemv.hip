@@ -35,7 +35,6 @@
 // the same f32 expression in the same order as on the dot4 path. The instruction count per chunk
 // no longer grows with M (M = 8: 130 -> 45 per wavefront).
 #include <algorithm>
-#include <cstdlib>
 
 #include "w4a32_internal.h"
 #include "w4a32_quant_math.h"
@@ -778,15 +777,18 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_batched_kernel(
   // the rows first (a few KB, normally in L2), then the weights: loads return in issue order
   float xv[kTasks][8];
   uint4 staged[kPreq ? kBatchedStageMax : 1];
-  const int units_per_row = Kp >> 4, units = M * units_per_row;
+  const int units = M * (Kp >> 4);
   if constexpr (kPreq) {
 #pragma unroll
+    // unit u of the LDS image (16 bytes at 16 u) is row (u / 2) % M, k = 32 * ((u / 2) / M) + 16 * (u % 2): threads
+    // take consecutive units, so a wavefront's LDS writes are contiguous (dealt by row, they would all fall into
+    // two banks)
     for (int r = 0; r < kBatchedStageMax; ++r) {
       const int u = threadIdx.x + r * 64 * kWaves;
       staged[r] = make_uint4(0, 0, 0, 0);
       if (u < units) {
-        const int m = u / units_per_row, c = u - m * units_per_row;
-        if (16 * c < K) staged[r] = *reinterpret_cast<const uint4*>(aq + (size_t)m * K + 16 * c);
+        const int m = (u >> 1) % M, k = kBlockLen * ((u >> 1) / M) + 16 * (u & 1);
+        if (k < K) staged[r] = *reinterpret_cast<const uint4*>(aq + (size_t)m * K + k);
       }
     }
     if (threadIdx.x < M) {
@@ -855,10 +857,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_batched_kernel(
 #pragma unroll
     for (int r = 0; r < kBatchedStageMax; ++r) {
       const int u = threadIdx.x + r * 64 * kWaves;
-      if (u < units) {
-        const int m = u / units_per_row, c = u - m * units_per_row;
-        *reinterpret_cast<uint4*>(s_a + ((size_t)(c >> 1) * M + m) * kBlockLen + 16 * (c & 1)) = staged[r];
-      }
+      if (u < units) *reinterpret_cast<uint4*>(s_a + (size_t)16 * u) = staged[r];
     }
   } else {
     quantise_row_tasks<M, kTasks, kWaves>(xv, K, Kp, s_a, s_mm, s_par, wave, lane);
@@ -887,8 +886,14 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_batched_kernel(
   if (owns) {
     const int o = threadIdx.x;
     const int to = o / (M * 16), rem = o - to * (M * 16), m = rem >> 4;
+    // all reads are issued before the first add (a loop over Wt would wait for each LDS read in turn); wavefronts
+    // past Wt re-read the last one and are not added
+    float part[kWaves];
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) part[w] = s_red[(to * Wt + (w < Wt ? w : Wt - 1)) * (M * 16) + rem];
     float sum = 0.0f;
-    for (int w = 0; w < Wt; ++w) sum += s_red[(to * Wt + w) * (M * 16) + rem];
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) sum = w < Wt ? sum + part[w] : sum;
     const float rcp = s_par[m];
     const int off = reinterpret_cast<const int*>(s_par)[M + m];
     float v = __fmaf_rn((float)off, rs, sum * 0.0625f);
@@ -1220,39 +1225,36 @@ static hipError_t launch_fused_m(const GroupArgs& ga, const float* x, int ldx, i
 struct BatchedPlan {
   int waves, Wt, CPW, R;
 };
-static int batched_env(const char* name, int dflt) {
-  const char* e = getenv(name);
-  return e ? atoi(e) : dflt;
-}
 // whole op: the kernel quantises the rows itself
 static BatchedPlan batched_plan(int M, int K) {
   const BatchedPlan none{0, 0, 0, 0};
-  static const int off = batched_env("W4A32_BATCHED_OFF", 0);
-  if (off || M < kBatchedMinM || M > kGemvMaxM) return none;
+  if (M < kBatchedMinM || M > kGemvMaxM) return none;
   const int KC = (K + kTileK - 1) / kTileK;
   const int nseg = (KC * (kTileK / 8) + 63) / 64;
   if (nseg > 8) return none;                        // a row's segment ranges meet in one 8-lane reduction
-  const int waves = 8;
+  const int waves = 8;  // measured: 12 and 16 wavefronts (three / four tile rows per workgroup) are no faster
   const int R = (M * nseg + waves - 1) / waves;
   if (R > 3) return none;
   for (int Wt = 1; Wt <= waves; Wt *= 2) {
     const int cpw = (KC + Wt - 1) / Wt;
-    if (cpw <= 3) return BatchedPlan{waves, Wt, cpw, R};  // about three chunks per wavefront, as in gemv_fused_kernel
+    // about three chunks per wavefront, as in gemv_fused_kernel; a thread stores at most one output, so the
+    // workgroup's waves / Wt tile rows x M rows x 16 columns must not exceed its threads (a short K then runs
+    // with idle wavefronts rather than more tile rows)
+    if (cpw <= 3 && (waves / Wt) * M * 16 <= 64 * waves) return BatchedPlan{waves, Wt, cpw, R};
   }
   return none;
 }
 // rows already quantised
 static BatchedPlan batched_preq_plan(int M, int K) {
   const BatchedPlan none{0, 0, 0, 0};
-  static const int off = batched_env("W4A32_BATCHED_PREQ_OFF", 0);
-  if (off || M < kBatchedMinM || M > kGemvMaxM) return none;
+  if (M < kBatchedMinM || M > kGemvMaxM) return none;
   const int KC = (K + kTileK - 1) / kTileK;
   const int waves = KC > 24 ? 16 : 8, cpw_max = KC > 24 ? 5 : 3;
   if ((M * KC * (kTileK / 16) + 64 * waves - 1) / (64 * waves) > kBatchedStageMax) return none;
   if ((size_t)M * KC * kTileK > 150 * 1024) return none;
   for (int Wt = 1; Wt <= waves; Wt *= 2) {
     const int cpw = (KC + Wt - 1) / Wt;
-    if (cpw <= cpw_max) return BatchedPlan{waves, Wt, cpw, 0};
+    if (cpw <= cpw_max && (waves / Wt) * M * 16 <= 64 * waves) return BatchedPlan{waves, Wt, cpw, 0};
   }
   return none;
 }
@@ -1441,12 +1443,12 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
   } else {
     const int vec_per_row = Kp / 16;
     for (int v = threadIdx.x; v < M * vec_per_row; v += blockDim.x) {
-      const int m = v / vec_per_row, c = v % vec_per_row;
+      // 16-byte unit v of the LDS image: row-major, or (interleaved) row (v / 2) % M at k = 32 ((v / 2) / M) + 16 (v % 2)
+      const int m = kInterleaved ? (v >> 1) % M : v / vec_per_row;
+      const int k = kInterleaved ? kBlockLen * ((v >> 1) / M) + 16 * (v & 1) : 16 * (v % vec_per_row);
       uint4 val = make_uint4(0, 0, 0, 0);
-      if (16 * c < K) val = *reinterpret_cast<const uint4*>(aq + (size_t)m * K + 16 * c);
-      int8_t* dst = kInterleaved ? s_a + ((size_t)(c >> 1) * M + m) * kBlockLen + 16 * (c & 1)
-                                 : s_a + (size_t)m * Kp + 16 * c;
-      *reinterpret_cast<uint4*>(dst) = val;
+      if (k < K) val = *reinterpret_cast<const uint4*>(aq + (size_t)m * K + k);
+      *reinterpret_cast<uint4*>(s_a + (size_t)16 * v) = val;
     }
 #pragma unroll
     for (int m = 0; m < M; ++m) {

@@ -152,24 +152,16 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
   // Every leading dimension is a row. (The reference reads M = shape[-2] and ignores the others,
   // Arm/Ops/LinearOp.cpp:68; the engine only ever runs batch 1, where the two agree.)
   const int M = static_cast<int>(x.numel() / static_cast<size_t>(K));
-  const size_t need = w4a32_workspace_bytes(M, K);
+  // The workspace holds the quantised rows and, behind them, room for the partial sums of a product whose k
+  // range the library deals to several workgroups (few output tiles and a long K: down_proj at prefill sizes).
+  const size_t need = w4a32_workspace_bytes_n(M, K, N);
   if (workspace_.isNil() || tensorBytes(workspace_) < need) {
     workspace_ = Tensor::empty({static_cast<int32_t>(need)}, kInt8, kHIP).alloc();
   }
   auto& hb = currentHipBackend();
-  if (const size_t lend = w4a32_splitk_scratch_bytes(M, K, N)) {
-    // few output tiles and a long K (down_proj at prefill sizes): the library deals each tile's k range to
-    // several workgroups when it is lent room for their partial sums
-    Tensor& scratch = hb.scratch(lend);
-    check(w4a32_quant_lhs(x.ptr<float>(), M, K, K, workspace_.ptr<void>(), hb.stream()), "w4a32_quant_lhs");
-    check(w4a32_matmul_quantized_splitk(y.ptr<float>(), workspace_.ptr<void>(), weight_.ptr<void>(), M, K, N,
-                                        scratch.ptr<void>(), tensorBytes(scratch), hb.stream()),
-          "w4a32_matmul_quantized_splitk");
-    return;
-  }
-  check(w4a32_matmul(y.ptr<float>(), x.ptr<float>(), weight_.ptr<void>(), workspace_.ptr<void>(), M, K,
-                     N, hb.stream()),
-        "w4a32_matmul");
+  check(w4a32_matmul_ws(y.ptr<float>(), x.ptr<float>(), weight_.ptr<void>(), workspace_.ptr<void>(),
+                        tensorBytes(workspace_), M, K, N, hb.stream()),
+        "w4a32_matmul_ws");
   // Stays asynchronous on the backend's stream: a host consumer goes through D2H, which waits.
 }
 

@@ -337,6 +337,30 @@ def test_decoder_runner_matches_oracle(pkg):
         assert dec.position == 12 + step
 
 
+@pytest.mark.parametrize("slices", [(8, 3), (3, 8), (5, 6), (1, 2, 8), (4, 7)])
+def test_decoder_prefill_in_slices_of_decode_sized_rows(pkg, slices):
+    """A prompt fed in slices of 1..8 rows runs every Linear through the decode-sized kernels on several rows (short
+    K: more tile rows per workgroup than at the model's widths), continuing the cache of the slices before."""
+    import decoder_oracle as do
+
+    rng = np.random.default_rng(21)
+    H, Hq, Hkv, I, V, L = 256, 2, 1, 384, 640, 2
+    weights = tiny_model(rng, H, Hq, Hkv, I, V, L)
+    dec = to_device_model(pkg, weights, Hq, Hkv, max_seq=64, max_batch_tokens=8, rope_theta=1e6)
+    ref = do.Decoder(weights, Hq, Hkv, rope_theta=1e6, max_seq=64)
+    prompt = rng.integers(0, V, size=sum(slices))
+    want = ref.forward(prompt)
+    for rep in range(2):                          # the second pass overwrites the first one's cache rows
+        pos = 0
+        for n in slices:
+            dec.prefill(dev(prompt[pos:pos + n].astype(np.int64)), pos0=pos)
+            pos += n
+        torch.cuda.synchronize()
+        got = dec.logits.cpu().numpy()
+        assert max_abs_rel(got, want) < 2e-3, rep
+        assert int(dec.token) == do.greedy(got) and dec.position == len(prompt)
+
+
 def test_decoder_ignores_what_its_state_memory_held(pkg):
     # The state is caller-owned memory that init does not clear: rows of the KV cache behind the position,
     # scratch areas and activations hold whatever was there. Bytes 0xFF (NaN as f32) against zeros: prefill

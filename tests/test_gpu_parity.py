@@ -227,7 +227,10 @@ def test_gemv_lm_head(pkg, orc, m):
     assert err <= GEMV_TOL and err <= TIGHT, err
 
 
-@pytest.mark.parametrize("m,k,n", [(1, 32, 16), (3, 64, 5), (8, 96, 50), (1, 1024, 1024)])
+@pytest.mark.parametrize("m,k,n", [(1, 32, 16), (3, 64, 5), (8, 96, 50), (1, 1024, 1024),
+                                   # several rows on a short K: a workgroup takes many tile rows
+                                   (8, 256, 512), (7, 384, 256), (5, 128, 300), (8, 96, 400), (6, 32, 1000),
+                                   (4, 4096, 100), (8, 3072, 48), (3, 2048, 33)])
 def test_gemv_ragged_shapes(pkg, orc, m, k, n):
     # N not a multiple of 16, K not a multiple of 128: padding inside the tiles must be inert
     y, ref = run_linear(pkg, orc, m, k, n, True, wseed=m + k, xseed=n)
@@ -350,6 +353,37 @@ def test_splitk_matches_oracle_and_plain(pkg, orc, m, k, n):
     import torch
     tiny = torch.empty((16,), dtype=torch.uint8, device="cuda")
     assert np.array_equal(host(pkg.matmul_quantized_splitk(ws, packed, m, k, n, scratch=tiny)), plain)
+
+
+@pytest.mark.parametrize("m,k,n", [(512, 8960, 1536), (128, 8960, 1536), (100, 8960, 50), (64, 256, 64), (4, 8960, 1536)])
+def test_whole_op_with_a_sized_workspace_takes_the_split_form_itself(pkg, orc, m, k, n):
+    # w4a32_matmul_ws: one call per Linear; with room for the partial sums behind the activation workspace the
+    # library deals a long k range to several workgroups itself, with the plain workspace it is w4a32_matmul
+    import torch
+    w = make_weights(n, k, seed=n + 3)
+    x = make_acts(m, k, seed=m + 1, outlier_frac=0.02)
+    bias = bias_for(n, True)
+    u4, sc = orc.quant_rhs(w)
+    packed = pkg.repack_native(dev(u4), dev(sc.view(np.int16)), dev(bias), n, k)
+    xd = dev(x)
+    L = pkg.lib()
+    small, large = int(L.w4a32_workspace_bytes(m, k)), int(L.w4a32_workspace_bytes_n(m, k, n))
+    scratch = int(L.w4a32_splitk_scratch_bytes(m, k, n))
+    assert large == (small + 255) // 256 * 256 + scratch and (scratch > 0) == (m > 8 and k >= 6144)
+    y = host(pkg.matmul_ws(xd, packed, n))
+    plain = host(pkg.matmul(xd, packed, n))
+    rows = np.unique(np.concatenate([np.arange(0, m, 37), [m - 1]]))
+    assert max_abs_rel(y[rows], orc.linear(x[rows], u4, sc, bias=bias, threads=8)) <= TIGHT
+    if scratch:
+        split = host(pkg.matmul_quantized_splitk(pkg.quant_lhs(xd), packed, m, k, n))
+        assert np.array_equal(y, split) and max_abs_rel(y, plain) <= 1e-6
+    else:
+        assert np.array_equal(y, plain)
+    # the plain workspace: w4a32_matmul, bit for bit; a shorter one is refused
+    ws_small = torch.empty((small,), dtype=torch.uint8, device="cuda")
+    assert np.array_equal(host(pkg.matmul_ws(xd, packed, n, ws=ws_small)), plain)
+    with pytest.raises(pkg.W4A32Error):
+        pkg.matmul_ws(xd, packed, n, ws=ws_small[: small - 256])
 
 
 @pytest.mark.parametrize("m,k,n", [(9, 64, 48), (33, 64, 48), (130, 160, 100), (256, 1536, 8960), (512, 1536, 8960),
