@@ -153,6 +153,8 @@ int w4a32_op_argmax(const float* d_logits, int n, void* d_scratch, int64_t* d_to
  * The fusions of QWenDecoder::forward / QWenMLP::forward (modeling_ds_qwen2.hpp:47-54,175-183) that cost a
  * launch each when run as separate operators. Returns W4A32_ENOTSUP when the shape does not fit the
  * single-launch kernel (the caller then runs the operators one by one). */
+/* Zero-initialise the struct before filling it: fields added at its end (in_parts, out_parts) select other
+ * forms of the call when they are not 0. */
 typedef struct {
   const float* d_x;
   const float* d_delta;
@@ -166,13 +168,15 @@ typedef struct {
   float* d_y[4];
   int silu_pair;
   int in_parts;   /* 0 or 1: a single row. 2 or 3: the row is given in that many partial rows, K floats apart, which
-                     the launch adds up ((r0 + r1) + r2) before it does anything else - at d_delta when
+                     the launch adds up ((r0 + r1) + r2), clamped to the finite f32 range like every Linear
+                     output, before it does anything else - at d_delta when
                      d_norm_weight is given (d_delta is then required), else at d_x. Not with silu_pair; for an
                      lm_head-sized Linear (N >= 32768) only as a single Linear with a norm (W4A32_ENOTSUP else). */
   int out_parts;  /* 0 or 1: d_y holds the Linears' outputs. > 1 (count == 1, no norm, no pair, in_parts <= 1;
                      must equal w4a32_decode_kparts(K, N[0])): the Linear's k range is dealt to that many workgroups
                      per tile row and d_y[0] receives [out_parts][N[0]] partial rows whose sum is the output (bias
-                     included), for a reader that adds them up - the next w4a32_decode_linear via in_parts. */
+                     included; the parts themselves are not clamped, a reader that adds them up clamps the sum),
+                     for the next w4a32_decode_linear via in_parts. */
 } w4a32_decode_linear_args;
 int w4a32_decode_linear(const w4a32_decode_linear_args* args, void* stream);
 

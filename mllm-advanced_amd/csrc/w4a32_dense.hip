@@ -96,6 +96,12 @@ __global__ __launch_bounds__(64 * kDenseWaves) void dense_rows_kernel(const floa
             const float4 e = *reinterpret_cast<const float4*>(pro.delta + (size_t)p * K + i);
             d.x += e.x; d.y += e.y; d.z += e.z; d.w += e.w;
           }
+          if (pro.delta_parts > 1) {  // the parts' sum is a Linear's output: clamped like every other one
+            d.x = fminf(fmaxf(d.x, -3.402823466e+38f), 3.402823466e+38f);
+            d.y = fminf(fmaxf(d.y, -3.402823466e+38f), 3.402823466e+38f);
+            d.z = fminf(fmaxf(d.z, -3.402823466e+38f), 3.402823466e+38f);
+            d.w = fminf(fmaxf(d.w, -3.402823466e+38f), 3.402823466e+38f);
+          }
           v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
         }
         ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;

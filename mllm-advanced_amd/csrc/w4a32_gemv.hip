@@ -449,12 +449,15 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
     for (int r = 0; r < kFusedR; ++r) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
+        // the sum of the parts is a Linear's output: clamped to the finite f32 range like every other one
         if constexpr (kNorm) {
           dv[0][r][e] += pv[0][r][e];
           if (in_parts > 2) dv[0][r][e] += pv[1][r][e];
+          dv[0][r][e] = fminf(fmaxf(dv[0][r][e], -3.402823466e+38f), 3.402823466e+38f);
         } else {
           xv[0][r][e] += pv[0][r][e];
           if (in_parts > 2) xv[0][r][e] += pv[1][r][e];
+          xv[0][r][e] = fminf(fmaxf(xv[0][r][e], -3.402823466e+38f), 3.402823466e+38f);
         }
       }
     }
@@ -908,8 +911,9 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_batched_kernel(
 // (part p, tile row nt) quantises the row as gemv_fused_kernel does (the range needs the whole row; only
 // the part's own k range is converted and kept), multiplies its chunks kc0 .. kc0 + KCp - 1 and stores
 //   part 0:  (sum/16 + off * rsum[n]) * lhs_scale + bias[n]        parts 1..:  (sum/16) * lhs_scale
-// to y[p][n]: the parts add up to the Linear's output (up to f32 rounding) and whoever reads it next adds
-// them, so no workgroup waits for another. W wavefronts hold three chunks each (KCp <= 3 W).
+// to y[p][n]: the parts add up to the Linear's output (up to f32 rounding; the parts themselves are not clamped,
+// the reader clamps their sum to the finite f32 range) and whoever reads it next adds them, so no workgroup
+// waits for another. W wavefronts hold three chunks each (KCp <= 3 W).
 // Two parts measured best for down_proj (K = 8960, N = 1536: 192 workgroups of 12 wavefronts, 4.9 us against
 // 5.2 us in three parts and 6.7 us unsplit); a reader adds up to kMaxInParts partial rows.
 constexpr int kDecodeParts = 2;
@@ -1390,6 +1394,10 @@ __global__ __launch_bounds__(64 * kWideWaves) void gemv_wide_kernel(
             const float4 e1 = *reinterpret_cast<const float4*>(dsrc + (size_t)p * K + 4);
             dd[0] += e0.x; dd[1] += e0.y; dd[2] += e0.z; dd[3] += e0.w;
             dd[4] += e1.x; dd[5] += e1.y; dd[6] += e1.z; dd[7] += e1.w;
+          }
+          if (pro.delta_parts > 1) {  // the parts' sum is a Linear's output: clamped like every other one
+#pragma unroll
+            for (int e = 0; e < 8; ++e) dd[e] = fminf(fmaxf(dd[e], -3.402823466e+38f), 3.402823466e+38f);
           }
 #pragma unroll
           for (int e = 0; e < 8; ++e) f[e] += dd[e];

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 import torch
 
-from conftest import max_abs_rel
+from conftest import make_weights, max_abs_rel
 
 pytestmark = pytest.mark.gpu
 
@@ -887,3 +887,26 @@ def test_decoder_refuses_to_run_past_its_cache(pkg):
     with pytest.raises(pkg.W4A32Error):
         dec.step()
     assert dec.position == 16
+
+
+def test_partial_rows_whose_sum_overflows_are_clamped_by_the_reader(pkg):
+    """A Linear that ran split over K leaves unclamped partial rows; the launch that adds them up clamps the sum
+    to the finite f32 range, as the unsplit kernel (and the reference's matmul, kai_linear.cpp:392-396) clamps
+    its output. Observed through the residual sum the reader stores: h + (p0 + p1) with h = 0."""
+    K, N = 1536, 256
+    big = np.float32(3e38)
+    parts = np.zeros((2, K), dtype=np.float32)
+    parts[:, 0] = (big, big)            # +inf as a plain sum
+    parts[:, 5] = (-big, -big)          # -inf
+    parts[:, 9] = (big, -big)           # cancels
+    parts[:, 17] = (1.5, 2.25)
+    flt_max = np.finfo(np.float32).max
+    w = make_weights(N, K, seed=3)
+    packed = pkg.quant_pack_rhs(dev(w))
+    nw = torch.ones((K,), device="cuda")
+    h = torch.zeros((1, K), device="cuda")
+    _, total = pkg.decode_linear(h, [packed], [N], norm_weight=nw, delta=dev(parts), want_sum=True, in_parts=2)
+    torch.cuda.synchronize()
+    t = total.cpu().numpy()[0]
+    assert t[0] == flt_max and t[5] == -flt_max and t[9] == 0.0 and t[17] == 3.75
+    assert not t[[1, 2, 3, 4, 6, 7, 8, 10]].any()

@@ -84,3 +84,29 @@ def test_patch_embed_conv3d_as_w4a32_linear(pkg, orc):
     conv = torch.nn.functional.conv3d(torch.from_numpy(a), torch.from_numpy(w), torch.from_numpy(bias),
                                       stride=stride).permute(0, 2, 3, 4, 1).reshape(-1, OC).numpy()
     assert max_abs_rel(y, conv) < 0.1
+
+
+def test_patch_embed_at_the_configuration_s_image_size(pkg, orc):
+    """One 448 x 448 image (two frames), 14 x 14 patches: 1024 rows of K = 1176 (padded to 1184) through the
+    1280 filters, as configuration 5 names it. The product against the oracle on sampled rows."""
+    rng = np.random.default_rng(2)
+    B, C, T, H, W, OC = 1, 3, 2, 448, 448, 1280
+    kernel = stride = (2, 14, 14)
+    a = rng.standard_normal((B, C, T, H, W)).astype(np.float32)
+    w = (rng.standard_normal((OC, C) + kernel) * 0.02).astype(np.float32)
+    bias = (rng.standard_normal(OC) * 0.02).astype(np.float32)
+    K = C * 2 * 14 * 14
+    Kp = (K + 31) // 32 * 32
+    wp = np.zeros((OC, Kp), dtype=np.float32)
+    wp[:, :K] = w.reshape(OC, K)
+    cols = pkg.op_im2col_conv3d(dev(a), kernel, stride)
+    assert tuple(cols.shape) == (1024, Kp)
+    y = pkg.matmul(cols, pkg.quant_pack_rhs(dev(wp), dev(bias)), OC).cpu().numpy()
+    assert y.shape == (1024, OC) and np.isfinite(y).all()
+    rows = np.unique(np.concatenate([np.arange(0, 1024, 41), [1023]]))
+    ref_cols = im2col_ref(a, kernel, stride)
+    assert np.array_equal(cols.cpu().numpy()[:, :K], ref_cols) and not cols.cpu().numpy()[:, K:].any()
+    zp = np.zeros((len(rows), Kp), dtype=np.float32)
+    zp[:, :K] = ref_cols[rows]
+    u4, sc = orc.quant_rhs(wp)
+    assert max_abs_rel(y[rows], orc.linear(zp, u4, sc, bias=bias, threads=8)) <= 2e-3

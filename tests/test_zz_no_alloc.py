@@ -72,3 +72,38 @@ def test_static_workspace_rejects_what_does_not_fit(pkg):
     assert L.w4a32_matmul_static_ws(y.data_ptr(), x.data_ptr(), packed.data_ptr(), 0, K, N, None) == -1
     assert L.w4a32_matmul_static_ws(y.data_ptr(), x.data_ptr(), packed.data_ptr(), 8, K + 1, N, None) == -2
     torch.cuda.synchronize()
+
+
+def test_static_workspace_call_replays_from_a_graph(pkg):
+    """What the entry point is for: after one eager call (which looks the array's address up), the call is
+    captured into a HIP graph and replayed on changed inputs, with eager work between the replays; every replay
+    must equal the eager w4a32_matmul on the same input bit for bit."""
+    import torch
+
+    L = pkg.lib()
+    for (M, K, N) in [(64, 1536, 256), (4, 8960, 1536)]:
+        w = make_weights(N, K, seed=M)
+        packed = pkg.quant_pack_rhs(torch.from_numpy(w).cuda())
+        x = torch.from_numpy(make_acts(M, K, seed=1)).cuda()
+        y = torch.empty((M, N), dtype=torch.float32, device="cuda")
+        stream = torch.cuda.Stream()
+        with torch.cuda.stream(stream):
+            sp = ctypes.c_void_p(stream.cuda_stream)
+            assert L.w4a32_matmul_static_ws(y.data_ptr(), x.data_ptr(), packed.data_ptr(), M, K, N, sp) == 0
+            stream.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                rc = L.w4a32_matmul_static_ws(y.data_ptr(), x.data_ptr(), packed.data_ptr(), M, K, N,
+                                              ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+            assert rc == 0
+            for rep in range(3):
+                x.copy_(torch.from_numpy(make_acts(M, K, seed=50 + rep)).cuda())
+                y.fill_(float("nan"))
+                g.replay()
+                stream.synchronize()
+                got = y.clone()
+                # eager work of the same kind between the replays (it shares the static array)
+                other = torch.from_numpy(make_acts(M, K, seed=90 + rep)).cuda()
+                assert L.w4a32_matmul_static_ws(y.data_ptr(), other.data_ptr(), packed.data_ptr(), M, K, N, sp) == 0
+                stream.synchronize()
+                assert torch.equal(got, pkg.matmul(x, packed, N)), (M, K, N, rep)
