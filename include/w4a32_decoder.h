@@ -116,6 +116,19 @@ int w4a32_op_attention_prefill(const float* d_q, const float* d_kcache, const fl
                                int max_seq, const int* d_pos0, int pos0, void* d_part, size_t part_bytes,
                                void* stream);
 
+/* The same operator for M >= 32 rows at a position the host knows, with both products on the 16-bit matrix
+ * pipe at f32 accuracy: every f32 operand is split into three bf16 terms and a product is the six partial
+ * products that matter (v_mfma_f32_32x32x16_bf16, f32 accumulation; 2.7 x the rate of the f32 matrix
+ * instruction, same exponent range as f32, error below 2^-22 of |x||y| per product). A first launch splits K and V
+ * of keys [0, pos0 + M) (V transposed) into d_scratch: at least
+ * w4a32_op_attention_prefill_bf16x3_scratch_bytes(pos0 + M, n_kv_heads) bytes, 16-byte aligned, contents need
+ * not be kept. Same reference operator as w4a32_op_attention (modeling_ds_qwen2.hpp:133-151). */
+size_t w4a32_op_attention_prefill_bf16x3_scratch_bytes(int n_keys, int n_kv_heads);
+int w4a32_op_attention_prefill_bf16x3(const float* d_q, const float* d_kcache, const float* d_vcache,
+                                      float* d_out, int M, int n_heads, int n_kv_heads, int head_dim,
+                                      int max_seq, int pos0, void* d_scratch, size_t scratch_bytes,
+                                      void* stream);
+
 /* Decode step (one token at position pos0) with w4a32_op_rope_kv folded into the attention launch:
  * d_q, d_k, d_v are the un-rotated outputs of the q/k/v Linears; the kernel rotates q and k, appends k
  * and v to the caches at pos0 and attends over keys 0..pos0. Same results as the two operators in

@@ -69,6 +69,8 @@ ABI = {
     "w4a32_op_attention_prefill_scratch_bytes": (_sz, [_ci, _ci]),
     "w4a32_op_attention_prefill": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _ci, _vp, _sz,
                                          _vp]),
+    "w4a32_op_attention_prefill_bf16x3_scratch_bytes": (_sz, [_ci, _ci]),
+    "w4a32_op_attention_prefill_bf16x3": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a32_op_rope_attention_decode": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci,
                                              _vp, _ci, _vp, _vp]),
     "w4a32_op_rope_attention_decode_linear": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _vp, _ci, _ci,
@@ -585,6 +587,20 @@ def op_attention_prefill(q, kcache, vcache, n_heads, n_kv_heads, head_dim, pos0,
                                             n_kv_heads, head_dim, kcache.shape[1], _ptr(d_pos0), pos0,
                                             _ptr(part), part.numel(), _stream()),
            "w4a32_op_attention_prefill")
+    return out
+
+
+def op_attention_prefill_bf16x3(q, kcache, vcache, n_heads, n_kv_heads, head_dim, pos0):
+    """The prefill attention with its products on the bf16 matrix pipe (three terms per f32 operand)."""
+    import torch
+
+    M = q.shape[0]
+    out = torch.empty((M, n_heads * head_dim), dtype=torch.float32, device="cuda")
+    scratch = _dev_empty(int(lib().w4a32_op_attention_prefill_bf16x3_scratch_bytes(pos0 + M, n_kv_heads)))
+    _check(lib().w4a32_op_attention_prefill_bf16x3(_ptr(q), _ptr(kcache), _ptr(vcache), _ptr(out), M, n_heads,
+                                                   n_kv_heads, head_dim, kcache.shape[1], pos0, _ptr(scratch),
+                                                   scratch.numel(), _stream()),
+           "w4a32_op_attention_prefill_bf16x3")
     return out
 
 

@@ -12,6 +12,7 @@ constexpr int kAttnSplit = 16;    // key slices (workgroups) per head group in t
 // ... when the slices are left to the Linear that follows: 16 measured better than 8 (0.794 ms per token against
 // 0.809 with the same 4 wavefronts, which then take two key blocks in sequence, and 0.810 with 8 wavefronts)
 constexpr int kAttnDeferSlices = 16;
+constexpr int kAttn16MinRows = 256;  // prefill rows from which the bf16-term attention kernel is the faster one
 constexpr int kArgmaxBlocks = 64;
 constexpr int kArgmaxParts = 4096;  // partial results an lm_head launch can leave (one per wavefront)
 
@@ -111,7 +112,8 @@ StateGeom state_geom(const w4a32_decoder_config* c) {
 // The model on M rows that are already embedded in the residual stream `h`. Leaves the last row's
 // logits in the state and the greedy token in *d_token_out. d_pos: device position of row 0.
 int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, uint8_t* st,
-               const StateGeom& g, int M, int64_t* d_token_out, bool advance_by_argmax, void* stream) {
+               const StateGeom& g, int M, int64_t* d_token_out, bool advance_by_argmax, void* stream,
+               int host_pos0 = -1) {
   hipStream_t s = S(stream);
   const int H = c->hidden, I = c->intermediate, D = c->head_dim;
   const int Hq = c->n_heads, Hkv = c->n_kv_heads, qd = Hq * D, kvd = Hkv * D;
@@ -181,10 +183,18 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
           reinterpret_cast<unsigned int*>(scratch + sg.counters_off), nullptr, nullptr, nullptr, nullptr, false,
           s)));
     } else {
-      // the gate and up buffers are dead here: they hold the per-chunk results of long query blocks
-      W4_TRY(from_hip(w4::launch_attention_prefill(q, kc, vc, attn, M, Hq, Hkv, c->max_seq, d_pos, 0, gate,
-                                                   lend, reinterpret_cast<unsigned int*>(st + g.pfcnt_off),
-                                                   s)));
+      // the gate and up buffers are dead here: they hold the bf16 terms of K and V for the matrix-pipe kernel
+      // (a prefill knows its position on the host; from kAttn16MinRows rows on that kernel is the faster one),
+      // or the per-chunk results of long query blocks for the f32 kernel
+      if (host_pos0 >= 0 && M >= kAttn16MinRows &&
+          w4::attention16_scratch_bytes(host_pos0 + M, Hkv) <= lend) {
+        W4_TRY(from_hip(w4::launch_attention16(q, kc, vc, attn, M, Hq, Hkv, c->max_seq, host_pos0,
+                                               reinterpret_cast<uint8_t*>(gate), s)));
+      } else {
+        W4_TRY(from_hip(w4::launch_attention_prefill(q, kc, vc, attn, M, Hq, Hkv, c->max_seq, d_pos, 0, gate,
+                                                     lend, reinterpret_cast<unsigned int*>(st + g.pfcnt_off),
+                                                     s)));
+      }
     }
     W4_TRY(w4a32_matmul(delta, attn, lw.o, ws, M, qd, H, stream));
     // h += attention output; xn = norm(h)
@@ -533,6 +543,28 @@ int w4a32_op_attention_prefill(const float* d_q, const float* d_kcache, const fl
                                                part_bytes, nullptr, S(stream)));
 }
 
+size_t w4a32_op_attention_prefill_bf16x3_scratch_bytes(int n_keys, int n_kv_heads) {
+  if (n_keys <= 0 || n_kv_heads <= 0) return 0;
+  return w4::attention16_scratch_bytes(n_keys, n_kv_heads);
+}
+
+int w4a32_op_attention_prefill_bf16x3(const float* d_q, const float* d_kcache, const float* d_vcache,
+                                      float* d_out, int M, int n_heads, int n_kv_heads, int head_dim,
+                                      int max_seq, int pos0, void* d_scratch, size_t scratch_bytes,
+                                      void* stream) {
+  if (!d_q || !d_kcache || !d_vcache || !d_out || !d_scratch) return W4A32_EINVAL;
+  if (M <= 0 || n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0) return W4A32_EINVAL;
+  if (head_dim != 128 || n_heads % n_kv_heads != 0) return W4A32_ESHAPE;
+  if (pos0 < 0 || pos0 + M > max_seq) return W4A32_ESHAPE;
+  if (reinterpret_cast<uintptr_t>(d_scratch) % 16 != 0 || reinterpret_cast<uintptr_t>(d_q) % 16 != 0 ||
+      reinterpret_cast<uintptr_t>(d_out) % 16 != 0) {
+    return W4A32_EINVAL;
+  }
+  if (scratch_bytes < w4::attention16_scratch_bytes(pos0 + M, n_kv_heads)) return W4A32_EINVAL;
+  return from_hip(w4::launch_attention16(d_q, d_kcache, d_vcache, d_out, M, n_heads, n_kv_heads, max_seq, pos0,
+                                         static_cast<uint8_t*>(d_scratch), S(stream)));
+}
+
 int w4a32_op_rope_attention_decode(const float* d_q, const float* d_k, const float* d_v,
                                    const float* d_sin, const float* d_cos, float* d_kcache,
                                    float* d_vcache, float* d_out, int n_heads, int n_kv_heads,
@@ -668,7 +700,7 @@ int w4a32_decoder_prefill(const w4a32_decoder_config* cfg, const w4a32_decoder_w
   W4_TRY(from_hip(w4::launch_set_int(d_pos, pos0, s)));
   W4_TRY(from_hip(w4::launch_embedding(d_tokens, w->embedding, n_tokens, cfg->hidden, cfg->vocab,
                                        reinterpret_cast<float*>(st + g.h_off), s)));
-  W4_TRY(run_layers(cfg, w, st, g, n_tokens, d_next_token, false, stream));
+  W4_TRY(run_layers(cfg, w, st, g, n_tokens, d_next_token, false, stream, pos0));
   return from_hip(w4::launch_add_to_int(d_pos, n_tokens, s));
 }
 

@@ -115,6 +115,11 @@ size_t attention_prefill_part_bytes(int M, int Hq);
 hipError_t launch_attention_prefill(const float* q, const float* kc, const float* vc, float* out,
                                     int M, int Hq, int Hkv, int max_seq, const int* d_pos0, int pos0,
                                     float* part, size_t part_bytes, unsigned int* counters, hipStream_t s);
+// the same operator with its products on the bf16 matrix pipe, every f32 operand as three bf16 terms
+// (w4a32_attention16.hip); scratch: attention16_scratch_bytes(pos0 + M, Hkv) bytes, 16-byte aligned
+size_t attention16_scratch_bytes(int n_keys, int Hkv);
+hipError_t launch_attention16(const float* q, const float* kc, const float* vc, float* out, int M, int Hq, int Hkv,
+                              int max_seq, int pos0, uint8_t* scratch, hipStream_t s);
 hipError_t launch_attention_bshd(const float* q, const float* k, const float* v, float* out, int M, int Hq,
                                  int Hkv, int n_keys, int pos0, hipStream_t s);
 // operators of the engine's op-by-op path (w4a32_engine_ops.hip)

@@ -204,6 +204,42 @@ def test_attention_prefill_and_decode(pkg, Hq, Hkv):
 
 
 @pytest.mark.parametrize("Hq,Hkv", [(12, 2), (4, 4), (3, 1)])
+def test_attention_prefill_on_bf16_terms(pkg, Hq, Hkv):
+    """The prefill attention with both products on the 16-bit matrix pipe, every f32 operand as three bf16 terms:
+    against torch's f32 attention to the same 2e-5 as the f32 kernels, on operands with a wide range of magnitudes
+    (the terms keep f32's exponent range), NaN in the cache rows past the last key (they must not reach the sums),
+    ragged row counts and positions."""
+    g = torch.Generator(device="cuda").manual_seed(3)
+    D, S = 128, 1024
+
+    def ref(q, kc, vc, pos0):
+        M = q.shape[0]
+        tq = q.view(M, Hq, D).permute(1, 0, 2)[None].double()
+        n = pos0 + M
+        tk = kc[:, :n].repeat_interleave(Hq // Hkv, dim=0)[None].double()
+        tv = vc[:, :n].repeat_interleave(Hq // Hkv, dim=0)[None].double()
+        mask = torch.ones(M, n, dtype=torch.bool, device="cuda").tril(diagonal=pos0)
+        with torch.nn.attention.sdpa_kernel(torch.nn.attention.SDPBackend.MATH):
+            o = torch.nn.functional.scaled_dot_product_attention(tq, tk, tv, attn_mask=mask)
+        return o[0].permute(1, 0, 2).reshape(M, Hq * D)
+
+    for M, pos0, kscale, vscale in [(32, 0, 1.0, 1.0), (70, 0, 1.0, 1.0), (130, 5, 1.0, 1.0), (256, 0, 1.0, 1.0),
+                                    (300, 200, 1.0, 1.0), (512, 0, 1.0, 1.0), (512, 512, 1.0, 1.0), (64, 960, 1.0, 1.0),
+                                    (100, 924, 1.0, 1.0), (200, 37, 30.0, 1e-6), (160, 0, 1e-4, 3e4)]:
+        kc = torch.randn((Hkv, S, D), generator=g, device="cuda") * kscale
+        vc = torch.randn((Hkv, S, D), generator=g, device="cuda") * vscale
+        # magnitudes spread over many binades inside one row as well
+        vc *= torch.exp2(torch.randint(-6, 7, (Hkv, S, D), generator=g, device="cuda").float())
+        q = torch.randn((M, Hq * D), generator=g, device="cuda") / max(kscale, 1.0)
+        want = ref(q, kc, vc, pos0).cpu().numpy()
+        kc[:, pos0 + M:] = float("nan")
+        vc[:, pos0 + M:] = float("nan")
+        out = pkg.op_attention_prefill_bf16x3(q, kc, vc, Hq, Hkv, D, pos0)
+        torch.cuda.synchronize()
+        assert max_abs_rel(out.cpu().numpy(), want) < 2e-5, (M, pos0, kscale, vscale)
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(12, 2), (4, 4), (3, 1)])
 def test_rope_attention_decode_equals_the_two_operators(pkg, Hq, Hkv):
     g = torch.Generator(device="cuda").manual_seed(6)
     D, S = 128, 256
