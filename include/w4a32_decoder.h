@@ -129,6 +129,17 @@ int w4a32_op_attention_prefill_bf16x3(const float* d_q, const float* d_kcache, c
                                       int max_seq, int pos0, void* d_scratch, size_t scratch_bytes,
                                       void* stream);
 
+/* w4a32_op_rope_kv (position given on the host) followed by w4a32_op_attention_prefill_bf16x3, in two launches
+ * instead of three: the launch that splits K and V into bf16 terms also rotates q (in place) and the new rows of
+ * k, and appends k and v to the caches. d_q, d_k, d_v are the un-rotated outputs of the q/k/v Linears for rows
+ * at positions pos0 .. pos0 + M - 1. Caches, d_q and d_out end up bit-identical to the two operators in
+ * sequence. normal_hf_rope (rope.cpp:39-80), ArmKVCacheOp::forward (KVCacheOp.cpp:44-72) and the attention of
+ * modeling_ds_qwen2.hpp:133-151. Scratch as for w4a32_op_attention_prefill_bf16x3. */
+int w4a32_op_rope_attention_prefill_bf16x3(float* d_q, const float* d_k, const float* d_v, const float* d_sin,
+                                           const float* d_cos, float* d_kcache, float* d_vcache, float* d_out,
+                                           int M, int n_heads, int n_kv_heads, int head_dim, int max_seq,
+                                           int pos0, void* d_scratch, size_t scratch_bytes, void* stream);
+
 /* Decode step (one token at position pos0) with w4a32_op_rope_kv folded into the attention launch:
  * d_q, d_k, d_v are the un-rotated outputs of the q/k/v Linears; the kernel rotates q and k, appends k
  * and v to the caches at pos0 and attends over keys 0..pos0. Same results as the two operators in

@@ -71,6 +71,8 @@ ABI = {
                                          _vp]),
     "w4a32_op_attention_prefill_bf16x3_scratch_bytes": (_sz, [_ci, _ci]),
     "w4a32_op_attention_prefill_bf16x3": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _vp, _sz, _vp]),
+    "w4a32_op_rope_attention_prefill_bf16x3": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci,
+                                                     _ci, _vp, _sz, _vp]),
     "w4a32_op_rope_attention_decode": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci,
                                              _vp, _ci, _vp, _vp]),
     "w4a32_op_rope_attention_decode_linear": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _vp, _ci, _ci,
@@ -601,6 +603,22 @@ def op_attention_prefill_bf16x3(q, kcache, vcache, n_heads, n_kv_heads, head_dim
                                                    n_kv_heads, head_dim, kcache.shape[1], pos0, _ptr(scratch),
                                                    scratch.numel(), _stream()),
            "w4a32_op_attention_prefill_bf16x3")
+    return out
+
+
+def op_rope_attention_prefill_bf16x3(q, k, v, sin, cos, kcache, vcache, n_heads, n_kv_heads, head_dim, pos0):
+    """op_rope_kv (q rotated in place, k and v appended to the caches at pos0..) + op_attention_prefill_bf16x3 with
+    the rotation and the append done by the launch that splits K and V."""
+    import torch
+
+    M = q.shape[0]
+    out = torch.empty((M, n_heads * head_dim), dtype=torch.float32, device="cuda")
+    scratch = _dev_empty(int(lib().w4a32_op_attention_prefill_bf16x3_scratch_bytes(pos0 + M, n_kv_heads)))
+    _check(lib().w4a32_op_rope_attention_prefill_bf16x3(_ptr(q), _ptr(k), _ptr(v), _ptr(sin), _ptr(cos),
+                                                        _ptr(kcache), _ptr(vcache), _ptr(out), M, n_heads,
+                                                        n_kv_heads, head_dim, kcache.shape[1], pos0,
+                                                        _ptr(scratch), scratch.numel(), _stream()),
+           "w4a32_op_rope_attention_prefill_bf16x3")
     return out
 
 

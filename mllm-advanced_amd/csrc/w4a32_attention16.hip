@@ -75,33 +75,13 @@ constexpr int kBlkBytes = 24 * kOpBytes;      // the 24 K operands (or the 24 V 
 __device__ __forceinline__ int k_op(int s, int t) { return s * 3 + t; }
 __device__ __forceinline__ int v_op(int t, int c, int ks) { return (t * 4 + c) * 2 + ks; }
 
-// grid (key blocks of 32, kv heads), 256 threads: thread (key = t / 8, 16 dims = one k-step)
-__global__ __launch_bounds__(256) void split_kv_kernel(const float* __restrict__ kc, const float* __restrict__ vc,
-                                                       uint8_t* __restrict__ ks, uint8_t* __restrict__ vts,
-                                                       int n_keys, int max_seq, int NKB) {
-  __shared__ __align__(16) uint16_t s_v[3][kHd][32];
-  const int kb = blockIdx.x, hk = blockIdx.y;
-  const int key_l = threadIdx.x >> 3, sstep = threadIdx.x & 7, d0 = 16 * sstep;
-  const int key = 32 * kb + key_l;
-  const bool real = key < n_keys;
-  const size_t src = ((size_t)hk * max_seq + (real ? key : 0)) * kHd + d0;
-  float kx[16], vx[16];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const float4 a = *reinterpret_cast<const float4*>(kc + src + 4 * i);
-    const float4 b = *reinterpret_cast<const float4*>(vc + src + 4 * i);
-    kx[4 * i] = a.x; kx[4 * i + 1] = a.y; kx[4 * i + 2] = a.z; kx[4 * i + 3] = a.w;
-    vx[4 * i] = b.x; vx[4 * i + 1] = b.y; vx[4 * i + 2] = b.z; vx[4 * i + 3] = b.w;
-  }
-  if (!real) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      kx[i] = 0.0f;
-      vx[i] = 0.0f;
-    }
-  }
+// The 16 dims (k-step sstep) of key key_l of a 32-key block, K and V, into the block's operands: called by all
+// 256 threads of a workgroup (thread = (key_l = t / 8, sstep = t % 8)); s_v is the workgroup's transpose buffer.
+__device__ __forceinline__ void store_block_operands(const float (&kx)[16], const float (&vx)[16], int key_l,
+                                                     int sstep, uint8_t* __restrict__ kblk,
+                                                     uint8_t* __restrict__ vblk, uint16_t (&s_v)[3][kHd][32]) {
+  const int d0 = 16 * sstep;
   // K operands of k-step sstep: the thread's 16 dims are the two halves (h = 0, 1) of lane key_l
-  uint8_t* kblk = ks + ((size_t)hk * NKB + kb) * kBlkBytes;
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
     float x8[8];
@@ -127,13 +107,132 @@ __global__ __launch_bounds__(256) void split_kv_kernel(const float* __restrict__
   __syncthreads();
   // 24 operands of 64 lanes: item u = operand * 64 + lane; lane (h, j) of operand (t, c, ks) is dim 32 c + j,
   // positions 16 ks + 8 h .. + 7
-  uint8_t* vblk = vts + ((size_t)hk * NKB + kb) * kBlkBytes;
   for (int u = threadIdx.x; u < 24 * 64; u += 256) {
     const int op = u >> 6, l = u & 63;
     const int ksx = op & 1, c = (op >> 1) & 3, t = op >> 3;
     const uint4 v = *reinterpret_cast<const uint4*>(&s_v[t][32 * c + (l & 31)][16 * ksx + 8 * (l >> 5)]);
     *reinterpret_cast<uint4*>(vblk + (size_t)u * 16) = v;
   }
+}
+
+__device__ __forceinline__ void load16(const float* __restrict__ src, float (&x)[16]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float4 a = *reinterpret_cast<const float4*>(src + 4 * i);
+    x[4 * i] = a.x; x[4 * i + 1] = a.y; x[4 * i + 2] = a.z; x[4 * i + 3] = a.w;
+  }
+}
+__device__ __forceinline__ void store16(float* __restrict__ dst, const float (&x)[16]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    *reinterpret_cast<float4*>(dst + 4 * i) = make_float4(x[4 * i], x[4 * i + 1], x[4 * i + 2], x[4 * i + 3]);
+  }
+}
+
+// grid (key blocks of 32, kv heads), 256 threads: thread (key = t / 8, 16 dims = one k-step)
+__global__ __launch_bounds__(256) void split_kv_kernel(const float* __restrict__ kc, const float* __restrict__ vc,
+                                                       uint8_t* __restrict__ ks, uint8_t* __restrict__ vts,
+                                                       int n_keys, int max_seq, int NKB) {
+  __shared__ __align__(16) uint16_t s_v[3][kHd][32];
+  const int kb = blockIdx.x, hk = blockIdx.y;
+  const int key_l = threadIdx.x >> 3, sstep = threadIdx.x & 7, d0 = 16 * sstep;
+  const int key = 32 * kb + key_l;
+  const bool real = key < n_keys;
+  const size_t src = ((size_t)hk * max_seq + (real ? key : 0)) * kHd + d0;
+  float kx[16], vx[16];
+  load16(kc + src, kx);
+  load16(vc + src, vx);
+  if (!real) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      kx[i] = 0.0f;
+      vx[i] = 0.0f;
+    }
+  }
+  const size_t blk = ((size_t)hk * NKB + kb) * kBlkBytes;
+  store_block_operands(kx, vx, key_l, sstep, ks + blk, vts + blk, s_v);
+}
+
+// rope_kv_kernel (w4a32_glue.hip) and split_kv_kernel in one launch, for a prefill that runs attention16_kernel
+// next: grid (key blocks of 32, Hkv + Hq), 256 threads.
+//   blockIdx.y <  Hkv: the operand blocks of kv head blockIdx.y. A key below pos0 comes from the caches as they
+//                      are; key pos0 + m is row m of k (rotated here, the arithmetic of rope_kv_kernel) and of v,
+//                      and is also appended to the caches; keys from n_keys on are zeros.
+//   blockIdx.y >= Hkv: rotates rows 32 blockIdx.x .. + 31 of query head blockIdx.y - Hkv in place; a thread owns
+//                      dims 8 i .. 8 i + 7 and their partners 64 + 8 i .. (nobody else reads what it writes).
+__global__ __launch_bounds__(256) void rope_split_kv_kernel(
+    float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
+    const float* __restrict__ sin_t, const float* __restrict__ cos_t, float* __restrict__ kc,
+    float* __restrict__ vc, uint8_t* __restrict__ ks, uint8_t* __restrict__ vts, int M, int Hq, int Hkv,
+    int pos0, int max_seq, int NKB) {
+  __shared__ __align__(16) uint16_t s_v[3][kHd][32];
+  constexpr int kHalf = kHd / 2;
+  const int kb = blockIdx.x;
+  const int row_l = threadIdx.x >> 3, sstep = threadIdx.x & 7;
+  if ((int)blockIdx.y >= Hkv) {
+    const int h = blockIdx.y - Hkv, m = 32 * kb + row_l;
+    if (m >= M) return;
+    float* x = q + ((size_t)m * Hq + h) * kHd + 8 * sstep;
+    const float* st = sin_t + (size_t)(pos0 + m) * kHalf + 8 * sstep;
+    const float* ct = cos_t + (size_t)(pos0 + m) * kHalf + 8 * sstep;
+    const float4 a0 = *reinterpret_cast<const float4*>(x), a1 = *reinterpret_cast<const float4*>(x + 4);
+    const float4 b0 = *reinterpret_cast<const float4*>(x + kHalf), b1 = *reinterpret_cast<const float4*>(x + kHalf + 4);
+    const float4 s0 = *reinterpret_cast<const float4*>(st), s1 = *reinterpret_cast<const float4*>(st + 4);
+    const float4 c0 = *reinterpret_cast<const float4*>(ct), c1 = *reinterpret_cast<const float4*>(ct + 4);
+    const float x0[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+    const float x1[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+    const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+    const float cs[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+    float y0[8], y1[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      y0[e] = x0[e] * cs[e] - x1[e] * sn[e];
+      y1[e] = x0[e] * sn[e] + x1[e] * cs[e];
+    }
+    *reinterpret_cast<float4*>(x) = make_float4(y0[0], y0[1], y0[2], y0[3]);
+    *reinterpret_cast<float4*>(x + 4) = make_float4(y0[4], y0[5], y0[6], y0[7]);
+    *reinterpret_cast<float4*>(x + kHalf) = make_float4(y1[0], y1[1], y1[2], y1[3]);
+    *reinterpret_cast<float4*>(x + kHalf + 4) = make_float4(y1[4], y1[5], y1[6], y1[7]);
+    return;
+  }
+  const int hk = blockIdx.y, d0 = 16 * sstep;
+  const int key = 32 * kb + row_l;
+  const int n_keys = pos0 + M;
+  float kx[16], vx[16];
+  if (key >= n_keys) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      kx[i] = 0.0f;
+      vx[i] = 0.0f;
+    }
+  } else if (key < pos0) {
+    const size_t src = ((size_t)hk * max_seq + key) * kHd + d0;
+    load16(kc + src, kx);
+    load16(vc + src, vx);
+  } else {
+    const int m = key - pos0;
+    const size_t src = ((size_t)m * Hkv + hk) * kHd;
+    // this thread's 16 dims and their partners in the other half of the head vector
+    const int dp = d0 < kHalf ? d0 + kHalf : d0 - kHalf, dt = d0 < kHalf ? d0 : d0 - kHalf;
+    float own[16], par[16], sn[16], cs[16];
+    load16(k + src + d0, own);
+    load16(k + src + dp, par);
+    load16(sin_t + (size_t)key * kHalf + dt, sn);
+    load16(cos_t + (size_t)key * kHalf + dt, cs);
+    load16(v + src + d0, vx);
+    if (d0 < kHalf) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) kx[i] = own[i] * cs[i] - par[i] * sn[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) kx[i] = par[i] * sn[i] + own[i] * cs[i];
+    }
+    const size_t dst = ((size_t)hk * max_seq + key) * kHd + d0;
+    store16(kc + dst, kx);
+    store16(vc + dst, vx);
+  }
+  const size_t blk = ((size_t)hk * NKB + kb) * kBlkBytes;
+  store_block_operands(kx, vx, row_l, sstep, ks + blk, vts + blk, s_v);
 }
 
 template <int kWaves>
@@ -338,10 +437,22 @@ __global__ __launch_bounds__(64 * kWaves) void attention16_kernel(
 
 }  // namespace
 
-// bytes of Ks + VTs for n_keys keys
 // bytes of the K and V operands for n_keys keys
 size_t attention16_scratch_bytes(int n_keys, int Hkv) {
   return 2 * (size_t)Hkv * ((n_keys + 31) / 32) * kBlkBytes;
+}
+
+static hipError_t launch_attention16_products(const float* q, const uint8_t* ks, const uint8_t* vts, float* out,
+                                              int M, int Hq, int Hkv, int NKB, int pos0, hipStream_t s) {
+  const float scale = 1.0f / sqrtf((float)kHd);
+  constexpr size_t kQBytes = 8 * 3 * 64 * 16;
+  constexpr int W = 4;  // one wavefront per SIMD: its operand prefetch takes most of the register file
+  const size_t lds = kQBytes + sizeof(float) * (W - 1) * 66 * 64;
+  static LdsLimitOnce raised;  // above the default limit of dynamic LDS
+  if (hipError_t e = raised.raise(reinterpret_cast<const void*>(attention16_kernel<W>), lds); e != hipSuccess) return e;
+  hipLaunchKernelGGL((attention16_kernel<W>), dim3(Hq, (M + 31) / 32), dim3(64 * W), lds, s, q, ks, vts, out, M, Hq,
+                     Hkv, NKB, pos0, scale);
+  return hipGetLastError();
 }
 
 hipError_t launch_attention16(const float* q, const float* kc, const float* vc, float* out, int M, int Hq, int Hkv,
@@ -352,15 +463,20 @@ hipError_t launch_attention16(const float* q, const float* kc, const float* vc, 
   uint8_t* vts = scratch + (size_t)Hkv * NKB * kBlkBytes;
   hipLaunchKernelGGL(split_kv_kernel, dim3(NKB, Hkv), dim3(256), 0, s, kc, vc, ks, vts, n_keys, max_seq, NKB);
   if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
-  const float scale = 1.0f / sqrtf((float)kHd);
-  constexpr size_t kQBytes = 8 * 3 * 64 * 16;
-  constexpr int W = 4;  // one wavefront per SIMD: its operand prefetch takes most of the register file
-  const size_t lds = kQBytes + sizeof(float) * (W - 1) * 66 * 64;
-  static LdsLimitOnce raised;  // above the default limit of dynamic LDS
-  if (hipError_t e = raised.raise(reinterpret_cast<const void*>(attention16_kernel<W>), lds); e != hipSuccess) return e;
-  hipLaunchKernelGGL((attention16_kernel<W>), dim3(Hq, (M + 31) / 32), dim3(64 * W), lds, s, q, ks, vts, out, M, Hq,
-                     Hkv, NKB, pos0, scale);
-  return hipGetLastError();
+  return launch_attention16_products(q, ks, vts, out, M, Hq, Hkv, NKB, pos0, s);
+}
+
+hipError_t launch_rope_attention16(float* q, const float* k, const float* v, const float* sin_t,
+                                   const float* cos_t, float* kc, float* vc, float* out, int M, int Hq, int Hkv,
+                                   int max_seq, int pos0, uint8_t* scratch, hipStream_t s) {
+  const int n_keys = pos0 + M;
+  const int NKB = (n_keys + 31) / 32;
+  uint8_t* ks = scratch;
+  uint8_t* vts = scratch + (size_t)Hkv * NKB * kBlkBytes;
+  hipLaunchKernelGGL(rope_split_kv_kernel, dim3(NKB, Hkv + Hq), dim3(256), 0, s, q, k, v, sin_t, cos_t, kc, vc, ks,
+                     vts, M, Hq, Hkv, pos0, max_seq, NKB);
+  if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+  return launch_attention16_products(q, ks, vts, out, M, Hq, Hkv, NKB, pos0, s);
 }
 
 }  // namespace w4

@@ -174,27 +174,29 @@ int run_layers(const w4a32_decoder_config* c, const w4a32_decoder_weights* w, ui
         W4_TRY(w4a32_matmul_grouped(ys, xn, ps, ns, 3, ws, M, H, stream));
       }
     }
-    W4_TRY(from_hip(w4::launch_rope_kv(q, k, v, sin_t, cos_t, kc, vc, M, Hq, Hkv, D, c->max_seq, d_pos,
-                                       0, s)));
-    if (M == 1) {
+    // a prefill knows its position on the host; from kAttn16MinRows rows on the matrix-pipe attention kernel is
+    // the faster one, and its operand split does the rotation and the cache append on the way. The gate and up
+    // buffers are dead here: they hold the bf16 terms of K and V.
+    const bool attn16 = M > 1 && host_pos0 >= 0 && M >= kAttn16MinRows && D == 128 &&
+                        w4::attention16_scratch_bytes(host_pos0 + M, Hkv) <= lend;
+    if (!attn16) {
+      W4_TRY(from_hip(w4::launch_rope_kv(q, k, v, sin_t, cos_t, kc, vc, M, Hq, Hkv, D, c->max_seq, d_pos,
+                                         0, s)));
+    }
+    if (attn16) {
+      W4_TRY(from_hip(w4::launch_rope_attention16(q, k, v, sin_t, cos_t, kc, vc, attn, M, Hq, Hkv, c->max_seq,
+                                                  host_pos0, reinterpret_cast<uint8_t*>(gate), s)));
+    } else if (M == 1) {
       W4_TRY(from_hip(w4::launch_attention_decode(
           q, kc, vc, attn, Hq, Hkv, c->max_seq, d_pos, 0, kAttnSplit,
           reinterpret_cast<float*>(scratch + sg.part_off),
           reinterpret_cast<unsigned int*>(scratch + sg.counters_off), nullptr, nullptr, nullptr, nullptr, false,
           s)));
     } else {
-      // the gate and up buffers are dead here: they hold the bf16 terms of K and V for the matrix-pipe kernel
-      // (a prefill knows its position on the host; from kAttn16MinRows rows on that kernel is the faster one),
-      // or the per-chunk results of long query blocks for the f32 kernel
-      if (host_pos0 >= 0 && M >= kAttn16MinRows &&
-          w4::attention16_scratch_bytes(host_pos0 + M, Hkv) <= lend) {
-        W4_TRY(from_hip(w4::launch_attention16(q, kc, vc, attn, M, Hq, Hkv, c->max_seq, host_pos0,
-                                               reinterpret_cast<uint8_t*>(gate), s)));
-      } else {
-        W4_TRY(from_hip(w4::launch_attention_prefill(q, kc, vc, attn, M, Hq, Hkv, c->max_seq, d_pos, 0, gate,
-                                                     lend, reinterpret_cast<unsigned int*>(st + g.pfcnt_off),
-                                                     s)));
-      }
+      // the gate and up buffers are dead here: they hold the per-chunk results of long query blocks
+      W4_TRY(from_hip(w4::launch_attention_prefill(q, kc, vc, attn, M, Hq, Hkv, c->max_seq, d_pos, 0, gate,
+                                                   lend, reinterpret_cast<unsigned int*>(st + g.pfcnt_off),
+                                                   s)));
     }
     W4_TRY(w4a32_matmul(delta, attn, lw.o, ws, M, qd, H, stream));
     // h += attention output; xn = norm(h)
@@ -563,6 +565,28 @@ int w4a32_op_attention_prefill_bf16x3(const float* d_q, const float* d_kcache, c
   if (scratch_bytes < w4::attention16_scratch_bytes(pos0 + M, n_kv_heads)) return W4A32_EINVAL;
   return from_hip(w4::launch_attention16(d_q, d_kcache, d_vcache, d_out, M, n_heads, n_kv_heads, max_seq, pos0,
                                          static_cast<uint8_t*>(d_scratch), S(stream)));
+}
+
+int w4a32_op_rope_attention_prefill_bf16x3(float* d_q, const float* d_k, const float* d_v, const float* d_sin,
+                                           const float* d_cos, float* d_kcache, float* d_vcache, float* d_out,
+                                           int M, int n_heads, int n_kv_heads, int head_dim, int max_seq,
+                                           int pos0, void* d_scratch, size_t scratch_bytes, void* stream) {
+  if (!d_q || !d_k || !d_v || !d_sin || !d_cos || !d_kcache || !d_vcache || !d_out || !d_scratch)
+    return W4A32_EINVAL;
+  if (M <= 0 || n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0) return W4A32_EINVAL;
+  if (head_dim != 128 || n_heads % n_kv_heads != 0) return W4A32_ESHAPE;
+  if (pos0 < 0 || pos0 + M > max_seq) return W4A32_ESHAPE;
+  for (const void* p : {static_cast<const void*>(d_q), static_cast<const void*>(d_k),
+                        static_cast<const void*>(d_v), static_cast<const void*>(d_sin),
+                        static_cast<const void*>(d_cos), static_cast<const void*>(d_kcache),
+                        static_cast<const void*>(d_vcache), static_cast<const void*>(d_out),
+                        static_cast<const void*>(d_scratch)}) {
+    if (reinterpret_cast<uintptr_t>(p) % 16 != 0) return W4A32_EINVAL;
+  }
+  if (scratch_bytes < w4::attention16_scratch_bytes(pos0 + M, n_kv_heads)) return W4A32_EINVAL;
+  return from_hip(w4::launch_rope_attention16(d_q, d_k, d_v, d_sin, d_cos, d_kcache, d_vcache, d_out, M, n_heads,
+                                              n_kv_heads, max_seq, pos0, static_cast<uint8_t*>(d_scratch),
+                                              S(stream)));
 }
 
 int w4a32_op_rope_attention_decode(const float* d_q, const float* d_k, const float* d_v,

@@ -764,7 +764,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_batched_kernel(
   constexpr bool kPreq = kR == 0;
   constexpr int kTasks = kPreq ? 1 : kR;
   const int Kp = KC * kTileK;
-  const int grp_per_row = Kp >> 3, groups = K >> 3;
+  const int grp_per_row = Kp >> 3;
   const int nseg = (grp_per_row + 63) >> 6;       // 64-group segments per row (at most 8 when quantising here)
   const int ntask = M * nseg;
   int8_t* s_a = reinterpret_cast<int8_t*>(smem);                               // [Kp / 32][M][32]

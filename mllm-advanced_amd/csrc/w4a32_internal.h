@@ -120,6 +120,11 @@ hipError_t launch_attention_prefill(const float* q, const float* kc, const float
 size_t attention16_scratch_bytes(int n_keys, int Hkv);
 hipError_t launch_attention16(const float* q, const float* kc, const float* vc, float* out, int M, int Hq, int Hkv,
                               int max_seq, int pos0, uint8_t* scratch, hipStream_t s);
+// launch_rope_kv at a position known on the host + launch_attention16, with the rotation, the cache append and the
+// operand split in one launch (head_dim 128)
+hipError_t launch_rope_attention16(float* q, const float* k, const float* v, const float* sin_t,
+                                   const float* cos_t, float* kc, float* vc, float* out, int M, int Hq, int Hkv,
+                                   int max_seq, int pos0, uint8_t* scratch, hipStream_t s);
 hipError_t launch_attention_bshd(const float* q, const float* k, const float* v, float* out, int M, int Hq,
                                  int Hkv, int n_keys, int pos0, hipStream_t s);
 // operators of the engine's op-by-op path (w4a32_engine_ops.hip)

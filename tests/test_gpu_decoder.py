@@ -240,6 +240,32 @@ def test_attention_prefill_on_bf16_terms(pkg, Hq, Hkv):
 
 
 @pytest.mark.parametrize("Hq,Hkv", [(12, 2), (4, 4), (3, 1)])
+def test_rope_attention_prefill_on_bf16_terms_equals_the_two_operators(pkg, Hq, Hkv):
+    """RoPE + cache append done by the launch that splits K and V == op_rope_kv, then op_attention_prefill_bf16x3:
+    rotated q, both caches (rows outside [pos0, pos0 + M) untouched) and the output, bit for bit; positions that
+    start inside a 32-key block, ragged row counts, a prompt that ends at the cache's last row."""
+    g = torch.Generator(device="cuda").manual_seed(8)
+    D, S = 128, 640
+    sin, cos = pkg.op_rope_table(S, D, 1e6)
+    for M, pos0 in [(1, 0), (32, 0), (70, 0), (256, 0), (512, 0), (100, 32), (130, 5), (64, 300), (37, 603),
+                    (128, 512)]:
+        kc = torch.randn((Hkv, S, D), generator=g, device="cuda")
+        vc = torch.randn((Hkv, S, D), generator=g, device="cuda")
+        q = torch.randn((M, Hq * D), generator=g, device="cuda")
+        k = torch.randn((M, Hkv * D), generator=g, device="cuda")
+        v = torch.randn((M, Hkv * D), generator=g, device="cuda")
+        kc1, vc1, q1 = kc.clone(), vc.clone(), q.clone()
+        pkg.op_rope_kv(q1, k, v, sin, cos, kc1, vc1, Hq, Hkv, D, pos0)
+        want = pkg.op_attention_prefill_bf16x3(q1, kc1, vc1, Hq, Hkv, D, pos0)
+        kc2, vc2, q2 = kc.clone(), vc.clone(), q.clone()
+        got = pkg.op_rope_attention_prefill_bf16x3(q2, k, v, sin, cos, kc2, vc2, Hq, Hkv, D, pos0)
+        torch.cuda.synchronize()
+        assert torch.equal(q2, q1), (M, pos0)
+        assert torch.equal(kc2, kc1) and torch.equal(vc2, vc1), (M, pos0)
+        assert torch.equal(got, want), (M, pos0)
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(12, 2), (4, 4), (3, 1)])
 def test_rope_attention_decode_equals_the_two_operators(pkg, Hq, Hkv):
     g = torch.Generator(device="cuda").manual_seed(6)
     D, S = 128, 256
