@@ -75,13 +75,10 @@ constexpr int kBlkBytes = 24 * kOpBytes;      // the 24 K operands (or the 24 V 
 __device__ __forceinline__ int k_op(int s, int t) { return s * 3 + t; }
 __device__ __forceinline__ int v_op(int t, int c, int ks) { return (t * 4 + c) * 2 + ks; }
 
-// The 16 dims (k-step sstep) of key key_l of a 32-key block, K and V, into the block's operands: called by all
-// 256 threads of a workgroup (thread = (key_l = t / 8, sstep = t % 8)); s_v is the workgroup's transpose buffer.
-__device__ __forceinline__ void store_block_operands(const float (&kx)[16], const float (&vx)[16], int key_l,
-                                                     int sstep, uint8_t* __restrict__ kblk,
-                                                     uint8_t* __restrict__ vblk, uint16_t (&s_v)[3][kHd][32]) {
-  const int d0 = 16 * sstep;
-  // K operands of k-step sstep: the thread's 16 dims are the two halves (h = 0, 1) of lane key_l
+// K operands of one 32-key block: called by 256 threads, thread = (key_l = t / 8, sstep = t % 8) holds the 16
+// dims of k-step sstep of key key_l, which are the two halves (h = 0, 1) of lane key_l of that k-step's operands.
+__device__ __forceinline__ void store_k_operands(const float (&kx)[16], int key_l, int sstep,
+                                                 uint8_t* __restrict__ kblk) {
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
     float x8[8];
@@ -94,24 +91,35 @@ __device__ __forceinline__ void store_block_operands(const float (&kx)[16], cons
       *reinterpret_cast<uint4*>(kblk + (size_t)k_op(sstep, k) * kOpBytes + (32 * half + key_l) * 16) = terms[k];
     }
   }
-  // V: transposed through LDS, keys of a group of 16 in operand order
-  const int pos = 16 * (key_l >> 4) + vt_pos(key_l & 15);
+}
+
+// V^T operands of one 32-key block, read transposed: called by 256 threads, thread = (dim d = t % 128, h = t / 128)
+// is lane (h, d % 32) of the operands of dim block d / 32; for k-step ks it holds the block's keys
+// 16 ks + 4 h + {0, 1, 2, 3, 8, 9, 10, 11} (positions 16 ks + 8 h .. + 7 in operand order, see the file header).
+// The 64 lanes of a load are 64 consecutive dims of one key: one coalesced 256-byte read; nothing goes through
+// LDS. `row(key_in_block)` returns the address of that key's V row (any valid row for a key past the last one) and
+// `keep(key_in_block, d, x)` the value to use (0 past the last key; it may append x to the cache). All 16 loads
+// are issued before the first result is looked at.
+template <typename Row, typename Keep>
+__device__ __forceinline__ void store_v_operands(Row row, Keep keep, uint8_t* __restrict__ vblk) {
+  const int d = threadIdx.x & 127, h = threadIdx.x >> 7;
+  float x[2][8];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    uint32_t t1, t2, t3;
-    split3(vx[i], t1, t2, t3);
-    s_v[0][d0 + i][pos] = (uint16_t)(t1 >> 16);
-    s_v[1][d0 + i][pos] = (uint16_t)(t2 >> 16);
-    s_v[2][d0 + i][pos] = (uint16_t)(t3 >> 16);
-  }
-  __syncthreads();
-  // 24 operands of 64 lanes: item u = operand * 64 + lane; lane (h, j) of operand (t, c, ks) is dim 32 c + j,
-  // positions 16 ks + 8 h .. + 7
-  for (int u = threadIdx.x; u < 24 * 64; u += 256) {
-    const int op = u >> 6, l = u & 63;
-    const int ksx = op & 1, c = (op >> 1) & 3, t = op >> 3;
-    const uint4 v = *reinterpret_cast<const uint4*>(&s_v[t][32 * c + (l & 31)][16 * ksx + 8 * (l >> 5)]);
-    *reinterpret_cast<uint4*>(vblk + (size_t)u * 16) = v;
+  for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[ks][e] = row(16 * ks + 4 * h + 8 * (e >> 2) + (e & 3))[d];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[ks][e] = keep(16 * ks + 4 * h + 8 * (e >> 2) + (e & 3), d, x[ks][e]);
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+    uint4 terms[3];
+    split3x8(x[ks], terms);
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      *reinterpret_cast<uint4*>(vblk + (size_t)v_op(k, d >> 5, ks) * kOpBytes + (32 * h + (d & 31)) * 16) = terms[k];
+    }
   }
 }
 
@@ -129,48 +137,56 @@ __device__ __forceinline__ void store16(float* __restrict__ dst, const float (&x
   }
 }
 
-// grid (key blocks of 32, kv heads), 256 threads: thread (key = t / 8, 16 dims = one k-step)
+// grid (key blocks of 32, 2 * kv heads), 256 threads: blockIdx.y < Hkv writes the K operands of a block,
+// the others its V^T operands
 __global__ __launch_bounds__(256) void split_kv_kernel(const float* __restrict__ kc, const float* __restrict__ vc,
                                                        uint8_t* __restrict__ ks, uint8_t* __restrict__ vts,
-                                                       int n_keys, int max_seq, int NKB) {
-  __shared__ __align__(16) uint16_t s_v[3][kHd][32];
-  const int kb = blockIdx.x, hk = blockIdx.y;
-  const int key_l = threadIdx.x >> 3, sstep = threadIdx.x & 7, d0 = 16 * sstep;
-  const int key = 32 * kb + key_l;
-  const bool real = key < n_keys;
-  const size_t src = ((size_t)hk * max_seq + (real ? key : 0)) * kHd + d0;
-  float kx[16], vx[16];
-  load16(kc + src, kx);
-  load16(vc + src, vx);
-  if (!real) {
+                                                       int n_keys, int max_seq, int NKB, int Hkv) {
+  const int kb = blockIdx.x;
+  if ((int)blockIdx.y < Hkv) {
+    const int hk = blockIdx.y;
+    const int key_l = threadIdx.x >> 3, sstep = threadIdx.x & 7;
+    const int key = 32 * kb + key_l;
+    float kx[16];
+    load16(kc + ((size_t)hk * max_seq + (key < n_keys ? key : 0)) * kHd + 16 * sstep, kx);
+    if (key >= n_keys) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      kx[i] = 0.0f;
-      vx[i] = 0.0f;
+      for (int i = 0; i < 16; ++i) kx[i] = 0.0f;
     }
+    store_k_operands(kx, key_l, sstep, ks + ((size_t)hk * NKB + kb) * kBlkBytes);
+    return;
   }
-  const size_t blk = ((size_t)hk * NKB + kb) * kBlkBytes;
-  store_block_operands(kx, vx, key_l, sstep, ks + blk, vts + blk, s_v);
+  const int hk = blockIdx.y - Hkv;
+  const float* vrow = vc + (size_t)hk * max_seq * kHd;
+  store_v_operands(
+      [&](int kl) {
+        const int key = 32 * kb + kl;  // wavefront-uniform
+        return vrow + (size_t)(key < n_keys ? key : 0) * kHd;
+      },
+      [&](int kl, int, float x) { return 32 * kb + kl < n_keys ? x : 0.0f; },
+      vts + ((size_t)hk * NKB + kb) * kBlkBytes);
 }
 
 // rope_kv_kernel (w4a32_glue.hip) and split_kv_kernel in one launch, for a prefill that runs attention16_kernel
-// next: grid (key blocks of 32, Hkv + Hq), 256 threads.
-//   blockIdx.y <  Hkv: the operand blocks of kv head blockIdx.y. A key below pos0 comes from the caches as they
-//                      are; key pos0 + m is row m of k (rotated here, the arithmetic of rope_kv_kernel) and of v,
-//                      and is also appended to the caches; keys from n_keys on are zeros.
-//   blockIdx.y >= Hkv: rotates rows 32 blockIdx.x .. + 31 of query head blockIdx.y - Hkv in place; a thread owns
-//                      dims 8 i .. 8 i + 7 and their partners 64 + 8 i .. (nobody else reads what it writes).
+// next: grid (key blocks of 32, 2 * Hkv + Hq), 256 threads.
+//   blockIdx.y <  Hkv:     the K operands of kv head blockIdx.y. A key below pos0 comes from the cache as it is;
+//                          key pos0 + m is row m of k, rotated here (the arithmetic of rope_kv_kernel) and also
+//                          appended to the cache; keys from n_keys on are zeros.
+//   blockIdx.y <  2 Hkv:   the V^T operands likewise (row m of v, appended to the cache).
+//   otherwise:             rotates rows 32 blockIdx.x .. + 31 of query head blockIdx.y - 2 Hkv in place; a thread
+//                          owns dims 8 i .. 8 i + 7 and their partners 64 + 8 i .. (nobody else reads what it
+//                          writes).
 __global__ __launch_bounds__(256) void rope_split_kv_kernel(
     float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
     const float* __restrict__ sin_t, const float* __restrict__ cos_t, float* __restrict__ kc,
     float* __restrict__ vc, uint8_t* __restrict__ ks, uint8_t* __restrict__ vts, int M, int Hq, int Hkv,
     int pos0, int max_seq, int NKB) {
-  __shared__ __align__(16) uint16_t s_v[3][kHd][32];
   constexpr int kHalf = kHd / 2;
   const int kb = blockIdx.x;
   const int row_l = threadIdx.x >> 3, sstep = threadIdx.x & 7;
-  if ((int)blockIdx.y >= Hkv) {
-    const int h = blockIdx.y - Hkv, m = 32 * kb + row_l;
+  const int n_keys = pos0 + M;
+  if ((int)blockIdx.y >= 2 * Hkv) {
+    const int h = blockIdx.y - 2 * Hkv, m = 32 * kb + row_l;
     if (m >= M) return;
     float* x = q + ((size_t)m * Hq + h) * kHd + 8 * sstep;
     const float* st = sin_t + (size_t)(pos0 + m) * kHalf + 8 * sstep;
@@ -195,23 +211,35 @@ __global__ __launch_bounds__(256) void rope_split_kv_kernel(
     *reinterpret_cast<float4*>(x + kHalf + 4) = make_float4(y1[4], y1[5], y1[6], y1[7]);
     return;
   }
+  if ((int)blockIdx.y >= Hkv) {
+    const int hk = blockIdx.y - Hkv;
+    float* vcache = vc + (size_t)hk * max_seq * kHd;
+    store_v_operands(
+        [&](int kl) {
+          const int key = 32 * kb + kl;  // wavefront-uniform
+          const float* cached = vcache + (size_t)(key < pos0 ? key : 0) * kHd;
+          const float* fresh = v + ((size_t)(key >= pos0 && key < n_keys ? key - pos0 : 0) * Hkv + hk) * kHd;
+          return key < pos0 ? cached : fresh;
+        },
+        [&](int kl, int d, float x) {
+          const int key = 32 * kb + kl;
+          if (key >= n_keys) return 0.0f;
+          if (key >= pos0) vcache[(size_t)key * kHd + d] = x;
+          return x;
+        },
+        vts + ((size_t)hk * NKB + kb) * kBlkBytes);
+    return;
+  }
   const int hk = blockIdx.y, d0 = 16 * sstep;
   const int key = 32 * kb + row_l;
-  const int n_keys = pos0 + M;
-  float kx[16], vx[16];
+  float kx[16];
   if (key >= n_keys) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      kx[i] = 0.0f;
-      vx[i] = 0.0f;
-    }
+    for (int i = 0; i < 16; ++i) kx[i] = 0.0f;
   } else if (key < pos0) {
-    const size_t src = ((size_t)hk * max_seq + key) * kHd + d0;
-    load16(kc + src, kx);
-    load16(vc + src, vx);
+    load16(kc + ((size_t)hk * max_seq + key) * kHd + d0, kx);
   } else {
-    const int m = key - pos0;
-    const size_t src = ((size_t)m * Hkv + hk) * kHd;
+    const size_t src = ((size_t)(key - pos0) * Hkv + hk) * kHd;
     // this thread's 16 dims and their partners in the other half of the head vector
     const int dp = d0 < kHalf ? d0 + kHalf : d0 - kHalf, dt = d0 < kHalf ? d0 : d0 - kHalf;
     float own[16], par[16], sn[16], cs[16];
@@ -219,7 +247,6 @@ __global__ __launch_bounds__(256) void rope_split_kv_kernel(
     load16(k + src + dp, par);
     load16(sin_t + (size_t)key * kHalf + dt, sn);
     load16(cos_t + (size_t)key * kHalf + dt, cs);
-    load16(v + src + d0, vx);
     if (d0 < kHalf) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) kx[i] = own[i] * cs[i] - par[i] * sn[i];
@@ -227,12 +254,9 @@ __global__ __launch_bounds__(256) void rope_split_kv_kernel(
 #pragma unroll
       for (int i = 0; i < 16; ++i) kx[i] = par[i] * sn[i] + own[i] * cs[i];
     }
-    const size_t dst = ((size_t)hk * max_seq + key) * kHd + d0;
-    store16(kc + dst, kx);
-    store16(vc + dst, vx);
+    store16(kc + ((size_t)hk * max_seq + key) * kHd + d0, kx);
   }
-  const size_t blk = ((size_t)hk * NKB + kb) * kBlkBytes;
-  store_block_operands(kx, vx, row_l, sstep, ks + blk, vts + blk, s_v);
+  store_k_operands(kx, row_l, sstep, ks + ((size_t)hk * NKB + kb) * kBlkBytes);
 }
 
 template <int kWaves>
@@ -461,7 +485,7 @@ hipError_t launch_attention16(const float* q, const float* kc, const float* vc, 
   const int NKB = (n_keys + 31) / 32;
   uint8_t* ks = scratch;
   uint8_t* vts = scratch + (size_t)Hkv * NKB * kBlkBytes;
-  hipLaunchKernelGGL(split_kv_kernel, dim3(NKB, Hkv), dim3(256), 0, s, kc, vc, ks, vts, n_keys, max_seq, NKB);
+  hipLaunchKernelGGL(split_kv_kernel, dim3(NKB, 2 * Hkv), dim3(256), 0, s, kc, vc, ks, vts, n_keys, max_seq, NKB, Hkv);
   if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
   return launch_attention16_products(q, ks, vts, out, M, Hq, Hkv, NKB, pos0, s);
 }
@@ -473,7 +497,7 @@ hipError_t launch_rope_attention16(float* q, const float* k, const float* v, con
   const int NKB = (n_keys + 31) / 32;
   uint8_t* ks = scratch;
   uint8_t* vts = scratch + (size_t)Hkv * NKB * kBlkBytes;
-  hipLaunchKernelGGL(rope_split_kv_kernel, dim3(NKB, Hkv + Hq), dim3(256), 0, s, q, k, v, sin_t, cos_t, kc, vc, ks,
+  hipLaunchKernelGGL(rope_split_kv_kernel, dim3(NKB, 2 * Hkv + Hq), dim3(256), 0, s, q, k, v, sin_t, cos_t, kc, vc, ks,
                      vts, M, Hq, Hkv, pos0, max_seq, NKB);
   if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
   return launch_attention16_products(q, ks, vts, out, M, Hq, Hkv, NKB, pos0, s);
