@@ -276,44 +276,64 @@ struct GroupArgs {
 //   and stores silu(y0) * y1 to y[0] - or, with ga.pair_both, each output to its own y: two Linears of equal
 //   N on one row then take half the workgroups of the grouped form, each with twice the weight loads in
 //   flight (gate,up at K = 1536: 6.1 against 6.4 us).
-template <int M, int kFusedR, bool kGrouped, int kCPW, bool kNorm, bool kPair>
+template <int M, int kFusedR, bool kGrouped, int kCPW, bool kNorm, bool kPair, int kInParts = 1>
 __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
-    const float* __restrict__ x, int ldx, int K, int KC, int W, const uint8_t* packed0, int N0,
-    const float* pro_delta, const float* pro_norm_w, float pro_eps, float* y0,  // 16 dwords: preloaded
-    float* pro_sum_out, const GroupArgs ga) {
-  // The leading scalar arguments (everything a single Linear needs) are preloaded into SGPRs by
-  // the dispatcher, so the first loads go out without waiting for the argument segment.
+    const float* __restrict__ x, int ldx, unsigned kw, const uint8_t* packed0, unsigned long long firsts,
+    const float* pro_delta, const float* pro_norm_w, const uint8_t* packed1,
+    const uint8_t* packed2,  // 16 dwords: preloaded
+    float pro_eps, float* pro_sum_out, const GroupArgs ga) {
+  // The leading arguments (everything the first loads need: the row, the weights of up to three Linears and the
+  // tile rows at which one Linear ends and the next begins) are preloaded into SGPRs by the dispatcher, so the
+  // first loads go out without waiting for the argument segment; a read of that segment takes about half a
+  // microsecond, which is why nothing that is needed before the epilogue lives there (with the group's table
+  // read from it, a grouped launch cost 0.33 us more than a single Linear of the same size).
+  //   kw     = K | wavefronts << 16 | Linears << 24
+  //   firsts = first[1] | first[2] << 16 | first[3] << 32 | first[4] << 48 (tile rows, see GroupArgs)
   extern __shared__ __align__(16) uint8_t smem[];
   constexpr int kSets = kPair ? 2 : 1;  // weight matrices a workgroup multiplies
+  const int K = (int)(kw & 0xFFFFu), W = (int)((kw >> 16) & 31u);
+  const int KC = (K + kTileK - 1) / kTileK;
   const uint8_t* packed = packed0;
-  float* y = y0;
-  int N = N0, nt_first = 0;
+  int nt_first = 0, gi = 0;
+  int NT = (int)(firsts & 0xFFFFu);
   if (kGrouped) {
-    // Which Linear this workgroup belongs to. All four table entries are fetched first (the
-    // empty asm pins them in scalar registers) and then selected, so that the choice costs a
-    // few scalar ops instead of a second, dependent load from the argument segment.
-    const uint8_t* pk[kMaxGroup];
-    float* yy[kMaxGroup];
-    int nn[kMaxGroup], ff[kMaxGroup];
-#pragma unroll
-    for (int i = 0; i < kMaxGroup; ++i) {
-      pk[i] = ga.packed[i];
-      yy[i] = ga.y[i];
-      nn[i] = ga.N[i];
-      ff[i] = ga.first[i];
-      asm volatile("" : "+s"(pk[i]), "+s"(yy[i]), "+s"(nn[i]), "+s"(ff[i]));
+    // Which Linear this workgroup belongs to: from preloaded registers only. (A fourth Linear's weights come
+    // from the table.)
+    const int count = (int)(kw >> 24);
+    const int f1 = (int)(firsts & 0xFFFFu), f2 = (int)((firsts >> 16) & 0xFFFFu),
+              f3 = (int)((firsts >> 32) & 0xFFFFu), f4 = (int)(firsts >> 48);
+    const int b = (int)blockIdx.x;
+    if (count > 1 && b >= f1) {
+      packed = packed1;
+      nt_first = f1;
+      NT = f2 - f1;
+      gi = 1;
     }
+    if (count > 2 && b >= f2) {
+      packed = packed2;
+      nt_first = f2;
+      NT = f3 - f2;
+      gi = 2;
+    }
+    if (count > 3 && b >= f3) {
+      packed = ga.packed[3];
+      nt_first = f3;
+      NT = f4 - f3;
+      gi = 3;
+    }
+  }
+  // Output pointer and width of this workgroup's Linear: read from the argument segment now, used in the epilogue
+  float* y = ga.y[0];
+  int N = ga.N[0];
+  if (kGrouped) {
 #pragma unroll
     for (int i = 1; i < kMaxGroup; ++i) {
-      if (i < ga.count && (int)blockIdx.x >= ff[i]) {
-        packed = pk[i];
-        y = yy[i];
-        N = nn[i];
-        nt_first = ff[i];
+      if (gi == i) {
+        y = ga.y[i];
+        N = ga.N[i];
       }
     }
   }
-  const int NT = (N + kTileRows - 1) / kTileRows;
   const float* rsum = reinterpret_cast<const float*>(packed + (size_t)NT * KC * kTileBytes);
   const int Kp = KC * kTileK;
   const int nthreads = 64 * W;  // the workgroup size, without a read of the hidden launch arguments
@@ -395,10 +415,13 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
   // A producer that ran split over K (gemv_kparts_kernel) leaves its result as up to three partial rows:
   // they are requested here with everything else and added up, ((r0 + r1) + r2), before the row is used.
   // Grouped kernels at M = 1 only (a consumer with parts is launched through the group table).
-  constexpr bool kParts = kGrouped && M == 1;
-  const int in_parts = kParts ? ga.in_parts : 1;
+  // The number of parts is a template argument: as a run-time value its branches around the loads and the sums cost
+  // every grouped launch 0.14 us, with or without parts.
+  static_assert(kInParts == 1 || (kGrouped && M == 1), "partial input rows: grouped kernels at M = 1");
+  constexpr bool kParts = kInParts > 1;
+  constexpr int in_parts = kInParts;
   float pv[2][kParts ? kFusedR : 1][8];
-  if (kParts && in_parts > 1) {
+  if constexpr (kParts) {
     const float* base = kNorm ? pro_delta : x;
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
@@ -420,7 +443,7 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
   u32x2 sc[kSets][kCPW];
 #pragma unroll
   for (int st = 0; st < kSets; ++st) {
-    const uint8_t* tiles = (st == 0 ? packed : ga.packed[1]) + (size_t)nt * KC * kTileBytes;
+    const uint8_t* tiles = (st == 0 ? packed : packed1) + (size_t)nt * KC * kTileBytes;
 #pragma unroll
     for (int i = 0; i < kCPW; ++i) {
       const int kc = wave + i * W < KC ? wave + i * W : KC - 1;  // masked where used
@@ -438,13 +461,13 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
     bs[st] = 0.0f;
     const int n = kTileRows * nt + j;
     if (threadIdx.x < kOutputs && n < N) {
-      const float* rsp = st == 0 ? rsum : reinterpret_cast<const float*>(ga.packed[1] + (size_t)NT * KC * kTileBytes);
+      const float* rsp = st == 0 ? rsum : reinterpret_cast<const float*>(packed1 + (size_t)NT * KC * kTileBytes);
       rs[st] = load_global<float>(rsp + n);
       bs[st] = load_global<float>(rsp + NT * kTileRows + n);
     }
   }
 
-  if (kParts && in_parts > 1) {
+  if constexpr (kParts) {
 #pragma unroll
     for (int r = 0; r < kFusedR; ++r) {
 #pragma unroll
@@ -592,7 +615,7 @@ __global__ __launch_bounds__(M == 1 ? 1024 : 512) void gemv_fused_kernel(
         float s = 0.0f;
 #pragma unroll 4
         for (int w = 0; w < W; ++w) s += s_red[(w * kSets + st) * kOutputs + o];
-        const float* rsp = st == 0 ? rsum : reinterpret_cast<const float*>(ga.packed[1] + (size_t)NT * KC * kTileBytes);
+        const float* rsp = st == 0 ? rsum : reinterpret_cast<const float*>(packed1 + (size_t)NT * KC * kTileBytes);
         const float rsn = prefetched ? rs[st] : load_global<float>(rsp + n);
         const float bsn = prefetched ? bs[st] : load_global<float>(rsp + NT * kTileRows + n);
         float v = __fmaf_rn((float)off, rsn, s * 0.0625f);
@@ -1208,19 +1231,29 @@ static hipError_t launch_fused_m(const GroupArgs& ga, const float* x, int ldx, i
   const size_t lds = (size_t)M * Kp + (size_t)W * sets * M * 16 * sizeof(float) +
                      (size_t)W * M * 3 * sizeof(float);
   const dim3 grid(kPair ? ga.first[1] : ga.first[ga.count]), block(64 * W);
-  static LdsLimitOnce raised1, raisedg;
-  if ((ga.count == 1 && ga.in_parts <= 1) || kPair) {
-    auto kern = gemv_fused_kernel<M, R, false, CPW, kNorm, kPair>;
-    if (hipError_t e = raise_lds_limit(kern, lds, &raised1); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, grid, block, lds, s, x, ldx, K, KC, W, ga.packed[0], ga.N[0], pro.delta, pro.norm_w,
-                       pro.eps, ga.y[0], pro.sum_out, ga);
-  } else {
-    auto kern = gemv_fused_kernel<M, R, true, CPW, kNorm, false>;
-    if (hipError_t e = raise_lds_limit(kern, lds, &raisedg); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, grid, block, lds, s, x, ldx, K, KC, W, ga.packed[0], ga.N[0], pro.delta, pro.norm_w,
-                       pro.eps, ga.y[0], pro.sum_out, ga);
+  // what the first loads need travels in the preloaded arguments (see the kernel)
+  if (K > 0xFFFF || W > 31 || ga.in_parts > kMaxInParts || ga.first[ga.count] > 0xFFFF) return hipErrorInvalidValue;
+  const unsigned kw = (unsigned)K | (unsigned)W << 16 | (unsigned)ga.count << 24;
+  unsigned long long firsts = 0;
+  for (int i = 1; i <= kMaxGroup; ++i) {
+    firsts |= (unsigned long long)(unsigned)ga.first[i <= ga.count ? i : ga.count] << (16 * (i - 1));
   }
-  return hipGetLastError();
+  auto launch = [&](auto kern, LdsLimitOnce* once) -> hipError_t {
+    if (hipError_t e = raise_lds_limit(kern, lds, once); e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, grid, block, lds, s, x, ldx, kw, ga.packed[0], firsts, pro.delta, pro.norm_w,
+                       ga.packed[1], ga.packed[2], pro.eps, pro.sum_out, ga);
+    return hipGetLastError();
+  };
+  static LdsLimitOnce raised1, raisedg, raisedp2, raisedp3;
+  if ((ga.count == 1 && ga.in_parts <= 1) || kPair) {
+    return launch(gemv_fused_kernel<M, R, false, CPW, kNorm, kPair>, &raised1);
+  }
+  if constexpr (M == 1) {
+    if (ga.in_parts == 2) return launch(gemv_fused_kernel<M, R, true, CPW, kNorm, false, 2>, &raisedp2);
+    if (ga.in_parts == 3) return launch(gemv_fused_kernel<M, R, true, CPW, kNorm, false, 3>, &raisedp3);
+  }
+  if (ga.in_parts > 1) return hipErrorInvalidValue;
+  return launch(gemv_fused_kernel<M, R, true, CPW, kNorm, false>, &raisedg);
 }
 
 // Launch shape of gemv_batched_kernel: `waves` wavefronts per workgroup, Wt of them per tile row (a divisor of
