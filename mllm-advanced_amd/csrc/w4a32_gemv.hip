@@ -781,11 +781,23 @@ __device__ __forceinline__ void quantise_row_tasks(const float (&xv)[kR][8], int
 
 template <int M, int kCPW, int kR, int kWaves>
 __global__ __launch_bounds__(64 * kWaves) void gemv_batched_kernel(
-    const float* __restrict__ x, int ldx, const int8_t* __restrict__ aq, const float* __restrict__ recip,
-    const int32_t* __restrict__ negzp, int K, int KC, int Wt, const GroupArgs ga) {
+    const void* __restrict__ src, int ldx, unsigned kw, const uint8_t* packed0, unsigned long long firsts,
+    const uint8_t* packed1, const uint8_t* packed2, const float* __restrict__ recip,
+    const int32_t* __restrict__ negzp,  // 16 dwords: preloaded
+    const GroupArgs ga) {
+  // As in gemv_fused_kernel, what the first loads need comes in the preloaded arguments:
+  //   src    = the f32 rows (kR > 0) or the quantised rows (kR = 0, with recip and negzp)
+  //   kw     = K | wavefronts per tile row << 16 | Linears << 24
+  //   firsts = first[1] | first[2] << 16 | first[3] << 32 | first[4] << 48 (tile rows, see GroupArgs)
   extern __shared__ __align__(16) uint8_t smem[];
   constexpr bool kPreq = kR == 0;
   constexpr int kTasks = kPreq ? 1 : kR;
+  const float* x = static_cast<const float*>(src);
+  const int8_t* aq = static_cast<const int8_t*>(src);
+  const int K = (int)(kw & 0xFFFFu), Wt = (int)((kw >> 16) & 31u), count = (int)(kw >> 24);
+  const int KC = (K + kTileK - 1) / kTileK;
+  const int first_of[kMaxGroup + 1] = {0, (int)(firsts & 0xFFFFu), (int)((firsts >> 16) & 0xFFFFu),
+                                       (int)((firsts >> 32) & 0xFFFFu), (int)(firsts >> 48)};
   const int Kp = KC * kTileK;
   const int grp_per_row = Kp >> 3;
   const int nseg = (grp_per_row + 63) >> 6;       // 64-group segments per row (at most 8 when quantising here)
@@ -798,7 +810,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_batched_kernel(
   const int g = lane >> 4, j = lane & 15;
   const int T = kWaves / Wt;                      // tile rows per workgroup
   const int tg = wave / Wt, wl = wave - tg * Wt;  // this wavefront's tile row and its place in it
-  const int total = ga.first[ga.count];
+  const int total = first_of[kMaxGroup];  // entries past the last Linear repeat the total
 
   // the rows first (a few KB, normally in L2), then the weights: loads return in issue order
   float xv[kTasks][8];
@@ -826,14 +838,19 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_batched_kernel(
   }
   // which Linear this wavefront's tile row belongs to
   const int gt = (int)blockIdx.x * T + tg;
-  const uint8_t* packed = ga.packed[0];
+  const uint8_t* packed = packed0;
   int nt_first = 0;
-#pragma unroll
-  for (int i = 1; i < kMaxGroup; ++i) {
-    if (i < ga.count && gt >= ga.first[i]) {
-      packed = ga.packed[i];
-      nt_first = ga.first[i];
-    }
+  if (count > 1 && gt >= first_of[1]) {
+    packed = packed1;
+    nt_first = first_of[1];
+  }
+  if (count > 2 && gt >= first_of[2]) {
+    packed = packed2;
+    nt_first = first_of[2];
+  }
+  if (count > 3 && gt >= first_of[3]) {
+    packed = ga.packed[3];
+    nt_first = first_of[3];
   }
   const int nt = gt < total ? gt - nt_first : 0;   // a wavefront past the last tile row repeats one (not stored)
   const uint8_t* tiles = packed + (size_t)nt * KC * kTileBytes;
@@ -855,23 +872,36 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_batched_kernel(
     const int o = threadIdx.x;
     const int to = o / (M * 16), ogt = (int)blockIdx.x * T + to;
     if (o < outputs && ogt < total) {
-      const uint8_t* opk = ga.packed[0];
-      int ofirst = 0;
+      const uint8_t* opk = packed0;
+      int ofirst = 0, oNT = first_of[1];
       oN = ga.N[0];
       oy = ga.y[0];
-#pragma unroll
-      for (int i = 1; i < kMaxGroup; ++i) {
-        if (i < ga.count && ogt >= ga.first[i]) {
-          opk = ga.packed[i];
-          oN = ga.N[i];
-          oy = ga.y[i];
-          ofirst = ga.first[i];
-        }
+      if (count > 1 && ogt >= first_of[1]) {
+        opk = packed1;
+        ofirst = first_of[1];
+        oNT = first_of[2] - first_of[1];
+        oN = ga.N[1];
+        oy = ga.y[1];
       }
-      const int oNT = (oN + kTileRows - 1) / kTileRows;
+      if (count > 2 && ogt >= first_of[2]) {
+        opk = packed2;
+        ofirst = first_of[2];
+        oNT = first_of[3] - first_of[2];
+        oN = ga.N[2];
+        oy = ga.y[2];
+      }
+      if (count > 3 && ogt >= first_of[3]) {
+        opk = ga.packed[3];
+        ofirst = first_of[3];
+        oNT = first_of[4] - first_of[3];
+        oN = ga.N[3];
+        oy = ga.y[3];
+      }
       on = kTileRows * (ogt - ofirst) + (o & 15);
-      owns = on < oN;
-      if (owns) {
+      owns = true;
+      // the weights' planes are requested for every output column of the padded tile row; whether the column
+      // exists (on < oN, with oN from the argument segment) only matters for the store
+      {
         const float* rsp = reinterpret_cast<const float*>(opk + (size_t)oNT * KC * kTileBytes);
         rs = load_global<float>(rsp + on);
         bs = load_global<float>(rsp + oNT * kTileRows + on);
@@ -909,7 +939,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_batched_kernel(
   __syncthreads();
 
   //   y = (sum/16 + off * rsum[n]) * lhs_scale + bias[n], clamped to the finite f32 range
-  if (owns) {
+  if (owns && on < oN) {
     const int o = threadIdx.x;
     const int to = o / (M * 16), rem = o - to * (M * 16), m = rem >> 4;
     // all reads are issued before the first add (a loop over Wt would wait for each LDS read in turn); wavefronts
@@ -1309,9 +1339,16 @@ static hipError_t launch_batched_k(const GroupArgs& ga, const float* x, int ldx,
   auto kern = gemv_batched_kernel<M, kCPW, kR, kWaves>;
   static LdsLimitOnce raised;
   if (hipError_t e = raise_lds_limit(kern, lds, &raised); e != hipSuccess) return e;
-  hipLaunchKernelGGL(kern, grid, block, lds, s, x, ldx, ws ? reinterpret_cast<const int8_t*>(ws + w.aq_off) : nullptr,
+  if (K > 0xFFFF || p.Wt > 31 || ga.first[ga.count] > 0xFFFF) return hipErrorInvalidValue;
+  const unsigned kw = (unsigned)K | (unsigned)p.Wt << 16 | (unsigned)ga.count << 24;
+  unsigned long long firsts = 0;
+  for (int i = 1; i <= kMaxGroup; ++i) {
+    firsts |= (unsigned long long)(unsigned)ga.first[i <= ga.count ? i : ga.count] << (16 * (i - 1));
+  }
+  const void* src = kR ? static_cast<const void*>(x) : static_cast<const void*>(ws + w.aq_off);
+  hipLaunchKernelGGL(kern, grid, block, lds, s, src, ldx, kw, ga.packed[0], firsts, ga.packed[1], ga.packed[2],
                      ws ? reinterpret_cast<const float*>(ws + w.scale_off) : nullptr,
-                     ws ? reinterpret_cast<const int32_t*>(ws + w.off_off) : nullptr, K, KC, p.Wt, ga);
+                     ws ? reinterpret_cast<const int32_t*>(ws + w.off_off) : nullptr, ga);
   return hipGetLastError();
 }
 
