@@ -31,7 +31,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the decode pass, measured with hardware counters (not re-measured by a
 # bench run: the counters need the profiler); algorithmic bytes per launch are 7,732,011.
-PASS_TRAFFIC_BYTES_PER_LAUNCH = 8_009_036
+PASS_TRAFFIC_BYTES_PER_LAUNCH = 8003128
 LAYERS = 28
 # name, K, N, bias, count per layer
 LAYER_LINEARS = [
@@ -265,7 +265,7 @@ def main():
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": PASS_TRAFFIC_BYTES_PER_LAUNCH,
                 "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over this pass's 113 launches "
-                                  "(3896.1 / 29.1 KiB per dispatch), scaled x2.00 / x1.00 by the same counters' "
+                                  "(3893.2 / 29.1 KiB per dispatch), scaled x2.00 / x1.00 by the same counters' "
                                   "reading for a 256 MiB copy; profiles/traffic_fetch_write_decode_prefill.md",
                 "kernel": "gemv_fused_kernel<1,1> for K=1536 (q,k,v grouped; o; gate,up as a pair), "
                           "gemv_kparts_kernel<2> for down_proj (K=8960 in two k-parts; gemv_fused_kernel<1,2> "
