@@ -188,11 +188,22 @@ struct GemmGroup {
 
 template <int WAVES_M, int WAVES_N, int WM, int WN, int DEPTH, int OCC, int MODE, int BE, int WK>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_kernel(
-    float* __restrict__ y_arg, const _Float16* __restrict__ ah, const float* __restrict__ recip,
-    const uint8_t* __restrict__ packed_arg, const uint8_t* __restrict__ hscale_arg,
-    const float* __restrict__ rowmul_arg, const float* __restrict__ bias_arg, int M, int N_arg, int K,
-    int NT_arg, int KC, int MB, int NB, int n_major, int ksplit, float* __restrict__ part,
-    const GemmGroup grp) {
+    const _Float16* __restrict__ ah, const uint8_t* __restrict__ packed0, const uint8_t* __restrict__ packed1,
+    const uint8_t* __restrict__ packed2, int M, int K, int N0, int N1, int N2, unsigned nbs, unsigned nbf,
+    unsigned flags,  // 16 dwords: preloaded by the dispatcher
+    float* __restrict__ y_arg, const float* __restrict__ recip, float* __restrict__ part, const GemmGroup grp) {
+  // Everything a workgroup needs to find its tile and request its first operands arrives in the preloaded
+  // registers (a read of the argument segment takes about half a microsecond, in front of every workgroup's
+  // first load): the activations, the weights of up to three Linears (plain and split-K: packed0; pair: gate,
+  // up) and their widths, from which the tile geometry and the scale / row-factor / bias planes follow, and
+  //   nbs   = row blocks | column blocks << 16
+  //   nbf   = grouped: first column block of Linear 1 | of Linear 2 << 16
+  //   flags = n_major | k-parts << 8 | Linears << 16 | grouped: first column block of Linear 3 << 20
+  // Outputs, the activations' row factors, the parts' scratch and a fourth Linear come from the segment and are
+  // used in the epilogue.
+  const int MB = (int)(nbs & 0xFFFFu), NB = (int)(nbs >> 16);
+  const int n_major = (int)(flags & 1u), ksplit = (int)((flags >> 8) & 0xFFu);
+  const int KC = (K + kTileK - 1) / kTileK;
   constexpr bool GROUPED = MODE == kModeGrouped, SPLITK = MODE == kModeSplitK, PAIR = MODE == kModePair;
   static_assert(!PAIR || (WAVES_N == 1 && WN % 2 == 0 && WK == 1), "a wavefront must own both halves");
   constexpr int D = DEPTH;
@@ -252,30 +263,34 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
   const int mb = n_major ? tile % MB : tile / NB;
   int nb = n_major ? tile / MB : tile % NB;
   float* y = y_arg;
-  const uint8_t* packed = packed_arg;
-  const uint8_t* hscale = hscale_arg;
-  const float* rowmul = rowmul_arg;
-  const float* bias = bias_arg;
-  int N = N_arg, NT = NT_arg;
+  const uint8_t* packed = packed0;
+  int N = N0;
   if constexpr (GROUPED) {
-    int gi = 0;
-#pragma unroll
-    for (int i = 1; i < kMaxGemmGroup; ++i) gi = nb >= grp.nb_first[i] ? i : gi;
-    nb -= grp.nb_first[gi];
-    N = grp.N[gi];
-    const WeightGeom wgm = weight_geom(N, K);
-    NT = wgm.NT;
-    y = grp.y[gi];
-    packed = grp.packed[gi];
-    hscale = packed + wgm.hscale_off;
-    rowmul = reinterpret_cast<const float*>(packed + wgm.rowmul_off);
-    bias = reinterpret_cast<const float*>(packed + wgm.bias_off);
-  }
-  if constexpr (PAIR) {
-    N = grp.N[0];
-    NT = weight_geom(N, K).NT;
+    const int count = (int)((flags >> 16) & 0xFu);
+    const int f1 = (int)(nbf & 0xFFFFu), f2 = (int)(nbf >> 16), f3 = (int)(flags >> 20);
     y = grp.y[0];
+    if (count > 1 && nb >= f1) {
+      packed = packed1;
+      N = N1;
+      y = grp.y[1];
+    }
+    if (count > 2 && nb >= f2) {
+      packed = packed2;
+      N = N2;
+      y = grp.y[2];
+    }
+    if (count > 3 && nb >= f3) {
+      packed = grp.packed[3];
+      N = grp.N[3];
+      y = grp.y[3];
+    }
+    nb -= count > 3 && nb >= f3 ? f3 : count > 2 && nb >= f2 ? f2 : count > 1 && nb >= f1 ? f1 : 0;
   }
+  const WeightGeom wgm = weight_geom(N, K);
+  const int NT = wgm.NT;
+  const uint8_t* hscale = packed + wgm.hscale_off;
+  const float* rowmul = reinterpret_cast<const float*>(packed + wgm.rowmul_off);
+  const float* bias = reinterpret_cast<const float*>(packed + wgm.bias_off);
   const int m0 = mb * BM + 32 * WM * wm;
   // first 16-row weight tile row of this workgroup's columns (PAIR: in both Linears, half the units each)
   const int nt0 = nb * (PAIR ? WNT / 2 : WNT);
@@ -316,8 +331,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
     if constexpr (PAIR) {
       const int side = ntl >= WNT / 2 ? 1 : 0;  // wavefront-uniform
       ntl -= side * (WNT / 2);
-      pk = grp.packed[side];
-      hs = pk + weight_geom(N, K).hscale_off;
+      pk = side ? packed1 : packed0;
+      hs = pk + wgm.hscale_off;
     }
     int nt = nt0 + ntl;
     nt = nt < NT ? nt : NT - 1;  // tile rows past the matrix: their columns are never stored
@@ -674,8 +689,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WK, OCC) void gemm_f16_ker
     const float* rmp = rowmul;
     const float* bsp = bias;
     if constexpr (PAIR) {
-      const WeightGeom wgm = weight_geom(N, K);
-      const uint8_t* pk = grp.packed[b / WNH];
+      const uint8_t* pk = b / WNH ? packed1 : packed0;
       rmp = reinterpret_cast<const float*>(pk + wgm.rowmul_off);
       bsp = reinterpret_cast<const float*>(pk + wgm.bias_off);
     }
@@ -798,10 +812,15 @@ static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed,
     }
     const int NB = nb;
     const int n_major = (double)M * 2.0 <= (double)n_total * 0.5625 ? 1 : 0;
+    const int f3 = count > 3 ? g.nb_first[3] : 0;  // the boundary in front of a fourth Linear has 12 bits
+    if (MB > 0xFFFF || NB > 0xFFFF || f3 > 0xFFF) return hipErrorInvalidValue;
+    const unsigned nbs = (unsigned)MB | (unsigned)NB << 16;
+    const unsigned nbf = (unsigned)g.nb_first[1] | (unsigned)g.nb_first[2] << 16;
+    const unsigned flags = (unsigned)n_major | 1u << 8 | (unsigned)count << 16 | (unsigned)f3 << 20;
     hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModeGrouped, BE, WK>),
-                       dim3(((MB * NB + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N * WK), 0, s, nullptr, ah,
-                       recip, nullptr, nullptr, nullptr, nullptr, M, 0, K, 0,
-                       weight_geom(group_N[0], K).KC, MB, NB, n_major, 1, nullptr, g);
+                       dim3(((MB * NB + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N * WK), 0, s, ah, g.packed[0],
+                       g.packed[1], g.packed[2], M, K, group_N[0], count > 1 ? group_N[1] : 0,
+                       count > 2 ? group_N[2] : 0, nbs, nbf, flags, nullptr, recip, nullptr, g);
     return hipGetLastError();
   }
   const WeightGeom g = weight_geom(N, K);
@@ -811,11 +830,13 @@ static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed,
   const int n_major = (double)M * 2.0 <= (double)N * 0.5625 ? 1 : 0;
   const float* rowmul = reinterpret_cast<const float*>(packed + g.rowmul_off);
   const float* bias = reinterpret_cast<const float*>(packed + g.bias_off);
+  if (MB > 0xFFFF || NB > 0xFFFF || ksplit > 0xFF) return hipErrorInvalidValue;
+  const unsigned nbs = (unsigned)MB | (unsigned)NB << 16;
+  const unsigned flags = (unsigned)n_major | (unsigned)(ksplit > 1 ? ksplit : 1) << 8 | 1u << 16;
   if (ksplit > 1) {
     hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModeSplitK, BE, WK>),
-                       dim3(((MB * NB * ksplit + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N * WK), 0, s, y, ah,
-                       recip, packed, packed + g.hscale_off, rowmul, bias, M, N, K, g.NT, g.KC, MB, NB,
-                       n_major, ksplit, part, GemmGroup{});
+                       dim3(((MB * NB * ksplit + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N * WK), 0, s, ah,
+                       packed, nullptr, nullptr, M, K, N, 0, 0, nbs, 0u, flags, y, recip, part, GemmGroup{});
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     if (!y) return hipSuccess;  // the caller's next kernel adds the (scaled) parts up
     const size_t total = (size_t)M * N;
@@ -829,9 +850,8 @@ static hipError_t launch_f16(float* y, const uint8_t* ws, const uint8_t* packed,
     return hipGetLastError();
   }
   hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, WAVES_N, WM, WN, DEPTH, OCC, kModePlain, BE, WK>),
-                     dim3(((MB * NB + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N * WK), 0, s, y, ah, recip,
-                     packed, packed + g.hscale_off, rowmul, bias, M, N, K, g.NT, g.KC, MB, NB, n_major,
-                     1, nullptr, GemmGroup{});
+                     dim3(((MB * NB + 7) / 8) * 8), dim3(64 * WAVES_M * WAVES_N * WK), 0, s, ah, packed, nullptr,
+                     nullptr, M, K, N, 0, 0, nbs, 0u, flags, y, recip, nullptr, GemmGroup{});
   return hipGetLastError();
 }
 
@@ -850,11 +870,13 @@ static hipError_t launch_f16_pair(float* act, const uint8_t* ws, const uint8_t* 
   g.packed[1] = up;
   g.N[0] = g.N[1] = N;
   const int n_major = (double)M * 2.0 <= (double)N * 2.0 * 0.5625 ? 1 : 0;
+  if (MB > 0xFFFF || NB > 0xFFFF) return hipErrorInvalidValue;
+  const unsigned nbs = (unsigned)MB | (unsigned)NB << 16;
+  const unsigned flags = (unsigned)n_major | 1u << 8 | 2u << 16;
   hipLaunchKernelGGL((gemm_f16_kernel<WAVES_M, 1, WM, WN, DEPTH, OCC, kModePair, 1, 1>),
-                     dim3(((MB * NB + 7) / 8) * 8), dim3(64 * WAVES_M), 0, s, nullptr,
-                     reinterpret_cast<const _Float16*>(ws + w.ah_off),
-                     reinterpret_cast<const float*>(ws + w.scale_off), nullptr, nullptr, nullptr, nullptr, M, 0,
-                     K, 0, wg.KC, MB, NB, n_major, 1, nullptr, g);
+                     dim3(((MB * NB + 7) / 8) * 8), dim3(64 * WAVES_M), 0, s,
+                     reinterpret_cast<const _Float16*>(ws + w.ah_off), gate, up, nullptr, M, K, N, N, 0, nbs, 0u,
+                     flags, act, reinterpret_cast<const float*>(ws + w.scale_off), nullptr, g);
   return hipGetLastError();
 }
 

@@ -89,9 +89,11 @@ constexpr int kSrcPlain = 0, kSrcNorm = 1, kSrcSiluMul = 2;
 template <int SRC, int R>
 __global__ __launch_bounds__(kLhsThreads) void quant_rows_kernel(
     const float* __restrict__ a, const float* __restrict__ b, const float* __restrict__ norm_w,
-    float eps, float* h_out, int K, int lda, float* __restrict__ recip_out,
-    int32_t* __restrict__ negzp_out, int8_t* __restrict__ aq, _Float16* __restrict__ ah, int nparts,
-    size_t part_stride, const float* __restrict__ part_bias) {
+    const float* __restrict__ part_bias, float eps, int K, int lda, int nparts, size_t part_stride,
+    float* h_out,  // 16 dwords: preloaded by the dispatcher, everything the loads need; a read of the argument
+                   // segment takes about half a microsecond
+    float* __restrict__ recip_out, int32_t* __restrict__ negzp_out, int8_t* __restrict__ aq,
+    _Float16* __restrict__ ah) {
   const int m = blockIdx.x;
   const int t = threadIdx.x;
   const size_t row = (size_t)m * lda;
@@ -261,8 +263,8 @@ static hipError_t launch_quant_rows(const float* a, const float* b, const float*
   _Float16* ah = (M > kGemvMaxM) ? reinterpret_cast<_Float16*>(ws + g.ah_off) : nullptr;
   const int groups = (K + 8 * kLhsThreads - 1) / (8 * kLhsThreads);
 #define W4_LAUNCH_ROWS(R)                                                                          \
-  hipLaunchKernelGGL((quant_rows_kernel<SRC, R>), dim3(M), dim3(kLhsThreads), 0, s, a, b, norm_w, eps, \
-                     h_out, K, lda, recip, negzp, aq, ah, nparts, (size_t)M * K, part_bias)
+  hipLaunchKernelGGL((quant_rows_kernel<SRC, R>), dim3(M), dim3(kLhsThreads), 0, s, a, b, norm_w,     \
+                     part_bias, eps, K, lda, nparts, (size_t)M * K, h_out, recip, negzp, aq, ah)
   if (groups <= 1) W4_LAUNCH_ROWS(1);
   else if (groups <= 2) W4_LAUNCH_ROWS(2);
   else if (groups <= 5) W4_LAUNCH_ROWS(5);
