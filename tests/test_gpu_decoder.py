@@ -423,6 +423,47 @@ def test_decoder_prefill_in_slices_of_decode_sized_rows(pkg, slices):
         assert int(dec.token) == do.greedy(got) and dec.position == len(prompt)
 
 
+@pytest.mark.parametrize("slices", [(300, 290), (256, 256, 70), (40, 330)])
+def test_decoder_prefill_in_long_slices_that_continue_a_cache(pkg, slices):
+    """Prompt slices of 256 rows and more take the matrix-pipe attention, whose operand split also rotates q and k
+    and appends to the caches: here at positions that continue earlier slices (inside a 32-key block too), against
+    the oracle on the whole prompt, and the cache rows against a run that takes the prompt in one slice."""
+    import decoder_oracle as do
+
+    rng = np.random.default_rng(23)
+    H, Hq, Hkv, I, V, L = 256, 2, 1, 384, 640, 2
+    n = sum(slices)
+    weights = tiny_model(rng, H, Hq, Hkv, I, V, L)
+    dec = to_device_model(pkg, weights, Hq, Hkv, max_seq=640, max_batch_tokens=max(slices), rope_theta=1e6)
+    one = to_device_model(pkg, weights, Hq, Hkv, max_seq=640, max_batch_tokens=n, rope_theta=1e6)
+    ref = do.Decoder(weights, Hq, Hkv, rope_theta=1e6, max_seq=640)
+    prompt = rng.integers(0, V, size=n)
+    want = ref.forward(prompt)
+    one.prefill(dev(prompt.astype(np.int64)))
+    pos = 0
+    for m in slices:
+        dec.prefill(dev(prompt[pos:pos + m].astype(np.int64)), pos0=pos)
+        pos += m
+    torch.cuda.synchronize()
+    got = dec.logits.cpu().numpy()
+    # 2e-2 throughout: after 600 tokens the logits come out either identical to the oracle's (1e-7) or between
+    # 1e-3 and 1e-2 off, with either attention kernel and however the prompt is sliced (582 tokens: 9e-3 through
+    # the matrix-pipe kernel, 1.3e-3 through the f32 one; 590 tokens: 3e-7 and 0): one int8 of a re-quantised row
+    # that flips on a last-bit difference moves a logit by a weight times a quantisation step. The operators
+    # themselves are held to 2e-5 and to bit-identity with the separate launches by the tests above; what this
+    # test looks for is a wrong or missing cache row, which is off by the size of the logits themselves.
+    assert max_abs_rel(got, want) < 2e-2
+    assert max_abs_rel(one.logits.cpu().numpy(), want) < 2e-2
+    assert int(dec.token) == do.greedy(got) and dec.position == n
+    # two more tokens continue from what the slices left in the caches
+    for _ in range(2):
+        fed = int(dec.token)
+        dec.step()
+        want = ref.forward([fed])
+        torch.cuda.synchronize()
+        assert max_abs_rel(dec.logits.cpu().numpy(), want) < 2e-2
+
+
 def test_decoder_ignores_what_its_state_memory_held(pkg):
     # The state is caller-owned memory that init does not clear: rows of the KV cache behind the position,
     # scratch areas and activations hold whatever was there. Bytes 0xFF (NaN as f32) against zeros: prefill
@@ -604,6 +645,12 @@ def test_prefill_layer_at_the_model_s_widths_every_operator_on_its_own_inputs(pk
     a_ref = np.stack([do.attention(q_rot.cpu().numpy().reshape(M, Hq, D)[r:r + 1], kc_h, vc_h, int(r))[0]
                       for r in arows])
     assert max_abs_rel(attn.cpu().numpy()[arows], a_ref) <= 2e-5
+    # the kernel a prefill of this many rows runs: products on bf16 terms, with the rotation and the cache append
+    # done by its operand split; same bar against the oracle, caches and rotated q bit-identical to the above
+    kc16, vc16, q16 = torch.zeros_like(kc), torch.zeros_like(vc), qkv[0].clone()
+    attn16 = pkg.op_rope_attention_prefill_bf16x3(q16, qkv[1], qkv[2], sin, cos, kc16, vc16, Hq, Hkv, D, 0)
+    assert torch.equal(q16, q_rot) and torch.equal(kc16, kc) and torch.equal(vc16, vc)
+    assert max_abs_rel(attn16.cpu().numpy()[arows], a_ref) <= 2e-5
 
     # [quantiser] [o]
     ws2 = pkg.quant_lhs(attn)
