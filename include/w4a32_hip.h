@@ -180,7 +180,8 @@ int w4a32_matmul_ws(float* d_y, const float* d_x, const void* d_packed, void* d_
  *     call overwrites the M rows it multiplies, and what the product kernels read beyond them (up to 31
  *     rows of padding) only feeds output rows that are never stored.
  *   - The first call on a device looks the array's address up (hipGetSymbolAddress); make that call outside
- *     stream capture. */
+ *     stream capture. A first call on a stream that is capturing returns W4A32_ENOTSUP and launches nothing
+ *     (the capture stays valid); after one call outside capture the same call captures and replays. */
 #define W4A32_STATIC_WS_BYTES (16u << 20)
 int w4a32_matmul_static_ws(float* d_y, const float* d_x, const void* d_packed, int M, int K, int N,
                            void* stream);

@@ -30,12 +30,19 @@ namespace {
 // Address of `scratch` on each device, looked up on the first call made with that device current.
 std::atomic<void*> g_static_ws[kMaxDevices];
 
-int static_ws_ptr(void** out) {
+int static_ws_ptr(void** out, hipStream_t stream) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return W4A32_ELAUNCH;
   if (dev < 0 || dev >= kMaxDevices) return W4A32_ENOTSUP;
   void* p = g_static_ws[dev].load(std::memory_order_acquire);
   if (!p) {
+    // The lookup is a runtime query, not stream work: it does not belong into a capture. A first call on a
+    // capturing stream is refused before anything is launched, so the capture stays valid and empty-handed.
+    if (stream) {
+      hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+      if (hipStreamIsCapturing(stream, &st) != hipSuccess) return W4A32_ELAUNCH;
+      if (st != hipStreamCaptureStatusNone) return W4A32_ENOTSUP;
+    }
     if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return W4A32_ELAUNCH;
     g_static_ws[dev].store(p, std::memory_order_release);  // racing first calls store the same address
   }
@@ -265,7 +272,7 @@ int w4a32_matmul_static_ws(float* d_y, const float* d_x, const void* d_packed, i
   if (int e = shape_ok(N, K)) return e;
   if (w4::ws_geom(M, K).total_bytes > (size_t)W4A32_STATIC_WS_BYTES) return W4A32_ETOOBIG;
   void* ws = nullptr;
-  if (int e = static_ws_ptr(&ws)) return e;
+  if (int e = static_ws_ptr(&ws, static_cast<hipStream_t>(stream))) return e;
   return w4a32_matmul(d_y, d_x, d_packed, ws, M, K, N, stream);
 }
 
